@@ -1,0 +1,103 @@
+"""Pins the oracle's table initialisers (reference: csrc/utils/initializer.cu:11-103).
+
+* Zero / Uniform: closed form of the minstd engine, computed here with python integers and exact
+  rationals (independent of the oracle's C++), and the reference's own initializer.cu compiled
+  against the image's thrust (oracle/_ref), when that library is present.
+* Normal / TruncatedNormal: the same reference build (its erfcinv is rocThrust's, not CUDA's, so
+  only a tolerance comparison is meaningful) + distribution moments + determinism.
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from oracle import oracle as orc
+
+M = 2**31 - 1
+A = 48271
+
+
+def _state(seed):
+    s = seed % M
+    return 1 if s == 0 else s
+
+
+def _round_f32(fr):
+    """Exact rational -> nearest float32 (ties to even) via numpy on an exactly representable double pair."""
+    # float(Fraction) is correctly rounded to double; a second rounding to f32 could double-round, so
+    # check the two neighbouring floats exactly instead.
+    c = np.float32(float(fr))
+    cands = [np.nextafter(c, np.float32(-np.inf)), c, np.nextafter(c, np.float32(np.inf))]
+    best = min(cands, key=lambda v: (abs(Fraction(float(v)) - fr), int(v.view(np.uint32)) & 1))
+    return best
+
+
+def _uniform_closed_form(n, a, b, seed):
+    x = _state(seed) * pow(A, n + 1, M) % M
+    r = np.float32(x - 1)                                  # exact conversion rounds to f32
+    r = np.float32(r) / (np.float32(1.0) + np.float32(M - 2))
+    width = np.float32(b) - np.float32(a)
+    return _round_f32(Fraction(float(r)) * Fraction(float(width)) + Fraction(float(np.float32(a))))
+
+
+@pytest.mark.parametrize("seed", [0, 1, 12345, M, M + 7])
+def test_uniform_closed_form(seed):
+    a, b = -0.01, 0.01
+    got = orc.init_values(4096, "Uniform", a, b, seed)
+    idx = list(range(64)) + [100, 1000, 4095]
+    for n in idx:
+        assert got[n] == _uniform_closed_form(n, a, b, seed), (n, seed)
+    assert got.min() >= a and got.max() < b
+
+
+def test_uniform_far_offsets_match_sequential():
+    # discard(n) for huge n equals n single steps: check the skip-ahead against a running product
+    seed, a, b = 3, 0.0, 1.0
+    n0 = 5_000_000
+    big = orc.init_values(n0 + 16, "Uniform", a, b, seed)[n0:]
+    for k in range(16):
+        assert big[k] == _uniform_closed_form(n0 + k, a, b, seed)
+
+
+def test_zero():
+    assert not orc.init_values(1000, "Zero", 1.0, 2.0, 5).any()
+
+
+def _ref(n, kind, a, b, seed):
+    l = orc.ref_lib()
+    if l is None:
+        pytest.skip("oracle/_ref not built (reference tree absent at build time)")
+    out = np.empty(n, dtype=np.float32)
+    l.ref_initialize_host(out.ctypes.data, n, orc.INIT[kind], a, b, seed)
+    return out
+
+
+@pytest.mark.parametrize("seed", [0, 7])
+def test_uniform_vs_reference_build(seed):
+    a, b = -0.01, 0.01
+    ref = _ref(20000, "Uniform", a, b, seed)
+    got = orc.init_values(20000, "Uniform", a, b, seed)
+    # the host build of the reference has no fused multiply-add: allow one ulp of the range
+    assert np.max(np.abs(ref - got)) <= 2e-9
+    assert _ref(1000, "Zero", a, b, seed).tolist() == [0.0] * 1000
+
+
+@pytest.mark.parametrize("kind", ["Normal", "TruncatedNormal"])
+def test_normal_vs_reference_build(kind):
+    ref = _ref(20000, kind, 0.5, 2.0, 11)
+    got = orc.init_values(20000, kind, 0.5, 2.0, 11)
+    # same uniform draws, same formula; erfcinv implementations differ in the last bits
+    assert np.max(np.abs(ref - got)) <= 2e-5 * 2.0
+
+
+def test_normal_moments_and_determinism():
+    x = orc.init_values(400000, "Normal", 1.0, 3.0, 2)
+    assert abs(x.mean() - 1.0) < 0.03 and abs(x.std() - 3.0) < 0.03
+    y = orc.init_values(1000, "Normal", 1.0, 3.0, 2)
+    assert np.array_equal(x[:1000], y)
+    t = orc.init_values(200000, "TruncatedNormal", 0.0, 1.0, 9)
+    assert t.min() >= -2.0 and t.max() <= 2.0 and abs(t.mean()) < 0.02
+    # a truncated draw equals the plain draw wherever the plain draw is already inside 2 sigma
+    n = orc.init_values(200000, "Normal", 0.0, 1.0, 9)
+    inside = np.abs(n) <= 2.0
+    assert np.array_equal(t[inside], n[inside])
