@@ -1,0 +1,141 @@
+"""ctypes binding of the C ABI (include/hetuctr_hip.h).  No fallback: if libhetuctr_hip.so is missing or does
+not load, importing a table fails loudly."""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libhetuctr_hip.so")
+INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
+SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_push_pull", "hctr_group_preprocess",
+           "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch",
+           "hctr_stream", "hctr_last_times", "hctr_version"]
+
+# items of hctr_debug_fetch (HCTR_F_*)
+UNIQUE, SORTED_ARG, RUN_START, IDX_MAP, ROOT, OFFSET, SEND_CNT, RECV_CNT = range(8)
+NEED_UPDATE, UPDATE_PREFIX, PUSH_CNT, PUSHRECV_CNT, OUTDATED, GOT, VERSION, UPDATES = range(8, 16)
+EMBEDDING, PENDING, STORE_IDS, STATS, SIZES, KEYS = range(16, 22)
+FLOAT_ITEMS = (EMBEDDING, PENDING)
+
+
+class Config(C.Structure):
+    _fields_ = [("rank", C.c_int), ("nrank", C.c_int), ("device_id", C.c_int), ("ip", C.c_char_p), ("port", C.c_int),
+                ("length", C.c_size_t), ("width", C.c_size_t), ("pull_bound", C.c_longlong),
+                ("push_bound", C.c_longlong), ("init_type", C.c_int), ("init_a", C.c_float), ("init_b", C.c_float),
+                ("learning_rate", C.c_float), ("verbose", C.c_int)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libhetuctr_hip.so is not built: run `python -m hetuctr_amd.build`")
+        l = C.CDLL(LIB_PATH)
+        l.hctr_create.argtypes = [C.POINTER(Config), C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]
+        l.hctr_destroy.argtypes = [C.c_void_p]
+        l.hctr_preprocess.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        l.hctr_push_pull.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        l.hctr_group_preprocess.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        l.hctr_group_push_pull.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        l.hctr_seed.argtypes = [C.c_ulong]
+        l.hctr_seed.restype = None
+        l.hctr_repr.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
+        l.hctr_debug.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
+        l.hctr_last_error.restype = C.c_char_p
+        l.hctr_version.restype = C.c_char_p
+        l.hctr_debug_fetch.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t)]
+        l.hctr_stream.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        l.hctr_last_times.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+        _lib = l
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise RuntimeError(lib().hctr_last_error().decode())
+
+
+def seed(n):
+    lib().hctr_seed(int(n))
+
+
+class Table:
+    """One shard.  Arguments as hetuCTR.HetuTable (csrc/pybind/pybind.cu:63-69); `init` is (kind, a, b)."""
+
+    def __init__(self, rank, nrank, device_id, ip, port, length, width, pull_bound, push_bound, root_arr,
+                 storage_arr, init, learning_rate, verbose=0):
+        root = np.ascontiguousarray(root_arr).astype(np.uint8, copy=False)
+        storage = np.ascontiguousarray(storage_arr, dtype=np.int64)
+        if root.shape[0] != length:
+            raise RuntimeError("root_arr must hold `length` entries")
+        kind = INIT[init[0]] if isinstance(init[0], str) else int(init[0])
+        cfg = Config(rank, nrank, device_id, (ip or "").encode(), port, length, width, pull_bound, push_bound, kind,
+                     float(init[1]), float(init[2]), float(learning_rate), verbose)
+        h = C.c_void_p()
+        _check(lib().hctr_create(C.byref(cfg), root.ctypes.data, storage.ctypes.data, storage.shape[0], C.byref(h)))
+        self._h = h
+        self.rank, self.nrank, self.width, self.length = rank, nrank, width, length
+
+    def preprocess(self, ptr, n):
+        _check(lib().hctr_preprocess(self._h, C.c_void_p(int(ptr)), n))
+
+    def push_pull(self, grad_ptr, dst_ptr):
+        _check(lib().hctr_push_pull(self._h, C.c_void_p(int(grad_ptr) or None), C.c_void_p(int(dst_ptr) or None)))
+
+    def fetch(self, which):
+        n = C.c_size_t()
+        _check(lib().hctr_debug_fetch(self._h, which, None, 0, C.byref(n)))
+        out = np.empty(n.value, dtype=np.float32 if which in FLOAT_ITEMS else np.int64)
+        _check(lib().hctr_debug_fetch(self._h, which, out.ctypes.data, n.value, C.byref(n)))
+        return out
+
+    def stream(self):
+        s = C.c_void_p()
+        _check(lib().hctr_stream(self._h, C.byref(s)))
+        return s.value
+
+    def last_times(self):
+        a, b = C.c_float(), C.c_float()
+        _check(lib().hctr_last_times(self._h, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def __repr__(self):
+        buf = C.create_string_buffer(256)
+        lib().hctr_repr(self._h, buf, 256)
+        return buf.value.decode()
+
+    def debug(self):
+        buf = C.create_string_buffer(512)
+        lib().hctr_debug(self._h, buf, 512)
+        return buf.value.decode()
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().hctr_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _ptrs(vals):
+    return (C.c_void_p * len(vals))(*[C.c_void_p(int(v) or None) for v in vals])
+
+
+def group_preprocess(tables, key_ptrs, ns):
+    """Lock-step preprocess of every shard of a loopback group from one caller."""
+    hs = (C.c_void_p * len(tables))(*[t._h for t in tables])
+    sizes = (C.c_size_t * len(tables))(*ns)
+    _check(lib().hctr_group_preprocess(hs, len(tables), _ptrs(key_ptrs), sizes))
+
+
+def group_push_pull(tables, grad_ptrs, dst_ptrs):
+    hs = (C.c_void_p * len(tables))(*[t._h for t in tables])
+    _check(lib().hctr_group_push_pull(hs, len(tables), _ptrs(grad_ptrs), _ptrs(dst_ptrs)))

@@ -1,0 +1,161 @@
+// extern "C" surface declared in include/hetuctr_hip.h.  Exceptions never cross it: every entry point returns
+// 0 or stores a message for hctr_last_error() and returns 1.
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+
+#include "table.h"
+
+using namespace hctr;
+
+struct hctr_table {
+  Shard *shard;
+};
+
+namespace {
+thread_local std::string g_error;
+std::atomic<unsigned long> g_seed{0}; // hetuCTR::__seed, csrc/core/hetu_gpu_table.cu:7
+
+template <typename F> int guarded(F &&f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception &e) {
+    g_error = e.what();
+  } catch (...) {
+    g_error = "hetuCTR: unknown error";
+  }
+  return 1;
+}
+
+int write_string(const std::string &s, char *buf, size_t cap) {
+  if (buf && cap) {
+    const size_t n = std::min(cap - 1, s.size());
+    memcpy(buf, s.data(), n);
+    buf[n] = 0;
+  }
+  return (int)s.size();
+}
+} // namespace
+
+extern "C" {
+#pragma GCC visibility push(default)
+
+const char *hctr_last_error(void) { return g_error.c_str(); }
+const char *hctr_version(void) { return "hetuctr-hip 0.1 (gfx950)"; }
+void hctr_seed(unsigned long seed) { g_seed = seed; }
+
+int hctr_create(const hctr_config *cfg, const uint8_t *root_arr, const int64_t *storage_arr, size_t n_storage,
+                hctr_table **out) {
+  return guarded([&] {
+    HCTR_CHECK(cfg && out, "null argument");
+    *out = nullptr;
+    HCTR_CHECK(cfg->nrank >= 1 && cfg->nrank <= 256, "nrank must be in 1..256 (worker ids are one byte)");
+    auto group = find_or_create_group(cfg->nrank, cfg->device_id, cfg->ip ? cfg->ip : "", cfg->port);
+    // the reference passes the global seed as an unsigned int (table_initialize.cu:156, initializer.h:37)
+    Shard *s = new Shard(*cfg, root_arr, storage_arr, n_storage, (unsigned)g_seed.load(), group);
+    try {
+      group->join(s);
+    } catch (...) {
+      delete s;
+      throw;
+    }
+    if (cfg->verbose >= 1)
+      printf("HetuTable rank %d: Table Init Successfully (%zu rows resident, %u cached)\n", cfg->rank, n_storage,
+             s->tv.n_cached);
+    *out = new hctr_table{s};
+  });
+}
+
+int hctr_destroy(hctr_table *t) {
+  return guarded([&] {
+    if (!t) return;
+    if (t->shard) {
+      (void)hipSetDevice(t->shard->cfg.device_id);
+      (void)hipStreamSynchronize(t->shard->group->stream);
+      t->shard->group->leave(t->shard);
+      delete t->shard;
+    }
+    delete t;
+  });
+}
+
+int hctr_preprocess(hctr_table *t, const int64_t *keys, size_t n) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->group->preprocess_one(t->shard->cfg.rank, keys, n);
+  });
+}
+
+int hctr_push_pull(hctr_table *t, const float *grad, float *dst) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->group->push_pull_one(t->shard->cfg.rank, grad, dst);
+  });
+}
+
+static Group *group_of(hctr_table *const *tables, int nrank) {
+  HCTR_CHECK(tables && nrank >= 1, "null table list");
+  for (int r = 0; r < nrank; r++) HCTR_CHECK(tables[r] && tables[r]->shard, "null table");
+  Group *g = tables[0]->shard->group.get();
+  HCTR_CHECK(g->nrank == nrank, "the table list must hold every rank of the group");
+  for (int r = 0; r < nrank; r++)
+    HCTR_CHECK(tables[r]->shard->group.get() == g && tables[r]->shard->cfg.rank == r,
+               "tables[r] must be rank r of one group");
+  return g;
+}
+
+int hctr_group_preprocess(hctr_table *const *tables, int nrank, const int64_t *const *keys, const size_t *n) {
+  return guarded([&] { group_of(tables, nrank)->preprocess_all(keys, n); });
+}
+
+int hctr_group_push_pull(hctr_table *const *tables, int nrank, const float *const *grads, float *const *dsts) {
+  return guarded([&] { group_of(tables, nrank)->push_pull_all(grads, dsts); });
+}
+
+// csrc/core/debug.cu:5-12
+int hctr_repr(hctr_table *t, char *buf, size_t cap) {
+  if (!t || !t->shard) return -1;
+  char b[256];
+  const Shard &s = *t->shard;
+  snprintf(b, sizeof b, "<HetuTable root/store/all=%ld/%ld/%ld>", (long)(s.tv.n_stored - s.tv.n_cached),
+           (long)s.tv.n_stored, (long)s.tv.id_max);
+  return write_string(b, buf, cap);
+}
+
+// csrc/core/debug.cu:14-24
+int hctr_debug(hctr_table *t, char *buf, size_t cap) {
+  if (!t || !t->shard) return -1;
+  char b[512];
+  const Shard &s = *t->shard;
+  snprintf(b, sizeof b, "<HetuTable root/store/all=%ld/%ld/%ld rank=%d nrank=%d device_id=%d width=%ld push/pull=%lld/%lld>",
+           (long)(s.tv.n_stored - s.tv.n_cached), (long)s.tv.n_stored, (long)s.tv.id_max, s.cfg.rank, s.cfg.nrank,
+           s.cfg.device_id, (long)s.tv.width, (long long)s.tv.push_bound, (long long)s.tv.pull_bound);
+  return write_string(b, buf, cap);
+}
+
+int hctr_debug_fetch(hctr_table *t, int which, void *host_out, size_t cap_elems, size_t *n_elems) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    const size_t n = t->shard->fetch(which, host_out, host_out ? cap_elems : 0);
+    if (n_elems) *n_elems = n;
+  });
+}
+
+int hctr_stream(hctr_table *t, void **stream_out) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard && stream_out, "null argument");
+    *stream_out = (void *)t->shard->group->stream;
+  });
+}
+
+int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    if (preprocess_ms) *preprocess_ms = t->shard->last_pre_ms;
+    if (push_pull_ms) *push_pull_ms = t->shard->last_pp_ms;
+  });
+}
+
+#pragma GCC visibility pop
+} // extern "C"

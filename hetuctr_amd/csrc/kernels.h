@@ -1,0 +1,111 @@
+// Host-callable launchers of the hot-path kernels.  Each one only enqueues work on `stream`.
+// Reference stages are cited where the launcher is defined.
+#pragma once
+#include "common.h"
+
+namespace hctr {
+
+// The sort key of a batch position: (owner << id_bits) | id.  Its order is the reference's
+// id + kEmbeddingIDMax*owner (csrc/core/preprocess.cu:17): owner first, id second.
+struct KeyLayout {
+  int id_bits;    // bits of an id
+  int total_bits; // id_bits + bits of an owner
+  bool wide;      // 64-bit sort keys (total_bits > 32)
+};
+
+// Device-side view of one preprocessed batch (the reference's PreprocessData,
+// csrc/core/preprocess_struct.h:7-24, with 32-bit positions and ranks).
+struct BatchView {
+  uint32_t n;                // keys in the batch (host-known)
+  const index_t *keys;       // [n]   the ids as handed in                      (d_idx)
+  uint32_t *sorted_arg;      // [n]   positions grouped by unique key, stable   (d_sorted_arg)
+  uint32_t *rank_sorted;     // [n]   unique rank of sorted position j
+  uint32_t *idx_map;         // [n]   unique rank of position i                 (d_idx_map)
+  void *ukey;                // [U]   sort key of unique rank u: id and owner   (d_unique_idx, d_root)
+  uint32_t *run_start;       // [U+1] first sorted position of rank u           (d_run_length)
+  slot_t *uoff;              // [U]   resident offset of rank u or -1           (d_offset)
+  uint32_t *bucket_lo;       // [R+1] first rank owned by each shard            (u_shape before :131)
+  uint32_t *d_U;             // [1]   number of unique keys                     (unique_size)
+};
+
+struct TableView {
+  int rank, nrank;
+  uint64_t id_max;
+  uint32_t width;
+  uint32_t n_stored, n_cached;   // kStorageMax, kNonLocalStorageMax
+  float neg_lr;
+  version_t pull_bound, push_bound;
+  const worker_t *root;          // [id_max]
+  const slot_t *slot;            // [id_max]  id -> resident offset or -1
+  embed_t *emb;                  // [n_stored][width]
+  version_t *ver;                // [n_stored]
+  embed_t *pend;                 // [n_cached][width]
+  version_t *upd;                // [n_cached]
+};
+
+// ---- preprocess ---------------------------------------------------------------------------------
+// ids -> sort keys; flags ids outside [0, id_max) in *err (and sorts them as id 0)
+void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
+                      void *comp_keys, uint32_t *err);
+// sorted keys -> everything per unique key + inverse index.  block_heads: scratch of sort_blocks(n) words.
+void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
+                   const BatchView &b, uint32_t *block_heads);
+
+// device-wide exclusive scan of n (<= *d_n if d_n != nullptr) 32-bit values; block_sums: div_up(n_max,2048)+1 words.
+// total (optional) receives the sum.
+void launch_exclusive_scan(hipStream_t s, const uint32_t *in, uint32_t *out, uint32_t n_max, const uint32_t *d_n,
+                           uint32_t *block_sums, uint32_t *total);
+
+// push plan of the previous batch (csrc/core/preprocess.cu:148-165): need[u] in {0,1}
+void launch_decide_update(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &prev,
+                          uint32_t *need);
+// pushed rows per owner from the scanned plan: cnt[d] = prefix[lo[d+1]] - prefix[lo[d]]
+void launch_bucket_counts(hipStream_t s, const BatchView &b, const uint32_t *prefix, const uint32_t *total,
+                          int nrank, uint64_t *cnt_out);
+void launch_bucket_sizes(hipStream_t s, const BatchView &b, int nrank, uint64_t *cnt_out);
+
+// ---- push: segment-sum of gradients by unique key + fused SGD ----------------------------------------
+struct PushArgs {
+  const embed_t *grad;       // [n_prev][width]
+  const uint32_t *need;      // [U_prev] or nullptr when nrank == 1
+  const uint32_t *prefix;    // [U_prev] push slot
+  index_t *g_idx;            // push buffers
+  version_t *g_cnt;
+  embed_t *g_val;
+};
+size_t push_tiles(uint32_t n_prev);
+void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &prev, const PushArgs &a);
+
+// ---- query / owner side / pull -------------------------------------------------------------------------
+void launch_lookup_version(hipStream_t s, const TableView &t, const BatchView &cur, version_t *q_ver);
+void launch_unique_ids(hipStream_t s, const KeyLayout &kl, const BatchView &cur, index_t *q_idx);
+// owner: received pushes of ONE source, [lo, hi) of the receive buffers
+void launch_apply_remote(hipStream_t s, const TableView &t, const index_t *rg_idx, const version_t *rg_cnt,
+                         const embed_t *rg_val, uint32_t lo, uint32_t hi, uint32_t *err);
+// owner: outdated flag per received query; queries in [self_lo, self_hi) came from this shard itself
+void launch_decide_outdated(hipStream_t s, const TableView &t, const index_t *rq_idx, const version_t *rq_ver,
+                            uint32_t q, uint32_t self_lo, uint32_t self_hi, uint32_t *outdated, uint32_t *err);
+// owner: pack version + row of every flagged query at its compacted position
+void launch_pack_rows(hipStream_t s, const TableView &t, const index_t *rq_idx, const uint32_t *outdated,
+                      const uint32_t *out_pos, uint32_t q, version_t *ret_ver, embed_t *ret_val);
+// requester: refresh cached rows that came back, then gather every key's row into dst
+struct PullArgs {
+  const uint32_t *got;       // [U] or nullptr: nothing came back (nrank == 1)
+  const uint32_t *ret_i;     // [U] index into the returned rows
+  const version_t *in_ver;
+  const embed_t *in_val;
+  embed_t *dst;              // [n][width]
+};
+void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a, uint32_t *stats);
+void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a);
+
+// ---- init -------------------------------------------------------------------------------------------------
+void launch_init_values(hipStream_t s, embed_t *out, size_t len, int type, float a, float b, unsigned seed);
+void launch_fill_i64(hipStream_t s, version_t *p, size_t n, version_t v);
+void launch_fill_i32(hipStream_t s, int32_t *p, size_t n, int32_t v);
+void launch_build_directory(hipStream_t s, const index_t *store_ids, uint32_t n_stored, slot_t *slot);
+// segmented copies of an exchange: n descriptors {src, dst, bytes}
+struct CopyDesc { const void *src; void *dst; size_t bytes; };
+void launch_copies(hipStream_t s, const CopyDesc *descs_device, uint32_t n, size_t max_bytes);
+
+} // namespace hctr

@@ -1,0 +1,249 @@
+// Key preprocess of one batch after the sort: unique keys, run starts, inverse index, owner buckets,
+// resident offsets; and the push plan of the previous batch.
+// Reference: csrc/core/preprocess.cu:11-182 (kernels generate_sort_kv, write_sort_result,
+// preprocess_batch_data, compute_idx_map, block_cvt_offset_to_shape, decide_update and the
+// cub RunLengthEncode / ExclusiveSum calls between them).
+#include "kernels.h"
+#include "radix_sort.h"
+
+namespace hctr {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kItems = 8;
+constexpr int kTile = kBlock * kItems; // == kSortTile, so sort_blocks(n) sizes the scratch
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
+                                                    int id_bits, int nrank, const worker_t *__restrict__ root,
+                                                    K *__restrict__ comp, uint32_t *__restrict__ err) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  uint64_t id = (uint64_t)keys[i];
+  if (id >= id_max) { // also catches negative ids
+    atomicOr(err, 1u);
+    id = 0;
+  }
+  const uint64_t r = nrank > 1 ? root[id] : 0;
+  comp[i] = (K)((r << id_bits) | id);
+}
+
+template <typename K>
+__device__ __forceinline__ void load_tile(const K *__restrict__ sk, uint32_t n, uint32_t j0, K (&key)[kItems], K &prev) {
+#pragma unroll
+  for (int k = 0; k < kItems; k++) key[k] = (j0 + k < n) ? sk[j0 + k] : (K)0;
+  prev = (j0 > 0 && j0 <= n) ? sk[j0 - 1] : (K)0;
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void head_count(const K *__restrict__ sk, uint32_t n,
+                                                     uint32_t *__restrict__ block_heads) {
+  __shared__ uint32_t sm[kBlock / kWave + 1];
+  const uint32_t j0 = blockIdx.x * kTile + threadIdx.x * kItems;
+  K key[kItems], prev;
+  load_tile(sk, n, j0, key, prev);
+  uint32_t c = 0;
+#pragma unroll
+  for (int k = 0; k < kItems; k++) {
+    const uint32_t j = j0 + k;
+    c += (j < n) && (j == 0 || key[k] != (k ? key[k - 1] : prev));
+  }
+  uint32_t total;
+  block_exclusive_scan<kBlock>(c, sm, total);
+  if (threadIdx.x == 0) block_heads[blockIdx.x] = total;
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void unique_emit(const K *__restrict__ sk, uint32_t n, int id_bits, int nrank,
+                                                      const slot_t *__restrict__ slot,
+                                                      const uint32_t *__restrict__ block_heads, BatchView b) {
+  __shared__ uint32_t sm[kBlock / kWave + 1];
+  // ranks before this block
+  uint32_t s = 0;
+  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlock) s += block_heads[i];
+  uint32_t prefix;
+  block_exclusive_scan<kBlock>(s, sm, prefix);
+
+  const uint32_t j0 = blockIdx.x * kTile + threadIdx.x * kItems;
+  K key[kItems], prev;
+  load_tile(sk, n, j0, key, prev);
+  bool head[kItems];
+  uint32_t c = 0;
+#pragma unroll
+  for (int k = 0; k < kItems; k++) {
+    const uint32_t j = j0 + k;
+    head[k] = (j < n) && (j == 0 || key[k] != (k ? key[k - 1] : prev));
+    c += head[k];
+  }
+  uint32_t total;
+  uint32_t run = prefix + block_exclusive_scan<kBlock>(c, sm, total); // heads before this thread's items
+  K *ukey = (K *)b.ukey;
+  const K id_mask = (K)(((uint64_t)1 << id_bits) - 1);
+#pragma unroll
+  for (int k = 0; k < kItems; k++) {
+    const uint32_t j = j0 + k;
+    if (j >= n) break;
+    run += head[k];
+    const uint32_t rank = run - 1;
+    const int r = (int)(key[k] >> id_bits);
+    if (head[k]) {
+      ukey[rank] = key[k];
+      b.run_start[rank] = j;
+      b.uoff[rank] = slot[(uint64_t)(key[k] & id_mask)];
+      const K pk = k ? key[k - 1] : prev;
+      const int r_prev = j == 0 ? -1 : (int)(pk >> id_bits);
+      for (int i = r_prev + 1; i <= r; i++) b.bucket_lo[i] = rank;
+    }
+    b.rank_sorted[j] = rank;
+    b.idx_map[b.sorted_arg[j]] = rank;
+    if (j == n - 1) {
+      const uint32_t U = rank + 1;
+      *b.d_U = U;
+      b.run_start[U] = n;
+      for (int i = r + 1; i <= nrank; i++) b.bucket_lo[i] = U;
+    }
+  }
+}
+
+// ---- generic device-wide exclusive scan (two launches, no inter-block waiting) ----------------------
+__global__ __launch_bounds__(kBlock) void scan_block_sums(const uint32_t *__restrict__ in, uint32_t n_max,
+                                                          const uint32_t *__restrict__ d_n,
+                                                          uint32_t *__restrict__ block_sums) {
+  __shared__ uint32_t sm[kBlock / kWave + 1];
+  const uint32_t n = d_n ? min(*d_n, n_max) : n_max;
+  const uint32_t j0 = blockIdx.x * kTile + threadIdx.x * kItems;
+  uint32_t c = 0;
+#pragma unroll
+  for (int k = 0; k < kItems; k++) c += (j0 + k < n) ? in[j0 + k] : 0u;
+  uint32_t total;
+  block_exclusive_scan<kBlock>(c, sm, total);
+  if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_emit(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
+                                                    uint32_t n_max, const uint32_t *__restrict__ d_n,
+                                                    const uint32_t *__restrict__ block_sums,
+                                                    uint32_t *__restrict__ total_out) {
+  __shared__ uint32_t sm[kBlock / kWave + 1];
+  const uint32_t n = d_n ? min(*d_n, n_max) : n_max;
+  uint32_t s = 0;
+  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlock) s += block_sums[i];
+  uint32_t prefix;
+  block_exclusive_scan<kBlock>(s, sm, prefix);
+  const uint32_t j0 = blockIdx.x * kTile + threadIdx.x * kItems;
+  uint32_t v[kItems], c = 0;
+#pragma unroll
+  for (int k = 0; k < kItems; k++) {
+    v[k] = (j0 + k < n) ? in[j0 + k] : 0u;
+    c += v[k];
+  }
+  uint32_t total;
+  uint32_t run = prefix + block_exclusive_scan<kBlock>(c, sm, total);
+#pragma unroll
+  for (int k = 0; k < kItems; k++) {
+    if (j0 + k < n) out[j0 + k] = run;
+    run += v[k];
+  }
+  if (total_out && blockIdx.x == gridDim.x - 1 && threadIdx.x == kBlock - 1) *total_out = run;
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void decide_update(TableView t, int id_bits, BatchView p,
+                                                        uint32_t *__restrict__ need) {
+  const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
+  if (u >= *p.d_U) return;
+  const K key = ((const K *)p.ukey)[u];
+  const int r = (int)(key >> id_bits);
+  const slot_t o = p.uoff[u];
+  const version_t cnt = (version_t)(p.run_start[u + 1] - p.run_start[u]);
+  uint32_t nd;
+  if (r == t.rank) nd = 0;
+  else if (o == kNoSlot) nd = 1;
+  else nd = (t.upd[o] + cnt <= t.push_bound) ? 0 : 1;
+  need[u] = nd;
+}
+
+__global__ void bucket_counts(BatchView b, const uint32_t *__restrict__ prefix, const uint32_t *__restrict__ total,
+                              int nrank, uint64_t *__restrict__ cnt_out) {
+  const int d = threadIdx.x;
+  if (d > nrank) return;
+  if (d == nrank) { cnt_out[d] = 0; return; }
+  const uint32_t U = *b.d_U;
+  const uint32_t lo = b.bucket_lo[d], hi = b.bucket_lo[d + 1];
+  const uint32_t a = lo >= U ? *total : prefix[lo];
+  const uint32_t e = hi >= U ? *total : prefix[hi];
+  cnt_out[d] = U ? (uint64_t)(e - a) : 0;
+}
+
+__global__ void bucket_sizes(BatchView b, int nrank, uint64_t *__restrict__ cnt_out) {
+  const int d = threadIdx.x;
+  if (d > nrank) return;
+  cnt_out[d] = d == nrank ? 0 : (uint64_t)(b.bucket_lo[d + 1] - b.bucket_lo[d]);
+}
+
+} // namespace
+
+void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
+                      void *comp_keys, uint32_t *err) {
+  if (!n) return;
+  if (kl.wide)
+    hipLaunchKernelGGL(make_keys<uint64_t>, dim3(div_up(n, kBlock)), dim3(kBlock), 0, s, keys, n, t.id_max,
+                       kl.id_bits, t.nrank, t.root, (uint64_t *)comp_keys, err);
+  else
+    hipLaunchKernelGGL(make_keys<uint32_t>, dim3(div_up(n, kBlock)), dim3(kBlock), 0, s, keys, n, t.id_max,
+                       kl.id_bits, t.nrank, t.root, (uint32_t *)comp_keys, err);
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
+                   const BatchView &b, uint32_t *block_heads) {
+  if (!b.n) return;
+  const unsigned nb = div_up(b.n, kTile);
+  if (kl.wide) {
+    hipLaunchKernelGGL(head_count<uint64_t>, dim3(nb), dim3(kBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
+                       block_heads);
+    hipLaunchKernelGGL(unique_emit<uint64_t>, dim3(nb), dim3(kBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
+                       kl.id_bits, t.nrank, t.slot, block_heads, b);
+  } else {
+    hipLaunchKernelGGL(head_count<uint32_t>, dim3(nb), dim3(kBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
+                       block_heads);
+    hipLaunchKernelGGL(unique_emit<uint32_t>, dim3(nb), dim3(kBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
+                       kl.id_bits, t.nrank, t.slot, block_heads, b);
+  }
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_exclusive_scan(hipStream_t s, const uint32_t *in, uint32_t *out, uint32_t n_max, const uint32_t *d_n,
+                           uint32_t *block_sums, uint32_t *total) {
+  if (!n_max) {
+    if (total) HCTR_HIP(hipMemsetAsync(total, 0, sizeof(uint32_t), s));
+    return;
+  }
+  const unsigned nb = div_up(n_max, kTile);
+  hipLaunchKernelGGL(scan_block_sums, dim3(nb), dim3(kBlock), 0, s, in, n_max, d_n, block_sums);
+  hipLaunchKernelGGL(scan_emit, dim3(nb), dim3(kBlock), 0, s, in, out, n_max, d_n, block_sums, total);
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_decide_update(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &prev,
+                          uint32_t *need) {
+  if (!prev.n) return;
+  if (kl.wide)
+    hipLaunchKernelGGL(decide_update<uint64_t>, dim3(div_up(prev.n, kBlock)), dim3(kBlock), 0, s, t, kl.id_bits, prev, need);
+  else
+    hipLaunchKernelGGL(decide_update<uint32_t>, dim3(div_up(prev.n, kBlock)), dim3(kBlock), 0, s, t, kl.id_bits, prev, need);
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_bucket_counts(hipStream_t s, const BatchView &b, const uint32_t *prefix, const uint32_t *total,
+                          int nrank, uint64_t *cnt_out) {
+  hipLaunchKernelGGL(bucket_counts, dim3(1), dim3(nrank + 1), 0, s, b, prefix, total, nrank, cnt_out);
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_bucket_sizes(hipStream_t s, const BatchView &b, int nrank, uint64_t *cnt_out) {
+  hipLaunchKernelGGL(bucket_sizes, dim3(1), dim3(nrank + 1), 0, s, b, nrank, cnt_out);
+  HCTR_HIP(hipGetLastError());
+}
+
+} // namespace hctr

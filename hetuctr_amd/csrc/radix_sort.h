@@ -1,0 +1,37 @@
+// Stable least-significant-digit radix sort of (key, position) pairs for one batch of sparse ids.
+// Replaces cub::DeviceRadixSort::SortPairs at csrc/core/preprocess.cu:105-109 of the reference.
+#pragma once
+#include "common.h"
+
+namespace hctr {
+
+constexpr int kSortBlock = 256;                 // threads per block (4 waves)
+constexpr int kSortItems = 8;                   // keys per thread
+constexpr int kSortTile = kSortBlock * kSortItems;
+constexpr int kSortMaxDigitBits = 10;           // up to 1024 bins: 4 wave-private rows of 4 KiB in LDS
+
+struct SortScratch {
+  uint32_t *ghist = nullptr;   // [bins][blocks] per-block digit counts, scanned in place per bin
+  uint32_t *bintot = nullptr;  // [bins] totals per digit value
+  size_t blocks_cap = 0;
+};
+
+inline size_t sort_blocks(size_t n) { return (n + kSortTile - 1) / kSortTile; }
+
+// Sorts n pairs by the low `bits` bits of the key.  The value of element i is its position i (never
+// materialised as an input).  keys_in is left untouched; tmp_k0/tmp_k1 and tmp_v0/tmp_v1 are ping-pong
+// buffers of n elements; the sorted keys end in *keys_sorted (one of tmp_k0/tmp_k1) and the sorted
+// positions in vals_out.  n == 0 is a no-op.
+template <typename K>
+void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
+                          uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
+                          const K **keys_sorted);
+
+extern template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *,
+                                                    uint32_t *, uint32_t *, uint32_t *, uint32_t *,
+                                                    const SortScratch &, const uint32_t **);
+extern template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *,
+                                                    uint64_t *, uint32_t *, uint32_t *, uint32_t *,
+                                                    const SortScratch &, const uint64_t **);
+
+} // namespace hctr

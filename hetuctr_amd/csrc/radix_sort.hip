@@ -1,0 +1,187 @@
+// Stable LSD radix sort for gfx950, 64-lane wavefronts.
+//
+// One pass = three launches:
+//   digit_histogram   per-block digit counts (LDS atomics) -> ghist[bin][block]
+//   scan_bins         one block per digit value: exclusive scan of its row over the blocks + row total
+//   scatter           per block: global base of every bin, stable rank of every key inside the block
+//                     (wave-level match by ballots, wave-private LDS counters), scatter to the output
+// Stability: a block's tile is split into 4 contiguous sub-tiles, one per wave; a wave walks its
+// sub-tile 64 keys at a time in ascending position; inside such a group the rank among equal digits is
+// the lane order.  Wave-private counters make the result independent of wave scheduling.
+#include "radix_sort.h"
+
+namespace hctr {
+namespace {
+
+constexpr int kWaves = kSortBlock / kWave;
+constexpr int kSub = kSortTile / kWaves; // keys per wave
+constexpr int kRounds = kSub / kWave;    // 64-key groups per wave
+
+template <typename K>
+__global__ __launch_bounds__(kSortBlock) void digit_histogram(const K *__restrict__ keys, uint32_t n, int shift,
+                                                              int dbits, uint32_t *__restrict__ ghist,
+                                                              uint32_t nblocks) {
+  __shared__ uint32_t h[1 << kSortMaxDigitBits];
+  const uint32_t nb = 1u << dbits, mask = nb - 1;
+  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
+  __syncthreads();
+  const uint32_t base = blockIdx.x * kSortTile;
+#pragma unroll
+  for (int k = 0; k < kSortItems; k++) {
+    uint32_t idx = base + k * kSortBlock + threadIdx.x;
+    if (idx < n) atomicAdd(&h[(uint32_t)(keys[idx] >> shift) & mask], 1u);
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) ghist[(size_t)i * nblocks + blockIdx.x] = h[i];
+}
+
+// grid = number of bins; block b scans row b of ghist in place (exclusive) and writes its total
+__global__ __launch_bounds__(kSortBlock) void scan_bins(uint32_t *__restrict__ ghist, uint32_t nblocks,
+                                                        uint32_t *__restrict__ bintot) {
+  __shared__ uint32_t sm[kWaves + 1];
+  uint32_t *row = ghist + (size_t)blockIdx.x * nblocks;
+  const uint32_t per = (nblocks + kSortBlock - 1) / kSortBlock;
+  const uint32_t lo = min(threadIdx.x * per, nblocks), hi = min(lo + per, nblocks);
+  uint32_t s = 0;
+  for (uint32_t i = lo; i < hi; i++) s += row[i];
+  uint32_t total;
+  uint32_t off = block_exclusive_scan<kSortBlock>(s, sm, total);
+  for (uint32_t i = lo; i < hi; i++) {
+    uint32_t v = row[i];
+    row[i] = off;
+    off += v;
+  }
+  if (threadIdx.x == 0) bintot[blockIdx.x] = total;
+}
+
+template <typename K, bool kFirst>
+__global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
+                                                      K *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
+                                                      uint32_t n, int shift, int dbits,
+                                                      const uint32_t *__restrict__ ghist, uint32_t nblocks,
+                                                      const uint32_t *__restrict__ bintot) {
+  __shared__ uint32_t cnt[kWaves][1 << kSortMaxDigitBits];
+  __shared__ uint32_t base[1 << kSortMaxDigitBits];
+  __shared__ uint32_t sm[kWaves + 1];
+  const uint32_t nb = 1u << dbits, mask = nb - 1;
+  const int w = threadIdx.x / kWave;
+  const unsigned lane = lane_id();
+
+  // global base of each bin for this block: sum of the totals of lower bins + this bin's lower blocks.
+  // 256 threads, up to 1024 bins: 4 consecutive bins per thread.
+  {
+    const uint32_t per = (nb + kSortBlock - 1) / kSortBlock;
+    const uint32_t lo = min(threadIdx.x * per, nb), hi = min(lo + per, nb);
+    uint32_t s = 0;
+    for (uint32_t i = lo; i < hi; i++) s += bintot[i];
+    uint32_t total;
+    uint32_t off = block_exclusive_scan<kSortBlock>(s, sm, total);
+    for (uint32_t i = lo; i < hi; i++) {
+      base[i] = off + ghist[(size_t)i * nblocks + blockIdx.x];
+      off += bintot[i];
+    }
+  }
+  for (uint32_t i = threadIdx.x; i < kWaves * nb; i += kSortBlock) cnt[i / nb][i % nb] = 0;
+  __syncthreads();
+
+  K key[kRounds];
+  uint32_t val[kRounds];
+  uint32_t dig[kRounds];  // digit | local rank << 10 would overflow for rank up to 512: keep separate
+  uint32_t rnk[kRounds];
+  const uint32_t wbase = blockIdx.x * kSortTile + w * kSub;
+#pragma unroll
+  for (int r = 0; r < kRounds; r++) {
+    const uint32_t idx = wbase + r * kWave + lane;
+    const bool valid = idx < n;
+    key[r] = valid ? keys_in[idx] : (K)0;
+    val[r] = kFirst ? idx : (valid ? vals_in[idx] : 0u);
+    const uint32_t d = (uint32_t)(key[r] >> shift) & mask;
+    uint64_t m = __ballot(valid);
+    for (int b = 0; b < dbits; b++) {
+      const bool bit = (d >> b) & 1u;
+      const uint64_t bal = __ballot(bit);
+      m &= bit ? bal : ~bal;
+    }
+    // m: valid lanes of this group with the same digit (meaningless on invalid lanes)
+    const uint32_t before = __popcll(m & ((1ull << lane) - 1ull));
+    uint32_t prior = 0;
+    if (valid) prior = cnt[w][d];
+    __builtin_amdgcn_wave_barrier();
+    const bool leader = valid && (m >> lane) == 1ull; // highest lane of the match group
+    if (leader) cnt[w][d] = prior + before + 1;
+    __builtin_amdgcn_wave_barrier();
+    dig[r] = d;
+    rnk[r] = prior + before;
+  }
+  __syncthreads();
+  // wave-private counts -> start of each wave's keys inside the bin, plus the bin's global base
+  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) {
+    uint32_t run = base[i];
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ww++) {
+      uint32_t t = cnt[ww][i];
+      cnt[ww][i] = run;
+      run += t;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kRounds; r++) {
+    const uint32_t idx = wbase + r * kWave + lane;
+    if (idx < n) {
+      const uint32_t pos = cnt[w][dig[r]] + rnk[r];
+      keys_out[pos] = key[r];
+      vals_out[pos] = val[r];
+    }
+  }
+}
+
+} // namespace
+
+template <typename K>
+void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
+                          uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
+                          const K **keys_sorted) {
+  *keys_sorted = keys_in;
+  if (n == 0) return;
+  if (bits < 1) bits = 1;
+  HCTR_CHECK(bits <= (int)sizeof(K) * 8, "sort key wider than its type");
+  const uint32_t nblocks = (uint32_t)sort_blocks(n);
+  HCTR_CHECK(nblocks <= scratch.blocks_cap, "sort scratch too small");
+  const int passes = (bits + kSortMaxDigitBits - 1) / kSortMaxDigitBits;
+  int shift = 0;
+  const K *kin = keys_in;
+  const uint32_t *vin = nullptr;
+  K *ktmp[2] = {tmp_k0, tmp_k1};
+  uint32_t *vtmp[2] = {tmp_v0, tmp_v1};
+  for (int p = 0; p < passes; p++) {
+    const int left = bits - shift;
+    const int dbits = (left + (passes - p) - 1) / (passes - p);
+    K *kout = ktmp[p & 1];
+    uint32_t *vout = (p == passes - 1) ? vals_out : vtmp[p & 1];
+    const uint32_t nb = 1u << dbits;
+    hipLaunchKernelGGL(digit_histogram<K>, dim3(nblocks), dim3(kSortBlock), 0, stream, kin, n, shift, dbits,
+                       scratch.ghist, nblocks);
+    hipLaunchKernelGGL(scan_bins, dim3(nb), dim3(kSortBlock), 0, stream, scratch.ghist, nblocks, scratch.bintot);
+    if (p == 0)
+      hipLaunchKernelGGL((scatter<K, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
+                         shift, dbits, scratch.ghist, nblocks, scratch.bintot);
+    else
+      hipLaunchKernelGGL((scatter<K, false>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
+                         shift, dbits, scratch.ghist, nblocks, scratch.bintot);
+    HCTR_HIP(hipGetLastError());
+    kin = kout;
+    vin = vout;
+    shift += dbits;
+  }
+  *keys_sorted = kin;
+}
+
+template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *, uint32_t *,
+                                             uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
+                                             const uint32_t **);
+template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *, uint64_t *,
+                                             uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
+                                             const uint64_t **);
+
+} // namespace hctr

@@ -1,0 +1,173 @@
+// Host-side state of one shard (the reference's HetuTable, csrc/core/hetu_gpu_table.h:21-144) and of the
+// in-process loopback group that stands in for the NCCL communicator.
+#pragma once
+#include <condition_variable>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/hetuctr_hip.h"
+#include "kernels.h"
+#include "radix_sort.h"
+
+namespace hctr {
+
+// growable device allocation; contents are NOT kept when it grows
+struct DeviceBuf {
+  void *p = nullptr;
+  size_t bytes = 0;
+  DeviceBuf() = default;
+  DeviceBuf(const DeviceBuf &) = delete;
+  DeviceBuf &operator=(const DeviceBuf &) = delete;
+  DeviceBuf(DeviceBuf &&o) noexcept : p(o.p), bytes(o.bytes) { o.p = nullptr; o.bytes = 0; }
+  DeviceBuf &operator=(DeviceBuf &&o) noexcept {
+    if (this != &o) {
+      release();
+      p = o.p;
+      bytes = o.bytes;
+      o.p = nullptr;
+      o.bytes = 0;
+    }
+    return *this;
+  }
+  ~DeviceBuf() { release(); }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    bytes = 0;
+  }
+  void reserve(size_t want) {
+    if (want <= bytes) return;
+    release();
+    size_t grow = want + want / 8; // headroom so that slowly growing batches do not reallocate every step
+    HCTR_HIP(hipMalloc(&p, grow));
+    bytes = grow;
+  }
+  template <typename T> T *as() const { return (T *)p; }
+};
+
+// per-batch buffers: the reference's PreprocessData (csrc/core/preprocess_struct.h:7-24)
+struct Batch {
+  uint32_t n = 0;   // keys
+  uint32_t U = 0;   // unique keys (host copy, valid after the preprocess call returned)
+  DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU;
+  std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
+  std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
+  void reserve(uint32_t n_keys, int nrank, bool wide);
+  BatchView view() const;
+};
+
+// values the host reads back after a call; lives in pinned host memory
+struct HostMirror {
+  uint32_t U;
+  uint32_t err;
+  uint32_t push_total;
+  uint32_t ret_total;
+  uint32_t stats[4];
+  uint64_t send_cnt[257];
+  uint64_t push_cnt[257];
+  uint32_t ret_seg[258];
+};
+
+class Group;
+
+class Shard {
+ public:
+  Shard(const hctr_config &cfg, const uint8_t *root_arr, const int64_t *storage_arr, size_t n_storage,
+        unsigned seed, std::shared_ptr<Group> group);
+  ~Shard();
+
+  hctr_config cfg;
+  std::string ip;
+  std::shared_ptr<Group> group;
+  KeyLayout kl;
+  TableView tv;
+  size_t n_owned = 0;
+
+  // ---- stages, each only enqueues on the group's stream (names follow hetu_gpu_table.h:82-97) ----
+  void swap_batches() { std::swap(cur, prev); }
+  void preprocess_index(const int64_t *keys, size_t n);
+  void preprocess_gradient();
+  void enqueue_readback_preprocess();
+  void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
+  void generate_gradient(const float *grad);
+  void generate_query();
+  void handle_gradient();
+  void handle_query();
+  void finish_handle_query();               // after the mid-step sync
+  void write_back(float *dst);
+  void finish_push_pull();
+
+  size_t fetch(int which, void *host_out, size_t cap);
+
+  Batch cur, prev;
+  bool prev_active = false; // false: inference step or no previous batch, nothing is pushed
+  DeviceBuf root, slot, emb, ver, pend, upd, store_ids;
+  // scratch shared by the stages
+  DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, ghist, bintot, block_sums, err, stats;
+  DeviceBuf need, prefix, push_total, cnt_dev;
+  // send side
+  DeviceBuf q_idx, q_ver, g_idx, g_cnt, g_val;
+  // receive side (owner role)
+  DeviceBuf rq_idx, rq_ver, rg_idx, rg_cnt, rg_val, outdated, out_pos, ret_total, ret_ver, ret_val, ret_seg_dev;
+  std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
+  // requester side of the return
+  DeviceBuf got, ret_i, in_ver, in_val;
+  uint64_t in_rows = 0;
+  HostMirror *mirror = nullptr;
+  long long last_stats[6] = {0, 0, 0, 0, 0, 0};
+  float last_pre_ms = 0.f, last_pp_ms = 0.f;
+
+ private:
+  void reserve_batch_scratch(uint32_t n);
+};
+
+// All shards of one loopback group live in one process on one device and share one stream.  The group
+// carries the collective calls: every shard's thread deposits its arguments, the last one to arrive runs the
+// step for all shards, the others wait for it.
+class Group {
+ public:
+  Group(int nrank, int device_id, std::string key);
+  ~Group();
+  const int nrank;
+  const int device_id;
+  const std::string key;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  std::vector<Shard *> members;
+  DeviceBuf desc_dev;
+  CopyDesc *desc_host = nullptr;
+  size_t desc_cap = 0;
+  double wait_seconds = 120.0;
+
+  void join(Shard *s);
+  void leave(Shard *s);
+  bool complete() const;
+
+  // lock-step bodies (one caller)
+  void preprocess_all(const int64_t *const *keys, const size_t *n);
+  void push_pull_all(const float *const *grads, float *const *dsts);
+  // per-shard entry points: rendezvous of nrank callers
+  void preprocess_one(int rank, const int64_t *keys, size_t n);
+  void push_pull_one(int rank, const float *grad, float *dst);
+
+ private:
+  void exchange_query();
+  void exchange_return();
+  void run_copies(std::vector<CopyDesc> &descs);
+  template <typename F> void collective(int rank, int op, F &&run_all);
+  std::mutex mu_;
+  std::condition_variable cv_;
+  int arrived_ = 0, pending_op_ = 0;
+  uint64_t generation_ = 0;
+  std::string failure_;
+  std::vector<const int64_t *> a_keys_;
+  std::vector<size_t> a_n_;
+  std::vector<const float *> a_grad_;
+  std::vector<float *> a_dst_;
+};
+
+std::shared_ptr<Group> find_or_create_group(int nrank, int device_id, const std::string &ip, int port);
+
+} // namespace hctr

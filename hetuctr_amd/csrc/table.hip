@@ -1,0 +1,749 @@
+// Host orchestration of the hot path: shard construction, the fixed stage order of preprocess and push_pull,
+// the loopback exchanges between the shards of a group, introspection.
+// Reference: csrc/core/hetu_gpu_table.cu:9-65 (stage order), csrc/core/table_initialize.cu:66-211 (state),
+// csrc/core/all2all.cu:6-130 (what travels between which buffers, in which order).
+#include "table.h"
+
+#include <algorithm>
+#include <chrono>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+
+namespace hctr {
+
+static int bits_for(uint64_t max_value) { // bits needed to represent values 0..max_value
+  int b = 0;
+  while (b < 64 && (max_value >> b)) b++;
+  return b;
+}
+
+// ================================================================================================
+// Batch
+// ================================================================================================
+void Batch::reserve(uint32_t n_keys, int nrank, bool wide) {
+  const size_t n = std::max<uint32_t>(n_keys, 1);
+  keys.reserve(n * sizeof(index_t));
+  sorted_arg.reserve(n * 4);
+  rank_sorted.reserve(n * 4);
+  idx_map.reserve(n * 4);
+  ukey.reserve(n * (wide ? 8 : 4));
+  run_start.reserve((n + 1) * 4);
+  uoff.reserve(n * sizeof(slot_t));
+  bucket_lo.reserve((size_t)(nrank + 1) * 4);
+  dU.reserve(4);
+}
+
+BatchView Batch::view() const {
+  BatchView v;
+  v.n = n;
+  v.keys = keys.as<index_t>();
+  v.sorted_arg = sorted_arg.as<uint32_t>();
+  v.rank_sorted = rank_sorted.as<uint32_t>();
+  v.idx_map = idx_map.as<uint32_t>();
+  v.ukey = ukey.p;
+  v.run_start = run_start.as<uint32_t>();
+  v.uoff = uoff.as<slot_t>();
+  v.bucket_lo = bucket_lo.as<uint32_t>();
+  v.d_U = dU.as<uint32_t>();
+  return v;
+}
+
+// ================================================================================================
+// Shard
+// ================================================================================================
+Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *storage_arr, size_t n_storage,
+             unsigned seed, std::shared_ptr<Group> grp)
+    : cfg(c), ip(c.ip ? c.ip : ""), group(std::move(grp)) {
+  cfg.ip = nullptr;
+  HCTR_CHECK(c.nrank >= 1 && c.nrank <= 256, "nrank must be in 1..256 (worker ids are one byte)");
+  HCTR_CHECK(c.rank >= 0 && c.rank < c.nrank, "rank out of range");
+  HCTR_CHECK(c.length >= 1, "length must be positive");
+  HCTR_CHECK(c.width >= 1 && c.width < (1u << 24), "width out of range");
+  HCTR_CHECK(n_storage < 0x7fffffffull, "a shard holds fewer than 2^31 rows");
+  HCTR_CHECK(root_arr != nullptr && (storage_arr != nullptr || n_storage == 0), "null root_arr / storage_arr");
+  HCTR_CHECK(c.init_type >= 0 && c.init_type <= 3, "unknown initializer");
+
+  kl.id_bits = std::max(1, bits_for(c.length - 1));
+  kl.total_bits = kl.id_bits + (c.nrank > 1 ? bits_for((uint64_t)c.nrank - 1) : 0);
+  HCTR_CHECK(kl.total_bits <= 64, "length * nrank does not fit a 64-bit sort key");
+  kl.wide = kl.total_bits > 32;
+  if (const char *f = getenv("HETUCTR_FORCE_WIDE_KEYS")) // exercises the 64-bit sort-key path on small tables
+    if (f[0] == '1') kl.wide = true;
+
+  // ---- host-side checks and the resident layout: cached ids first, then owned ids, order kept
+  // (thrust::stable_partition at table_initialize.cu:81)
+  const size_t L = c.length;
+  size_t owned_total = 0;
+  for (size_t i = 0; i < L; i++) {
+    HCTR_CHECK(root_arr[i] < c.nrank, "root_arr holds an owner >= nrank");
+    owned_total += root_arr[i] == c.rank;
+  }
+  std::vector<bool> seen(L, false);
+  std::vector<index_t> ids(n_storage);
+  size_t n_cached = 0, n_own = 0;
+  for (size_t i = 0; i < n_storage; i++) {
+    const int64_t id = storage_arr[i];
+    HCTR_CHECK(id >= 0 && (uint64_t)id < L, "storage_arr holds an id outside [0, length)");
+    HCTR_CHECK(!seen[id], "storage_arr holds an id twice");
+    seen[id] = true;
+    if (root_arr[id] != c.rank) ids[n_cached++] = id;
+  }
+  size_t w = n_cached;
+  for (size_t i = 0; i < n_storage; i++)
+    if (root_arr[storage_arr[i]] == c.rank) { ids[w++] = storage_arr[i]; n_own++; }
+  // the reference only notices this when another shard queries the row (handle_query.cu:14-15)
+  HCTR_CHECK(n_own == owned_total, "storage_arr must contain every id whose owner is this rank");
+  n_owned = n_own;
+
+  HCTR_HIP(hipSetDevice(cfg.device_id));
+  hipStream_t s = group->stream;
+  const size_t S = n_storage, C = n_cached, W = c.width;
+  root.reserve(L);
+  slot.reserve(L * sizeof(slot_t));
+  store_ids.reserve(std::max<size_t>(S, 1) * sizeof(index_t));
+  emb.reserve(std::max<size_t>(S * W, 1) * sizeof(embed_t));
+  ver.reserve(std::max<size_t>(S, 1) * sizeof(version_t));
+  pend.reserve(std::max<size_t>(C * W, 1) * sizeof(embed_t));
+  upd.reserve(std::max<size_t>(C, 1) * sizeof(version_t));
+  HCTR_HIP(hipMemcpyAsync(root.p, root_arr, L, hipMemcpyHostToDevice, s));
+  if (S) HCTR_HIP(hipMemcpyAsync(store_ids.p, ids.data(), S * sizeof(index_t), hipMemcpyHostToDevice, s));
+  launch_fill_i32(s, slot.as<int32_t>(), L, kNoSlot);
+  launch_build_directory(s, store_ids.as<index_t>(), (uint32_t)S, slot.as<slot_t>());
+  launch_init_values(s, emb.as<embed_t>(), S * W, c.init_type, c.init_a, c.init_b, seed);
+  launch_fill_i64(s, ver.as<version_t>(), C, kInvalidVersion);          // table_initialize.cu:110
+  launch_fill_i64(s, ver.as<version_t>() + C, S - C, 0);                // table_initialize.cu:111
+  HCTR_HIP(hipMemsetAsync(pend.p, 0, pend.bytes, s));
+  HCTR_HIP(hipMemsetAsync(upd.p, 0, upd.bytes, s));
+
+  err.reserve(4);
+  stats.reserve(16);
+  push_total.reserve(4);
+  ret_total.reserve(4);
+  ret_seg_dev.reserve(2 * 258 * 4);
+  cnt_dev.reserve(2 * 257 * sizeof(uint64_t));
+  HCTR_HIP(hipMemsetAsync(err.p, 0, 4, s));
+  HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
+  HCTR_HIP(hipMemsetAsync(push_total.p, 0, 4, s));
+  HCTR_HIP(hipMemsetAsync(cnt_dev.p, 0, cnt_dev.bytes, s));
+  for (Batch *b : {&cur, &prev}) {
+    b->reserve(1, c.nrank, kl.wide);
+    HCTR_HIP(hipMemsetAsync(b->dU.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(b->bucket_lo.p, 0, b->bucket_lo.bytes, s));
+    HCTR_HIP(hipMemsetAsync(b->run_start.p, 0, 4, s));
+    b->send_cnt.assign(c.nrank + 1, 0);
+    b->recv_cnt.assign(c.nrank + 1, 0);
+    b->push_cnt.assign(c.nrank + 1, 0);
+    b->pushrecv_cnt.assign(c.nrank + 1, 0);
+  }
+  rq_seg.assign(c.nrank + 1, 0);
+  rg_seg.assign(c.nrank + 1, 0);
+  ret_seg.assign(c.nrank + 1, 0);
+  HCTR_HIP(hipHostMalloc((void **)&mirror, sizeof(HostMirror), hipHostMallocDefault));
+  memset(mirror, 0, sizeof(HostMirror));
+  HCTR_HIP(hipStreamSynchronize(s)); // root_arr / ids are host temporaries
+
+  tv.rank = c.rank;
+  tv.nrank = c.nrank;
+  tv.id_max = L;
+  tv.width = (uint32_t)W;
+  tv.n_stored = (uint32_t)S;
+  tv.n_cached = (uint32_t)C;
+  tv.neg_lr = -c.learning_rate;
+  tv.pull_bound = c.pull_bound;
+  tv.push_bound = c.push_bound;
+  tv.root = root.as<worker_t>();
+  tv.slot = slot.as<slot_t>();
+  tv.emb = emb.as<embed_t>();
+  tv.ver = ver.as<version_t>();
+  tv.pend = pend.as<embed_t>();
+  tv.upd = upd.as<version_t>();
+}
+
+Shard::~Shard() {
+  if (mirror) (void)hipHostFree(mirror);
+}
+
+void Shard::reserve_batch_scratch(uint32_t n) {
+  const size_t m = std::max<uint32_t>(n, 1);
+  const size_t ks = kl.wide ? 8 : 4;
+  comp.reserve(m * ks);
+  ktmp0.reserve(m * ks);
+  ktmp1.reserve(m * ks);
+  vtmp0.reserve(m * 4);
+  vtmp1.reserve(m * 4);
+  const size_t blocks = sort_blocks(m);
+  ghist.reserve(((size_t)1 << kSortMaxDigitBits) * blocks * 4);
+  bintot.reserve(((size_t)1 << kSortMaxDigitBits) * 4);
+  block_sums.reserve((blocks + 2) * 4);
+}
+
+// csrc/core/preprocess.cu:92-141
+void Shard::preprocess_index(const int64_t *keys, size_t n) {
+  HCTR_CHECK(n < 0xfffffff0ull, "a batch holds fewer than 2^32 keys");
+  HCTR_CHECK(keys != nullptr || n == 0, "null key pointer");
+  hipStream_t s = group->stream;
+  cur.n = (uint32_t)n;
+  cur.U = 0;
+  cur.reserve(cur.n, cfg.nrank, kl.wide);
+  if (n == 0) { // :93-95
+    HCTR_HIP(hipMemsetAsync(cur.dU.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(cur.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
+    HCTR_HIP(hipMemsetAsync(cur.run_start.p, 0, 4, s));
+  } else {
+    reserve_batch_scratch(cur.n);
+    HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s)); // :98-99
+    launch_make_keys(s, tv, kl, cur.keys.as<index_t>(), cur.n, comp.p, err.as<uint32_t>());
+    SortScratch sc;
+    sc.ghist = ghist.as<uint32_t>();
+    sc.bintot = bintot.as<uint32_t>();
+    sc.blocks_cap = sort_blocks(cur.n);
+    const void *sorted_keys = nullptr;
+    if (kl.wide) {
+      const uint64_t *sk;
+      radix_sort_positions<uint64_t>(s, comp.as<uint64_t>(), cur.n, kl.total_bits, ktmp0.as<uint64_t>(),
+                                     ktmp1.as<uint64_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
+                                     cur.sorted_arg.as<uint32_t>(), sc, &sk);
+      sorted_keys = sk;
+    } else {
+      const uint32_t *sk;
+      radix_sort_positions<uint32_t>(s, comp.as<uint32_t>(), cur.n, kl.total_bits, ktmp0.as<uint32_t>(),
+                                     ktmp1.as<uint32_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
+                                     cur.sorted_arg.as<uint32_t>(), sc, &sk);
+      sorted_keys = sk;
+    }
+    launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>());
+  }
+  launch_bucket_sizes(s, cur.view(), cfg.nrank, cnt_dev.as<uint64_t>());
+}
+
+// csrc/core/preprocess.cu:148-182
+void Shard::preprocess_gradient() {
+  hipStream_t s = group->stream;
+  uint64_t *cnt = cnt_dev.as<uint64_t>() + 257;
+  if (cfg.nrank == 1 || prev.n == 0) { // single shard: every key is owned, nothing is ever pushed
+    HCTR_HIP(hipMemsetAsync(cnt, 0, (size_t)(cfg.nrank + 1) * sizeof(uint64_t), s));
+    HCTR_HIP(hipMemsetAsync(push_total.p, 0, 4, s));
+    return;
+  }
+  need.reserve((size_t)prev.n * 4);
+  prefix.reserve((size_t)prev.n * 4);
+  reserve_batch_scratch(prev.n);
+  launch_decide_update(s, tv, kl, prev.view(), need.as<uint32_t>());
+  launch_exclusive_scan(s, need.as<uint32_t>(), prefix.as<uint32_t>(), prev.n, prev.dU.as<uint32_t>(),
+                        block_sums.as<uint32_t>(), push_total.as<uint32_t>());
+  launch_bucket_counts(s, prev.view(), prefix.as<uint32_t>(), push_total.as<uint32_t>(), cfg.nrank, cnt);
+}
+
+void Shard::enqueue_readback_preprocess() {
+  hipStream_t s = group->stream;
+  const size_t r1 = (size_t)(cfg.nrank + 1) * sizeof(uint64_t);
+  HCTR_HIP(hipMemcpyAsync(&mirror->U, cur.dU.p, 4, hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipMemcpyAsync(&mirror->err, err.p, 4, hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipMemcpyAsync(&mirror->push_total, push_total.p, 4, hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipMemcpyAsync(mirror->send_cnt, cnt_dev.p, r1, hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipMemcpyAsync(mirror->push_cnt, cnt_dev.as<uint64_t>() + 257, r1, hipMemcpyDeviceToHost, s));
+}
+
+void Shard::finish_preprocess() {
+  cur.U = mirror->U;
+  prev_active = prev.n > 0;
+  for (int i = 0; i <= cfg.nrank; i++) {
+    cur.send_cnt[i] = mirror->send_cnt[i];
+    prev.push_cnt[i] = mirror->push_cnt[i];
+  }
+  if (mirror->err) {
+    HCTR_HIP(hipMemsetAsync(err.p, 0, 4, group->stream));
+    HCTR_CHECK(!(mirror->err & 1u), "preprocess: a key lies outside [0, length) (it was treated as id 0)");
+  }
+}
+
+// csrc/core/generate_query.cu:85-89; inference rule of csrc/core/hetu_gpu_table.cu:14-21
+void Shard::generate_gradient(const float *grad) {
+  hipStream_t s = group->stream;
+  if (grad == nullptr) {
+    prev.n = 0;
+    prev.U = 0;
+    HCTR_HIP(hipMemsetAsync(prev.dU.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(prev.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
+    std::fill(prev.push_cnt.begin(), prev.push_cnt.end(), 0);
+    std::fill(prev.pushrecv_cnt.begin(), prev.pushrecv_cnt.end(), 0);
+  }
+  prev_active = prev.n > 0;
+  last_stats[3] = 0;
+  if (!prev_active) return;
+  uint64_t pushes = 0;
+  for (int i = 0; i < cfg.nrank; i++) pushes += prev.push_cnt[i];
+  last_stats[3] = (long long)pushes;
+  const size_t W = cfg.width;
+  PushArgs a;
+  a.grad = grad;
+  a.need = nullptr;
+  a.prefix = nullptr;
+  a.g_idx = nullptr;
+  a.g_cnt = nullptr;
+  a.g_val = nullptr;
+  if (cfg.nrank > 1) {
+    g_idx.reserve(std::max<uint64_t>(pushes, 1) * sizeof(index_t));
+    g_cnt.reserve(std::max<uint64_t>(pushes, 1) * sizeof(version_t));
+    g_val.reserve(std::max<uint64_t>(pushes, 1) * W * sizeof(embed_t));
+    a.need = need.as<uint32_t>();
+    a.prefix = prefix.as<uint32_t>();
+    a.g_idx = g_idx.as<index_t>();
+    a.g_cnt = g_cnt.as<version_t>();
+    a.g_val = g_val.as<embed_t>();
+  }
+  launch_push(s, tv, kl, prev.view(), a);
+}
+
+// csrc/core/generate_query.cu:91-106
+void Shard::generate_query() {
+  if (cfg.nrank == 1) return; // a shard never finds its own rows outdated (handle_query.cu:47-54)
+  hipStream_t s = group->stream;
+  q_idx.reserve(std::max<uint32_t>(cur.U, 1) * sizeof(index_t));
+  q_ver.reserve(std::max<uint32_t>(cur.U, 1) * sizeof(version_t));
+  launch_lookup_version(s, tv, cur.view(), q_ver.as<version_t>());
+  launch_unique_ids(s, kl, cur.view(), q_idx.as<index_t>());
+}
+
+// csrc/core/handle_query.cu:106-116: one source after the other, in rank order
+void Shard::handle_gradient() {
+  hipStream_t s = group->stream;
+  last_stats[5] = (long long)rg_seg[cfg.nrank];
+  for (int src = 0; src < cfg.nrank; src++)
+    launch_apply_remote(s, tv, rg_idx.as<index_t>(), rg_cnt.as<version_t>(), rg_val.as<embed_t>(),
+                        (uint32_t)rg_seg[src], (uint32_t)rg_seg[src + 1], err.as<uint32_t>());
+}
+
+__global__ void segment_bounds(const uint32_t *__restrict__ out_pos, const uint32_t *__restrict__ total,
+                               const uint32_t *__restrict__ seg, int nseg, uint32_t q, uint32_t *__restrict__ out) {
+  const int i = threadIdx.x;
+  if (i > nseg) return;
+  const uint32_t k = seg[i];
+  out[i] = k >= q ? *total : out_pos[k];
+}
+
+// csrc/core/handle_query.cu:42-78
+void Shard::handle_query() {
+  hipStream_t s = group->stream;
+  const int R = cfg.nrank;
+  const uint32_t Q = (uint32_t)rq_seg[R];
+  outdated.reserve(std::max<uint32_t>(Q, 1) * 4);
+  out_pos.reserve(std::max<uint32_t>(Q, 1) * 4);
+  ret_ver.reserve(std::max<uint32_t>(Q, 1) * sizeof(version_t));
+  ret_val.reserve((size_t)std::max<uint32_t>(Q, 1) * cfg.width * sizeof(embed_t));
+  reserve_batch_scratch(Q);
+  launch_decide_outdated(s, tv, rq_idx.as<index_t>(), rq_ver.as<version_t>(), Q, (uint32_t)rq_seg[cfg.rank],
+                         (uint32_t)rq_seg[cfg.rank + 1], outdated.as<uint32_t>(), err.as<uint32_t>());
+  launch_exclusive_scan(s, outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q, nullptr, block_sums.as<uint32_t>(),
+                        ret_total.as<uint32_t>());
+  launch_pack_rows(s, tv, rq_idx.as<index_t>(), outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q,
+                   ret_ver.as<version_t>(), ret_val.as<embed_t>());
+  // rows to return per requester: positions of the segment starts in the compacted order
+  uint32_t *seg_h = mirror->ret_seg; // staged through the pinned mirror, overwritten by the result below
+  for (int i = 0; i <= R; i++) seg_h[i] = (uint32_t)rq_seg[i];
+  uint32_t *seg_d = ret_seg_dev.as<uint32_t>();
+  HCTR_HIP(hipMemcpyAsync(seg_d, seg_h, (size_t)(R + 1) * 4, hipMemcpyHostToDevice, s));
+  hipLaunchKernelGGL(segment_bounds, dim3(1), dim3(R + 1), 0, s, out_pos.as<uint32_t>(), ret_total.as<uint32_t>(),
+                     seg_d, R, Q, seg_d + 258);
+  HCTR_HIP(hipGetLastError());
+  HCTR_HIP(hipMemcpyAsync(seg_h, seg_d + 258, (size_t)(R + 1) * 4, hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipMemcpyAsync(&mirror->err, err.p, 4, hipMemcpyDeviceToHost, s));
+}
+
+void Shard::finish_handle_query() {
+  for (int i = 0; i <= cfg.nrank; i++) ret_seg[i] = mirror->ret_seg[i];
+  last_stats[4] = (long long)ret_seg[cfg.nrank];
+  if (mirror->err) {
+    const uint32_t e = mirror->err;
+    HCTR_HIP(hipMemsetAsync(err.p, 0, 4, group->stream));
+    HCTR_CHECK(!(e & 2u), "a pushed row reached a shard that does not own it");
+    HCTR_CHECK(!(e & 4u), "a queried row reached a shard that does not own it");
+  }
+}
+
+// csrc/core/writeback.cu:43-56
+void Shard::write_back(float *dst) {
+  hipStream_t s = group->stream;
+  PullArgs a;
+  a.got = nullptr;
+  a.ret_i = nullptr;
+  a.in_ver = nullptr;
+  a.in_val = nullptr;
+  a.dst = dst;
+  if (cfg.nrank > 1) {
+    ret_i.reserve(std::max<uint32_t>(cur.U, 1) * 4);
+    reserve_batch_scratch(cur.U);
+    HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
+    launch_exclusive_scan(s, got.as<uint32_t>(), ret_i.as<uint32_t>(), cur.U, nullptr, block_sums.as<uint32_t>(),
+                          nullptr);
+    a.got = got.as<uint32_t>();
+    a.ret_i = ret_i.as<uint32_t>();
+    a.in_ver = in_ver.as<version_t>();
+    a.in_val = in_val.as<embed_t>();
+    launch_refresh(s, tv, cur.view(), a, stats.as<uint32_t>());
+    HCTR_HIP(hipMemcpyAsync(mirror->stats, stats.p, 16, hipMemcpyDeviceToHost, s));
+  }
+  if (dst != nullptr) launch_gather(s, tv, cur.view(), a);
+}
+
+void Shard::finish_push_pull() {
+  if (cfg.nrank > 1) {
+    last_stats[0] = mirror->stats[0];
+    last_stats[1] = mirror->stats[1];
+    last_stats[2] = mirror->stats[2];
+    HCTR_CHECK(!(mirror->stats[3] & 8u), "an owned row came back as outdated");
+  }
+}
+
+// ---- introspection -------------------------------------------------------------------------------
+namespace {
+template <typename T> std::vector<T> download(const void *dev, size_t n) {
+  std::vector<T> h(n);
+  if (n) HCTR_HIP(hipMemcpy(h.data(), dev, n * sizeof(T), hipMemcpyDeviceToHost));
+  return h;
+}
+template <typename V> size_t put64(const V &v, size_t n, void *out, size_t cap) {
+  long long *o = (long long *)out;
+  for (size_t i = 0; i < n && i < cap; i++) o[i] = (long long)v[i];
+  return n;
+}
+} // namespace
+
+size_t Shard::fetch(int which, void *out, size_t cap) {
+  HCTR_HIP(hipSetDevice(cfg.device_id));
+  HCTR_HIP(hipStreamSynchronize(group->stream));
+  const int R = cfg.nrank;
+  const uint64_t id_mask = kl.id_bits >= 64 ? ~0ull : (((uint64_t)1 << kl.id_bits) - 1);
+  auto ukeys = [&](const Batch &b) {
+    std::vector<uint64_t> k(b.U);
+    if (kl.wide) {
+      auto h = download<uint64_t>(b.ukey.p, b.U);
+      for (size_t i = 0; i < b.U; i++) k[i] = h[i];
+    } else {
+      auto h = download<uint32_t>(b.ukey.p, b.U);
+      for (size_t i = 0; i < b.U; i++) k[i] = h[i];
+    }
+    return k;
+  };
+  switch (which) {
+    case HCTR_F_UNIQUE: { auto k = ukeys(cur); for (auto &x : k) x &= id_mask; return put64(k, cur.U, out, cap); }
+    case HCTR_F_ROOT: { auto k = ukeys(cur); for (auto &x : k) x >>= kl.id_bits; return put64(k, cur.U, out, cap); }
+    case HCTR_F_SORTED_ARG: return put64(download<uint32_t>(cur.sorted_arg.p, cur.n), cur.n, out, cap);
+    case HCTR_F_RUN_START: return put64(download<uint32_t>(cur.run_start.p, (size_t)cur.U + 1), (size_t)cur.U + 1, out, cap);
+    case HCTR_F_IDX_MAP: return put64(download<uint32_t>(cur.idx_map.p, cur.n), cur.n, out, cap);
+    case HCTR_F_OFFSET: return put64(download<slot_t>(cur.uoff.p, cur.U), cur.U, out, cap);
+    case HCTR_F_SEND_CNT: return put64(cur.send_cnt, R, out, cap);
+    case HCTR_F_RECV_CNT: return put64(cur.recv_cnt, R, out, cap);
+    case HCTR_F_NEED_UPDATE:
+    case HCTR_F_UPDATE_PREFIX: {
+      if (R == 1 || prev.U == 0) { std::vector<long long> z(prev.U, 0); return put64(z, prev.U, out, cap); }
+      return put64(download<uint32_t>(which == HCTR_F_NEED_UPDATE ? need.p : prefix.p, prev.U), prev.U, out, cap);
+    }
+    case HCTR_F_PUSH_CNT: return put64(prev.push_cnt, R, out, cap);
+    case HCTR_F_PUSHRECV_CNT: return put64(prev.pushrecv_cnt, R, out, cap);
+    case HCTR_F_OUTDATED: {
+      if (R == 1) { std::vector<long long> z(cur.U, 0); return put64(z, cur.U, out, cap); }
+      return put64(download<uint32_t>(outdated.p, rq_seg[R]), rq_seg[R], out, cap);
+    }
+    case HCTR_F_GOT: {
+      if (R == 1) { std::vector<long long> z(cur.U, 0); return put64(z, cur.U, out, cap); }
+      return put64(download<uint32_t>(got.p, cur.U), cur.U, out, cap);
+    }
+    case HCTR_F_VERSION: return put64(download<version_t>(ver.p, tv.n_stored), tv.n_stored, out, cap);
+    case HCTR_F_UPDATES: return put64(download<version_t>(upd.p, tv.n_cached), tv.n_cached, out, cap);
+    case HCTR_F_STORE_IDS: return put64(download<index_t>(store_ids.p, tv.n_stored), tv.n_stored, out, cap);
+    case HCTR_F_KEYS: return put64(download<index_t>(cur.keys.p, cur.n), cur.n, out, cap);
+    case HCTR_F_EMBEDDING:
+    case HCTR_F_PENDING: {
+      const size_t n = (size_t)(which == HCTR_F_EMBEDDING ? tv.n_stored : tv.n_cached) * tv.width;
+      const void *src = which == HCTR_F_EMBEDDING ? emb.p : pend.p;
+      if (std::min(n, cap)) HCTR_HIP(hipMemcpy(out, src, std::min(n, cap) * sizeof(embed_t), hipMemcpyDeviceToHost));
+      return n;
+    }
+    case HCTR_F_STATS: return put64(last_stats, 6, out, cap);
+    case HCTR_F_SIZES: {
+      long long z[6] = {(long long)cur.n, (long long)cur.U, (long long)prev.n, (long long)prev.U,
+                        (long long)tv.n_stored, (long long)tv.n_cached};
+      return put64(z, 6, out, cap);
+    }
+  }
+  throw Error("hetuCTR: unknown item for debug_fetch");
+}
+
+// ================================================================================================
+// Group
+// ================================================================================================
+Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(std::move(k)), members(nr, nullptr) {
+  int ndev = 0;
+  HCTR_HIP(hipGetDeviceCount(&ndev));
+  HCTR_CHECK(dev >= 0 && dev < ndev, "InCorrect device number."); // table_initialize.cu:144-146
+  HCTR_HIP(hipSetDevice(dev));
+  // a blocking stream, like the reference's cudaStreamCreate (table_initialize.cu:16): work the caller queued on the
+  // legacy default stream (torch's default) is ordered before ours without an explicit synchronisation
+  HCTR_HIP(hipStreamCreate(&stream));
+  HCTR_HIP(hipEventCreate(&ev0));
+  HCTR_HIP(hipEventCreate(&ev1));
+  a_keys_.resize(nr);
+  a_n_.resize(nr);
+  a_grad_.resize(nr);
+  a_dst_.resize(nr);
+  if (const char *w = getenv("HETUCTR_GROUP_WAIT_SECONDS")) wait_seconds = atof(w);
+}
+
+Group::~Group() {
+  if (desc_host) (void)hipHostFree(desc_host);
+  if (ev0) (void)hipEventDestroy(ev0);
+  if (ev1) (void)hipEventDestroy(ev1);
+  if (stream) (void)hipStreamDestroy(stream);
+}
+
+void Group::join(Shard *s) {
+  std::lock_guard<std::mutex> lk(mu_);
+  HCTR_CHECK(members[s->cfg.rank] == nullptr, "this rank already exists in the group named by (ip, port)");
+  members[s->cfg.rank] = s;
+}
+
+void Group::leave(Shard *s) {
+  std::lock_guard<std::mutex> lk(mu_);
+  if (members[s->cfg.rank] == s) members[s->cfg.rank] = nullptr;
+}
+
+bool Group::complete() const {
+  for (Shard *m : members)
+    if (!m) return false;
+  return true;
+}
+
+void Group::run_copies(std::vector<CopyDesc> &descs) {
+  if (descs.empty()) return;
+  if (descs.size() > desc_cap) {
+    if (desc_host) HCTR_HIP(hipHostFree(desc_host));
+    desc_host = nullptr;
+    desc_cap = descs.size() * 2;
+    HCTR_HIP(hipHostMalloc((void **)&desc_host, desc_cap * sizeof(CopyDesc), hipHostMallocDefault));
+  }
+  desc_dev.reserve(desc_cap * sizeof(CopyDesc));
+  memcpy(desc_host, descs.data(), descs.size() * sizeof(CopyDesc));
+  HCTR_HIP(hipMemcpyAsync(desc_dev.p, desc_host, descs.size() * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
+  size_t max_bytes = 0;
+  for (auto &d : descs) max_bytes = std::max(max_bytes, d.bytes);
+  for (size_t lo = 0; lo < descs.size(); lo += 32768)
+    launch_copies(stream, desc_dev.as<CopyDesc>() + lo, (uint32_t)std::min<size_t>(32768, descs.size() - lo), max_bytes);
+  descs.clear();
+}
+
+// csrc/core/all2all.cu:18-87: every receive buffer is the senders' buckets for this shard, in source order
+void Group::exchange_query() {
+  const int R = nrank;
+  std::vector<CopyDesc> descs;
+  for (int d = 0; d < R; d++) {
+    Shard &dst = *members[d];
+    const size_t W = dst.cfg.width;
+    uint64_t Q = 0, G = 0;
+    for (int s = 0; s < R; s++) {
+      Shard &src = *members[s];
+      dst.rq_seg[s] = Q;
+      dst.rg_seg[s] = G;
+      Q += src.cur.send_cnt[d];
+      if (src.prev_active) G += src.prev.push_cnt[d];
+    }
+    dst.rq_seg[R] = Q;
+    dst.rg_seg[R] = G;
+    HCTR_CHECK(Q < 0xfffffff0ull && G < 0xfffffff0ull, "more than 2^32 rows arrive at one shard");
+    dst.rq_idx.reserve(std::max<uint64_t>(Q, 1) * sizeof(index_t));
+    dst.rq_ver.reserve(std::max<uint64_t>(Q, 1) * sizeof(version_t));
+    dst.rg_idx.reserve(std::max<uint64_t>(G, 1) * sizeof(index_t));
+    dst.rg_cnt.reserve(std::max<uint64_t>(G, 1) * sizeof(version_t));
+    dst.rg_val.reserve(std::max<uint64_t>(G, 1) * W * sizeof(embed_t));
+    for (int s = 0; s < R; s++) {
+      Shard &src = *members[s];
+      uint64_t qlo = 0, glo = 0;
+      for (int i = 0; i < d; i++) {
+        qlo += src.cur.send_cnt[i];
+        glo += src.prev.push_cnt[i];
+      }
+      const uint64_t qn = src.cur.send_cnt[d];
+      if (qn) {
+        descs.push_back({src.q_idx.as<index_t>() + qlo, dst.rq_idx.as<index_t>() + dst.rq_seg[s], qn * sizeof(index_t)});
+        descs.push_back({src.q_ver.as<version_t>() + qlo, dst.rq_ver.as<version_t>() + dst.rq_seg[s], qn * sizeof(version_t)});
+      }
+      const uint64_t gn = src.prev_active ? src.prev.push_cnt[d] : 0;
+      if (gn) {
+        descs.push_back({src.g_idx.as<index_t>() + glo, dst.rg_idx.as<index_t>() + dst.rg_seg[s], gn * sizeof(index_t)});
+        descs.push_back({src.g_cnt.as<version_t>() + glo, dst.rg_cnt.as<version_t>() + dst.rg_seg[s], gn * sizeof(version_t)});
+        descs.push_back({src.g_val.as<embed_t>() + glo * W, dst.rg_val.as<embed_t>() + dst.rg_seg[s] * W, gn * W * sizeof(embed_t)});
+      }
+    }
+  }
+  run_copies(descs);
+}
+
+// csrc/core/all2all.cu:89-130: flags go back to the requesters, then versions and rows of the flagged queries
+void Group::exchange_return() {
+  const int R = nrank;
+  std::vector<CopyDesc> descs;
+  for (int s = 0; s < R; s++) { // requester
+    Shard &req = *members[s];
+    const size_t W = req.cfg.width;
+    uint64_t rows = 0;
+    for (int d = 0; d < R; d++) rows += members[d]->ret_seg[s + 1] - members[d]->ret_seg[s];
+    req.in_rows = rows;
+    req.got.reserve(std::max<uint32_t>(req.cur.U, 1) * 4);
+    req.in_ver.reserve(std::max<uint64_t>(rows, 1) * sizeof(version_t));
+    req.in_val.reserve(std::max<uint64_t>(rows, 1) * W * sizeof(embed_t));
+    uint64_t uoff = 0, roff = 0;
+    for (int d = 0; d < R; d++) { // owner, in rank order
+      Shard &own = *members[d];
+      const uint64_t qn = own.rq_seg[s + 1] - own.rq_seg[s];
+      if (qn) descs.push_back({own.outdated.as<uint32_t>() + own.rq_seg[s], req.got.as<uint32_t>() + uoff, qn * 4});
+      const uint64_t rn = own.ret_seg[s + 1] - own.ret_seg[s];
+      if (rn) {
+        descs.push_back({own.ret_ver.as<version_t>() + own.ret_seg[s], req.in_ver.as<version_t>() + roff, rn * sizeof(version_t)});
+        descs.push_back({own.ret_val.as<embed_t>() + own.ret_seg[s] * W, req.in_val.as<embed_t>() + roff * W, rn * W * sizeof(embed_t)});
+      }
+      uoff += qn;
+      roff += rn;
+    }
+    HCTR_CHECK(uoff == req.cur.U, "internal: returned flags do not cover the unique keys");
+  }
+  run_copies(descs);
+}
+
+// csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
+void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
+  HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
+  HCTR_HIP(hipSetDevice(device_id));
+  HCTR_HIP(hipEventRecord(ev0, stream));
+  for (Shard *m : members) {
+    m->swap_batches();
+    m->preprocess_index(keys[m->cfg.rank], n[m->cfg.rank]);
+    m->preprocess_gradient();
+    m->enqueue_readback_preprocess();
+  }
+  HCTR_HIP(hipEventRecord(ev1, stream));
+  HCTR_HIP(hipStreamSynchronize(stream));
+  float ms = 0.f;
+  HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+  std::string first_error;
+  for (Shard *m : members) {
+    m->last_pre_ms = ms;
+    try {
+      m->finish_preprocess();
+    } catch (const Error &e) {
+      if (first_error.empty()) first_error = e.what();
+    }
+  }
+  // all2allExchangeShape, csrc/core/all2all.cu:6-16
+  for (Shard *m : members)
+    for (int s = 0; s < nrank; s++) {
+      m->cur.recv_cnt[s] = members[s]->cur.send_cnt[m->cfg.rank];
+      m->prev.pushrecv_cnt[s] = members[s]->prev.push_cnt[m->cfg.rank];
+    }
+  if (!first_error.empty()) throw Error(first_error);
+}
+
+// csrc/core/hetu_gpu_table.cu:9-41 for every shard of the group
+void Group::push_pull_all(const float *const *grads, float *const *dsts) {
+  HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
+  HCTR_HIP(hipSetDevice(device_id));
+  HCTR_HIP(hipEventRecord(ev0, stream));
+  for (Shard *m : members) {
+    m->generate_gradient(grads[m->cfg.rank]);
+    m->generate_query();
+  }
+  if (nrank > 1) {
+    exchange_query();
+    for (Shard *m : members) m->handle_gradient();
+    for (Shard *m : members) m->handle_query();
+    HCTR_HIP(hipStreamSynchronize(stream)); // hetu_gpu_table.cu:33: the return counts size the next exchange
+    for (Shard *m : members) m->finish_handle_query();
+    exchange_return();
+  }
+  for (Shard *m : members) m->write_back(dsts[m->cfg.rank]);
+  HCTR_HIP(hipEventRecord(ev1, stream));
+  HCTR_HIP(hipStreamSynchronize(stream));
+  float ms = 0.f;
+  HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+  for (Shard *m : members) {
+    m->last_pp_ms = ms;
+    m->finish_push_pull();
+  }
+}
+
+// Rendezvous of the nrank per-shard callers: the last one to arrive runs the step for all.
+template <typename F> void Group::collective(int rank, int op, F &&run_all) {
+  std::unique_lock<std::mutex> lk(mu_);
+  if (arrived_ > 0 && pending_op_ != op)
+    throw Error("hetuCTR: shards of one group are in different calls (preprocess vs push_pull)");
+  pending_op_ = op;
+  arrived_++;
+  if (arrived_ == nrank) {
+    failure_.clear();
+    try {
+      run_all();
+    } catch (const std::exception &e) {
+      failure_ = e.what();
+    }
+    arrived_ = 0;
+    generation_++;
+    cv_.notify_all();
+  } else {
+    const uint64_t gen = generation_;
+    const bool ok = cv_.wait_for(lk, std::chrono::duration<double>(wait_seconds), [&] { return generation_ != gen; });
+    if (!ok) {
+      arrived_--;
+      throw Error("hetuCTR: timed out waiting for the other shards of the group to make the same call");
+    }
+  }
+  if (!failure_.empty()) throw Error(failure_);
+}
+
+void Group::preprocess_one(int rank, const int64_t *keys, size_t n) {
+  if (nrank == 1) {
+    preprocess_all(&keys, &n);
+    return;
+  }
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    a_keys_[rank] = keys;
+    a_n_[rank] = n;
+  }
+  collective(rank, 1, [&] { preprocess_all(a_keys_.data(), a_n_.data()); });
+}
+
+void Group::push_pull_one(int rank, const float *grad, float *dst) {
+  if (nrank == 1) {
+    push_pull_all(&grad, &dst);
+    return;
+  }
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    a_grad_[rank] = grad;
+    a_dst_[rank] = dst;
+  }
+  collective(rank, 2, [&] { push_pull_all(a_grad_.data(), a_dst_.data()); });
+}
+
+// ---- registry of groups by (ip, port) --------------------------------------------------------------
+static std::mutex g_registry_mu;
+static std::map<std::string, std::weak_ptr<Group>> g_registry;
+
+std::shared_ptr<Group> find_or_create_group(int nrank, int device_id, const std::string &ip, int port) {
+  if (nrank == 1) return std::make_shared<Group>(1, device_id, "");
+  const std::string key = ip + ":" + std::to_string(port);
+  std::lock_guard<std::mutex> lk(g_registry_mu);
+  auto it = g_registry.find(key);
+  if (it != g_registry.end()) {
+    if (auto g = it->second.lock()) {
+      HCTR_CHECK(g->nrank == nrank, "a group with this (ip, port) exists with a different nrank");
+      HCTR_CHECK(g->device_id == device_id, "all shards of a loopback group live on one device");
+      return g;
+    }
+  }
+  auto g = std::make_shared<Group>(nrank, device_id, key);
+  g_registry[key] = g;
+  return g;
+}
+
+} // namespace hctr

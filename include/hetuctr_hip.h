@@ -1,0 +1,111 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of HetuCTR's per-GPU embedding hot path.
+ *
+ * This is the boundary a binding of the reference's table API sits on: plain pointers and sizes,
+ * an opaque handle, an int status (0 = ok) and a per-thread error string.  No torch, pybind or C++
+ * types cross it.  The python module `hetuCTR` (same surface as the reference's
+ * csrc/pybind/pybind.cu:42-79) is a thin pybind11 layer over exactly these entry points.
+ *
+ * Citations are relative to the reference tree.
+ */
+#ifndef HETUCTR_HIP_H_
+#define HETUCTR_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct hctr_table hctr_table;
+
+/* hetuCTR::InitType, csrc/utils/initializer.h:8-14 (same numeric order) */
+enum { HCTR_INIT_ZERO = 0, HCTR_INIT_NORMAL = 1, HCTR_INIT_UNIFORM = 2, HCTR_INIT_TRUNCATED_NORMAL = 3 };
+
+/* Constructor arguments of hetuCTR::HetuTable, csrc/core/hetu_gpu_table.h:109-124 /
+ * csrc/pybind/pybind.cu:63-69, in the same order. */
+typedef struct hctr_config {
+  int rank;            /* this shard's rank, 0 <= rank < nrank */
+  int nrank;           /* number of shards, <= 256 (worker ids are one byte, csrc/core/types.h:28) */
+  int device_id;       /* HIP device ordinal */
+  const char *ip;      /* with nrank > 1: (ip, port) names the in-process loopback group the table joins */
+  int port;            /*   (the reference uses them for its NCCL rendezvous, table_initialize.cu:14-31) */
+  size_t length;       /* kEmbeddingIDMax: ids are 0 .. length-1 */
+  size_t width;        /* kEmbeddingWidth: floats per row */
+  long long pull_bound;
+  long long push_bound;
+  int init_type;       /* HCTR_INIT_* */
+  float init_a;        /* mean, or lower bound */
+  float init_b;        /* stddev, or upper bound */
+  float learning_rate;
+  int verbose;
+} hctr_config;
+
+/* Replaces HetuTable::HetuTable + initializeTable + initialize
+ * (csrc/core/table_initialize.cu:66-164, csrc/utils/initializer.cu:94-103).
+ * root_arr: `length` owner bytes; storage_arr: the ids resident on this shard (owned and cached),
+ * both HOST pointers read only during the call.  Every id owned by `rank` must be in storage_arr. */
+int hctr_create(const hctr_config *cfg, const uint8_t *root_arr, const int64_t *storage_arr, size_t n_storage,
+                hctr_table **out);
+
+/* Replaces HetuTable::~HetuTable (csrc/core/table_initialize.cu:231-245). */
+int hctr_destroy(hctr_table *t);
+
+/* Replaces HetuTable::preprocess (csrc/core/hetu_gpu_table.cu:43-65): the previous batch becomes the
+ * one whose gradients come next, `keys` (int64[n], HOST OR DEVICE memory) becomes the current batch.
+ * Synchronous.  With nrank > 1 the call completes when every shard of the group has made it. */
+int hctr_preprocess(hctr_table *t, const int64_t *keys, size_t n);
+
+/* Replaces HetuTable::pushPull (csrc/core/hetu_gpu_table.cu:9-41).  grad: DEVICE float[n_prev][width]
+ * for the batch before the current one, or NULL (inference: nothing is pushed).  dst: DEVICE
+ * float[n][width] receives the rows of the current batch.  Synchronous. */
+int hctr_push_pull(hctr_table *t, const float *grad, float *dst);
+
+/* Single-caller forms of the two calls above for a whole loopback group: entry r of each array belongs
+ * to tables[r], which must be rank r of one complete group.  What R reference processes do in
+ * lock-step with NCCL between the stages (csrc/core/all2all.cu:6-130) happens inside one call. */
+int hctr_group_preprocess(hctr_table *const *tables, int nrank, const int64_t *const *keys, const size_t *n);
+int hctr_group_push_pull(hctr_table *const *tables, int nrank, const float *const *grads, float *const *dsts);
+
+/* Replaces the module function hetuCTR.seed (csrc/pybind/pybind.cu:77): seed of tables created later. */
+void hctr_seed(unsigned long seed);
+
+/* Replace HetuTable::debugString / debugStringFull (csrc/core/debug.cu:5-24).  Return the length
+ * the full string needs (excluding the terminator); write at most cap bytes including it. */
+int hctr_repr(hctr_table *t, char *buf, size_t cap);
+int hctr_debug(hctr_table *t, char *buf, size_t cap);
+
+/* Message of the last failed call on this thread (the reference prints and exits instead,
+ * csrc/common/helper_cuda.h:586-599). */
+const char *hctr_last_error(void);
+
+/* Introspection of the integer intermediates and of the table state; the reference exposes none
+ * (csrc/pybind/pybind.cu:62-75) although they are what its kernels compute
+ * (csrc/core/preprocess_struct.h:7-24, csrc/core/hetu_gpu_table.h:38-70).  `which` is HCTR_F_*;
+ * *n_elems receives the element count; at most cap_elems elements are written to host_out.
+ * Integer items are int64, HCTR_F_EMBEDDING and HCTR_F_PENDING are float. */
+enum {
+  HCTR_F_UNIQUE = 0, HCTR_F_SORTED_ARG = 1, HCTR_F_RUN_START = 2, HCTR_F_IDX_MAP = 3, HCTR_F_ROOT = 4,
+  HCTR_F_OFFSET = 5, HCTR_F_SEND_CNT = 6, HCTR_F_RECV_CNT = 7, HCTR_F_NEED_UPDATE = 8, HCTR_F_UPDATE_PREFIX = 9,
+  HCTR_F_PUSH_CNT = 10, HCTR_F_PUSHRECV_CNT = 11, HCTR_F_OUTDATED = 12, HCTR_F_GOT = 13, HCTR_F_VERSION = 14,
+  HCTR_F_UPDATES = 15, HCTR_F_EMBEDDING = 16, HCTR_F_PENDING = 17, HCTR_F_STORE_IDS = 18, HCTR_F_STATS = 19,
+  HCTR_F_SIZES = 20, HCTR_F_KEYS = 21
+};
+int hctr_debug_fetch(hctr_table *t, int which, void *host_out, size_t cap_elems, size_t *n_elems);
+
+/* The HIP stream (hipStream_t) every kernel of this table's group is launched on, for callers that time
+ * or order work against it (the reference's stream_main_, csrc/core/hetu_gpu_table.h:40). */
+int hctr_stream(hctr_table *t, void **stream_out);
+
+/* Device time of the last preprocess and push_pull calls in milliseconds, measured with HIP events on
+ * that stream around the launched work (host-side waits excluded). */
+int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
+
+/* Version string of the library. */
+const char *hctr_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HETUCTR_HIP_H_ */

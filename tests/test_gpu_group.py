@@ -1,0 +1,172 @@
+"""Several shards on one GPU behind the in-process loopback: the reference's multi-GPU tests
+(tests/test_update.py, tests/check.py) with their closed forms, plus step-by-step parity with the oracle
+including cache hit / miss / refresh decisions and bounded staleness."""
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+from hetuctr_amd import capi
+from tests.gpu_util import Pair, INT_ITEMS_PRE, INT_ITEMS_POST, assert_close
+from tests.helpers import zipf_sampler
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def update_pair(nrank, length, width, bounds=(0, 0), init=("Zero", 0.0, 0.0), lr=-1.0, cache="lower", seed=0):
+    rs = np.random.RandomState(seed)
+    root = rs.randint(nrank, size=length).astype(np.uint8)
+    if cache == "lower":      # tests/test_update.py:21
+        storage = [np.where(root <= r)[0].astype(np.int64) for r in range(nrank)]
+    elif cache == "none":     # tests/check.py:30
+        storage = [np.where(root == r)[0].astype(np.int64) for r in range(nrank)]
+    else:                     # a random third of the remote rows, shuffled
+        storage = []
+        for r in range(nrank):
+            own, other = np.where(root == r)[0], np.where(root != r)[0]
+            st = np.concatenate([own, rs.choice(other, other.shape[0] // 3, replace=False)])
+            rs.shuffle(st)
+            storage.append(st.astype(np.int64))
+    return Pair(nrank, length, width, root, storage, init=init, lr=lr, bounds=bounds, seed=seed), root
+
+
+@pytest.mark.parametrize("nrank", [2, 4])
+def test_occurrence_count_closed_form(nrank):
+    say("test_update::test_one nrank", nrank)
+    length, width, bs = 1024, 128, 1024
+    p, root = update_pair(nrank, length, width)
+    rngs = [np.random.RandomState(r) for r in range(nrank)]
+    store = np.zeros(length)
+    p.preprocess([np.zeros(0, np.int64)] * nrank)
+    prev = [np.zeros(0, np.int64)] * nrank
+    for step in range(50):
+        for r in range(nrank):
+            np.add.at(store, prev[r], 1.0)
+        keys = [rngs[r].randint(length, size=bs).astype(np.int64) for r in range(nrank)]
+        p.preprocess(keys)
+        out, ref = p.push_pull([np.ones((prev[r].shape[0], width), np.float32) for r in range(nrank)])
+        for r in range(nrank):
+            assert np.array_equal(out[r][:, 0], store[keys[r]].astype(np.float32)), (step, r)
+            assert np.array_equal(out[r], ref[r])
+        prev = keys
+    p.compare_ints(INT_ITEMS_PRE + INT_ITEMS_POST)
+    p.close()
+
+
+def test_gradient_sum_closed_form():
+    say("test_update::test_two")
+    nrank, length, width, bs = 4, 1024, 16, 1024
+    p, root = update_pair(nrank, length, width)
+    rngs = [np.random.RandomState(100 + r) for r in range(nrank)]
+    store = np.zeros((length, width))
+    prev = [np.zeros(0, np.int64)] * nrank
+    for step in range(50):
+        grads = [rngs[r].rand(prev[r].shape[0], width).astype(np.float32) for r in range(nrank)]
+        for r in range(nrank):
+            np.add.at(store, prev[r], grads[r].astype(np.float64))
+        keys = [rngs[r].randint(length, size=bs).astype(np.int64) for r in range(nrank)]
+        p.preprocess(keys)
+        out, ref = p.push_pull(grads)
+        for r in range(nrank):
+            assert np.max(np.abs(out[r] - store[keys[r]])) < 1e-4   # tests/test_update.py:70
+            assert_close(out[r], ref[r], 1e-5, "step %d rank %d" % (step, r))
+        prev = keys
+    p.close()
+
+
+@pytest.mark.parametrize("nrank,bounds,cache,width", [(4, (0, 0), "lower", 8), (4, (10, 10), "none", 128),
+                                                      (3, (2, 3), "third", 20), (8, (1, 0), "third", 64),
+                                                      (2, (0, 5), "lower", 3)])
+def test_stepwise_parity_with_staleness(nrank, bounds, cache, width):
+    say("stepwise", nrank, bounds, cache, width)
+    length, bs = 3000, 2500
+    p, root = update_pair(nrank, length, width, bounds=bounds, init=("Uniform", -1.0, 1.0), lr=0.5, cache=cache, seed=3)
+    rng = np.random.default_rng(nrank * 10 + bounds[0])
+    draw = zipf_sampler(length, 1.05, rng)
+    prev_n = [0] * nrank
+    for step in range(12):
+        keys = [draw(bs - 7 * r) if step % 3 else rng.integers(0, length, bs - 7 * r).astype(np.int64) for r in range(nrank)]
+        if step == 5:
+            keys[0] = np.zeros(0, np.int64)       # one shard sits a step out
+        p.preprocess(keys)
+        p.compare_ints(INT_ITEMS_PRE, "step %d" % step)
+        grads = [rng.normal(0, 0.1, size=(prev_n[r], width)).astype(np.float32) for r in range(nrank)]
+        if step == 8:
+            grads[1] = None                        # inference on one shard
+        out, ref = p.push_pull(grads)
+        p.compare_ints(INT_ITEMS_POST, "step %d" % step)
+        for r in range(nrank):
+            assert_close(out[r], ref[r], 1e-5, "dst step %d rank %d" % (step, r))
+        p.compare_state(1e-5, "step %d" % step)
+        prev_n = [k.shape[0] for k in keys]
+    p.close()
+
+
+def test_hand_computed_staleness_scenario():
+    # same scenario as tests/test_oracle_update.py::test_staleness_scenario_both_update, on the GPU
+    root = np.array([0, 1], np.uint8)
+    p = Pair(2, 2, 4, root, [np.array([0, 1]), np.array([1])], lr=-1.0, bounds=(1, 2))
+    one = np.array([1], np.int64)
+    r0, r1 = [], []
+    n_prev = 0
+    for step in range(4):
+        p.preprocess([one, one])
+        g = np.ones((n_prev, 4), np.float32)
+        out, ref = p.push_pull([g, g]); n_prev = 1
+        r0.append(float(out[0][0, 0])); r1.append(float(out[1][0, 0]))
+    assert r0 == [0.0, 1.0, 4.0, 5.0] and r1 == [0.0, 1.0, 2.0, 6.0]
+    assert p.tables[0].fetch(capi.STATS).tolist()[:3] == [1, 0, 0]
+    p.close()
+
+
+def test_per_shard_calls_from_threads():
+    # the reference's per-process call pattern (tests/check.py:40-44), one thread per shard
+    say("threads")
+    nrank, length, width, bs = 4, 1024, 32, 512
+    p, root = update_pair(nrank, length, width, bounds=(0, 0))
+    rng = np.random.RandomState(5)
+    steps = 6
+    keys = [[rng.randint(length, size=bs).astype(np.int64) for _ in range(steps)] for _ in range(nrank)]
+    outs = [[None] * steps for _ in range(nrank)]
+    errors = []
+
+    def worker(r):
+        try:
+            dst = torch.zeros((bs, width), device="cuda")
+            grad = torch.ones((bs, width), device="cuda")
+            torch.cuda.synchronize()
+            for s in range(steps):
+                p.tables[r].preprocess(keys[r][s].ctypes.data, bs)
+                p.tables[r].push_pull(grad.data_ptr() if s else 0, dst.data_ptr())
+                outs[r][s] = dst.cpu().numpy().copy()
+        except Exception as e:  # pragma: no cover
+            errors.append(e)
+
+    ts = [threading.Thread(target=worker, args=(r,)) for r in range(nrank)]
+    [t.start() for t in ts]
+    [t.join(60) for t in ts]
+    assert not errors, errors
+    store = np.zeros(length)
+    for s in range(steps):
+        if s > 0:
+            for r in range(nrank):
+                np.add.at(store, keys[r][s - 1], 1.0)
+        for r in range(nrank):
+            assert np.array_equal(outs[r][s][:, 0], store[keys[r][s]].astype(np.float32)), (s, r)
+    p.close()
+
+
+def test_group_errors():
+    root = np.array([0, 1], np.uint8)
+    t0 = capi.Table(0, 2, 0, "10.0.0.1", 999, 2, 4, 0, 0, root, np.array([0]), ("Zero", 0, 0), 0.1)
+    k = np.array([0], np.int64)
+    with pytest.raises(RuntimeError, match="every rank|missing ranks"):
+        capi.group_preprocess([t0], [k.ctypes.data], [1])
+    with pytest.raises(RuntimeError, match="already exists"):
+        capi.Table(0, 2, 0, "10.0.0.1", 999, 2, 4, 0, 0, root, np.array([0]), ("Zero", 0, 0), 0.1)
+    t0.close()
