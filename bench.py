@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Benchmark of the embedding hot path on one MI355X.
+
+One "step" = preprocess(batch t) + push_pull(grad of batch t-1, dst of batch t) on synthetic keys that are
+already resident in HBM, in steady state (every timed step both pushes and pulls).  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="cfg2")
+    ap.add_argument("--batches", type=int, default=4, help="distinct key batches cycled through")
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and samples (debugging only)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-steps", type=int, default=3)
+    ap.add_argument("--no-stage-timing", action="store_true")
+    return ap.parse_args()
+
+
+def cpu_baseline(cfg, ks, batches, width, lr, steps):
+    """Times the CPU restatement of the same step (the parity oracle, all host threads it is given) on a
+    bounded sample of the same workload: same table size, same batches, Zero-initialised table."""
+    from oracle import oracle as orc
+    rows = ks.rows
+    root = np.zeros(rows, np.uint8)
+    o = orc.Oracle(1, rows, width, 0, 0, root, [np.arange(rows, dtype=np.int64)], init=("Zero", 0.0, 0.0),
+                   learning_rate=lr)
+    o.set_parallel(True)
+    n = batches[0].shape[0]
+    rng = np.random.default_rng(7)
+    grad = rng.normal(0, 1e-3, size=(n, width)).astype(np.float32)
+    dst = np.empty((n, width), np.float32)
+    o.preprocess_raw([batches[0]])
+    o.push_pull_into([None], [dst])                       # warm-up: first pull, nothing to push yet
+    o.preprocess_raw([batches[1 % len(batches)]])
+    o.push_pull_into([grad], [dst])
+    t0 = time.perf_counter()
+    for s in range(steps):
+        o.preprocess_raw([batches[(s + 2) % len(batches)]])
+        o.push_pull_into([grad], [dst])
+    dt = time.perf_counter() - t0
+    cores = o.num_threads()
+    o.close()
+    return dict(value=n * steps / dt, unit="IDs/s", cores=cores, kind="port",
+                ms_per_step=1e3 * dt / steps,
+                sample="%d full-size steps (%d keys each, %d-row x %d table, zero-initialised) of the same batches, "
+                       "OpenMP oracle, warm" % (steps, n, rows, width))
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no second device); --gpus %d is not supported"
+              % a.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from hetuctr_amd import capi, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    cfg = workloads.CONFIGS[a.config]
+    width, lr = cfg["width"], cfg["lr"]
+    t_gen = time.perf_counter()
+    ks = workloads.KeyStream(cfg, seed=0, scale=a.scale)
+    batches = [ks.batch() for _ in range(max(2, a.batches))]
+    ks.release_tables()
+    n = batches[0].shape[0]
+    print("[bench] %s: %d rows x %d, %d keys/batch, %d batches generated in %.1fs" %
+          (a.config, ks.rows, width, n, len(batches), time.perf_counter() - t_gen), file=sys.stderr, flush=True)
+
+    torch.cuda.set_device(0)
+    t_init = time.perf_counter()
+    root = np.zeros(ks.rows, np.uint8)
+    storage = np.arange(ks.rows, dtype=np.int64)
+    capi.seed(0)
+    table = capi.Table(0, 1, 0, "127.0.0.1", 23456, ks.rows, width, 0, 0, root, storage, cfg["init"], lr, 0)
+    del root, storage
+    dkeys = [torch.from_numpy(b).cuda() for b in batches]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    grad = torch.randn((n, width), device="cuda", generator=gen) * 1e-3
+    dst = torch.empty((n, width), device="cuda")
+    torch.cuda.synchronize()
+    print("[bench] table + inputs resident in HBM after %.1fs" % (time.perf_counter() - t_init), file=sys.stderr, flush=True)
+
+    def step(i):
+        table.preprocess(dkeys[i % len(dkeys)].data_ptr(), n)
+        table.push_pull(grad.data_ptr(), dst.data_ptr())
+
+    uniq = {}
+    for i in range(max(a.warmup, 1)):
+        step(i)
+        uniq[i % len(dkeys)] = int(table.fetch(capi.SIZES)[1])
+    for i in range(len(dkeys)):                      # make sure U of every batch is known
+        if i not in uniq:
+            table.preprocess(dkeys[i].data_ptr(), n)
+            uniq[i] = int(table.fetch(capi.SIZES)[1])
+            table.push_pull(grad.data_ptr(), dst.data_ptr())
+    w0 = max(a.warmup, 1) + len(dkeys)
+    if not a.no_stage_timing:
+        table.stage_timing(True)
+    pre_ms = pp_ms = 0.0
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(w0 + i)
+        p, q = table.last_times()
+        pre_ms += p
+        pp_ms += q
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    stages = table.stage_times() if not a.no_stage_timing else {}
+    table.stage_timing(False)
+
+    ms_step = 1e3 * dt / a.steps
+    # distinct keys of the batches the timed steps used (current batch = pulled, previous = pushed)
+    u_cur = np.mean([uniq[(w0 + i) % len(dkeys)] for i in range(a.steps)])
+    u_prev = np.mean([uniq[(w0 + i - 1) % len(dkeys)] for i in range(a.steps)])
+    bytes_step = workloads.algorithmic_bytes(n, 0.5 * (u_cur + u_prev), width)
+    step_gbs = bytes_step / (ms_step * 1e-3) / 1e9
+
+    roof = None
+    if stages:
+        wide = {k: v for k, v in stages.items() if k in ("segment_sum_apply", "gather") and v[1] > 0}
+        dom = max(wide, key=lambda k: wide[k][0])
+        avg_ms = wide[dom][0] / wide[dom][1]
+        b = workloads.stage_bytes(dom, n, u_cur, n, u_prev, width)
+        roof = dict(bound="hbm", kernel=dom, achieved=b / (avg_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=b / (avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, traffic=None, avg_ms=avg_ms,
+                    algorithmic_bytes=int(b))
+
+    out = {
+        "metric": "sparse IDs/sec per train step (pull+push)", "value": n * a.steps / dt, "unit": "IDs/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: %d-row x %d fp32 table, batch %d samples x %d fields x %d ids = %d keys, %s, "
+                               "SGD lr %g, one shard (all rows local)" %
+                               (a.config, ks.rows, width, ks.samples, ks.fields, ks.hot, n,
+                                "uniform ids" if cfg["alpha"] is None else "per-field Zipf %.2f" % cfg["alpha"], lr),
+                   "keys_per_step": n, "unique_keys_per_step": float(u_cur), "width": width, "rows": ks.rows},
+        "unique_rows_per_sec": u_cur * a.steps / dt,
+        "device_ms_per_step": {"preprocess": pre_ms / a.steps, "push_pull": pp_ms / a.steps},
+        "step_hbm": {"algorithmic_bytes": int(bytes_step), "achieved_GBps": step_gbs, "frac": step_gbs / HBM_PEAK_GBS},
+        "stage_ms": {k: v[0] / max(v[1], 1) for k, v in stages.items() if v[1]},
+        "roofline": roof,
+    }
+    if not a.no_cpu:
+        del dst
+        torch.cuda.empty_cache()
+        try:
+            out["cpu_baseline"] = cpu_baseline(cfg, ks, batches, width, lr, a.cpu_steps)
+        except MemoryError as e:  # pragma: no cover
+            out["cpu_baseline"] = {"value": None, "error": str(e)}
+    table.close()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

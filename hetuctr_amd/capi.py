@@ -10,7 +10,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libhetuctr_hip.so")
 INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
 SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_push_pull", "hctr_group_preprocess",
            "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch",
-           "hctr_stream", "hctr_last_times", "hctr_version"]
+           "hctr_stream", "hctr_last_times", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
+           "hctr_stage_times", "hctr_version"]
 
 # items of hctr_debug_fetch (HCTR_F_*)
 UNIQUE, SORTED_ARG, RUN_START, IDX_MAP, ROOT, OFFSET, SEND_CNT, RECV_CNT = range(8)
@@ -50,6 +51,10 @@ def lib():
         l.hctr_debug_fetch.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t)]
         l.hctr_stream.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         l.hctr_last_times.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+        l.hctr_stage_timing.argtypes = [C.c_void_p, C.c_int]
+        l.hctr_stage_name.argtypes = [C.c_int]
+        l.hctr_stage_name.restype = C.c_char_p
+        l.hctr_stage_times.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
         _lib = l
     return _lib
 
@@ -102,6 +107,18 @@ class Table:
         a, b = C.c_float(), C.c_float()
         _check(lib().hctr_last_times(self._h, C.byref(a), C.byref(b)))
         return a.value, b.value
+
+    def stage_timing(self, on):
+        """Switches per-stage HIP-event timing on (resetting the accumulators) or off."""
+        _check(lib().hctr_stage_timing(self._h, int(on)))
+
+    def stage_times(self):
+        """{stage name: (accumulated ms, bracketed intervals)} since stage_timing(True)."""
+        n = lib().hctr_stage_count()
+        ms = (C.c_double * n)()
+        calls = (C.c_longlong * n)()
+        _check(lib().hctr_stage_times(self._h, ms, calls, n))
+        return {lib().hctr_stage_name(i).decode(): (ms[i], calls[i]) for i in range(n)}
 
     def __repr__(self):
         buf = C.create_string_buffer(256)

@@ -157,5 +157,31 @@ int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms) {
   });
 }
 
+int hctr_stage_timing(hctr_table *t, int on) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    Group &g = *t->shard->group;
+    g.stage_timing = on != 0;
+    for (int i = 0; i < S_COUNT; i++) {
+      g.stage_ms[i] = 0;
+      g.stage_calls[i] = 0;
+    }
+  });
+}
+
+int hctr_stage_count(void) { return S_COUNT; }
+const char *hctr_stage_name(int stage) { return stage_name(stage); }
+
+int hctr_stage_times(hctr_table *t, double *ms_total, long long *launches, int cap) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    Group &g = *t->shard->group;
+    for (int i = 0; i < S_COUNT && i < cap; i++) {
+      if (ms_total) ms_total[i] = g.stage_ms[i];
+      if (launches) launches[i] = g.stage_calls[i];
+    }
+  });
+}
+
 #pragma GCC visibility pop
 } // extern "C"

@@ -72,6 +72,10 @@ struct HostMirror {
 
 class Group;
 
+// stages whose device time can be measured separately (HIP events on the group's stream)
+enum Stage { S_KEYS = 0, S_SORT, S_UNIQUE, S_PLAN, S_PUSH, S_QUERY, S_EXCHANGE, S_OWNER, S_REFRESH, S_GATHER, S_COUNT };
+const char *stage_name(int s);
+
 class Shard {
  public:
   Shard(const hctr_config &cfg, const uint8_t *root_arr, const int64_t *storage_arr, size_t n_storage,
@@ -141,6 +145,16 @@ class Group {
   size_t desc_cap = 0;
   double wait_seconds = 120.0;
 
+  // per-stage device time, accumulated over calls while stage_timing is on
+  bool stage_timing = false;
+  double stage_ms[S_COUNT] = {};
+  long long stage_calls[S_COUNT] = {};
+  struct StageMark { int stage; hipEvent_t a, b; };
+  std::vector<StageMark> marks;          // of the call in flight
+  std::vector<hipEvent_t> event_pool;
+  hipEvent_t take_event();
+  void collect_marks();                  // after a stream sync
+
   void join(Shard *s);
   void leave(Shard *s);
   bool complete() const;
@@ -166,6 +180,22 @@ class Group {
   std::vector<size_t> a_n_;
   std::vector<const float *> a_grad_;
   std::vector<float *> a_dst_;
+};
+
+// brackets the launches of one stage with two events when stage timing is on
+struct StageScope {
+  Group &g;
+  int idx = -1;
+  StageScope(Group &grp, int stage) : g(grp) {
+    if (!g.stage_timing) return;
+    Group::StageMark m{stage, g.take_event(), g.take_event()};
+    HCTR_HIP(hipEventRecord(m.a, g.stream));
+    g.marks.push_back(m);
+    idx = (int)g.marks.size() - 1;
+  }
+  ~StageScope() {
+    if (idx >= 0) (void)hipEventRecord(g.marks[idx].b, g.stream);
+  }
 };
 
 std::shared_ptr<Group> find_or_create_group(int nrank, int device_id, const std::string &ip, int port);

@@ -12,6 +12,12 @@
 
 namespace hctr {
 
+const char *stage_name(int s) {
+  static const char *names[S_COUNT] = {"make_keys", "radix_sort", "unique_emit", "push_plan", "segment_sum_apply",
+                                       "query_build", "exchange", "owner_side", "cache_refresh", "gather"};
+  return s >= 0 && s < S_COUNT ? names[s] : "?";
+}
+
 static int bits_for(uint64_t max_value) { // bits needed to represent values 0..max_value
   int b = 0;
   while (b < 64 && (max_value >> b)) b++;
@@ -193,12 +199,16 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
   } else {
     reserve_batch_scratch(cur.n);
     HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s)); // :98-99
-    launch_make_keys(s, tv, kl, cur.keys.as<index_t>(), cur.n, comp.p, err.as<uint32_t>());
+    {
+      StageScope st(*group, S_KEYS);
+      launch_make_keys(s, tv, kl, cur.keys.as<index_t>(), cur.n, comp.p, err.as<uint32_t>());
+    }
     SortScratch sc;
     sc.ghist = ghist.as<uint32_t>();
     sc.bintot = bintot.as<uint32_t>();
     sc.blocks_cap = sort_blocks(cur.n);
     const void *sorted_keys = nullptr;
+    StageScope *sort_scope = new StageScope(*group, S_SORT);
     if (kl.wide) {
       const uint64_t *sk;
       radix_sort_positions<uint64_t>(s, comp.as<uint64_t>(), cur.n, kl.total_bits, ktmp0.as<uint64_t>(),
@@ -212,6 +222,8 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
                                      cur.sorted_arg.as<uint32_t>(), sc, &sk);
       sorted_keys = sk;
     }
+    delete sort_scope;
+    StageScope st(*group, S_UNIQUE);
     launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>());
   }
   launch_bucket_sizes(s, cur.view(), cfg.nrank, cnt_dev.as<uint64_t>());
@@ -229,6 +241,7 @@ void Shard::preprocess_gradient() {
   need.reserve((size_t)prev.n * 4);
   prefix.reserve((size_t)prev.n * 4);
   reserve_batch_scratch(prev.n);
+  StageScope st(*group, S_PLAN);
   launch_decide_update(s, tv, kl, prev.view(), need.as<uint32_t>());
   launch_exclusive_scan(s, need.as<uint32_t>(), prefix.as<uint32_t>(), prev.n, prev.dU.as<uint32_t>(),
                         block_sums.as<uint32_t>(), push_total.as<uint32_t>());
@@ -293,6 +306,7 @@ void Shard::generate_gradient(const float *grad) {
     a.g_cnt = g_cnt.as<version_t>();
     a.g_val = g_val.as<embed_t>();
   }
+  StageScope st(*group, S_PUSH);
   launch_push(s, tv, kl, prev.view(), a);
 }
 
@@ -302,6 +316,7 @@ void Shard::generate_query() {
   hipStream_t s = group->stream;
   q_idx.reserve(std::max<uint32_t>(cur.U, 1) * sizeof(index_t));
   q_ver.reserve(std::max<uint32_t>(cur.U, 1) * sizeof(version_t));
+  StageScope st(*group, S_QUERY);
   launch_lookup_version(s, tv, cur.view(), q_ver.as<version_t>());
   launch_unique_ids(s, kl, cur.view(), q_idx.as<index_t>());
 }
@@ -310,6 +325,7 @@ void Shard::generate_query() {
 void Shard::handle_gradient() {
   hipStream_t s = group->stream;
   last_stats[5] = (long long)rg_seg[cfg.nrank];
+  StageScope st(*group, S_OWNER);
   for (int src = 0; src < cfg.nrank; src++)
     launch_apply_remote(s, tv, rg_idx.as<index_t>(), rg_cnt.as<version_t>(), rg_val.as<embed_t>(),
                         (uint32_t)rg_seg[src], (uint32_t)rg_seg[src + 1], err.as<uint32_t>());
@@ -333,6 +349,7 @@ void Shard::handle_query() {
   ret_ver.reserve(std::max<uint32_t>(Q, 1) * sizeof(version_t));
   ret_val.reserve((size_t)std::max<uint32_t>(Q, 1) * cfg.width * sizeof(embed_t));
   reserve_batch_scratch(Q);
+  StageScope st(*group, S_OWNER);
   launch_decide_outdated(s, tv, rq_idx.as<index_t>(), rq_ver.as<version_t>(), Q, (uint32_t)rq_seg[cfg.rank],
                          (uint32_t)rq_seg[cfg.rank + 1], outdated.as<uint32_t>(), err.as<uint32_t>());
   launch_exclusive_scan(s, outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q, nullptr, block_sums.as<uint32_t>(),
@@ -374,6 +391,7 @@ void Shard::write_back(float *dst) {
   if (cfg.nrank > 1) {
     ret_i.reserve(std::max<uint32_t>(cur.U, 1) * 4);
     reserve_batch_scratch(cur.U);
+    StageScope st(*group, S_REFRESH);
     HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
     launch_exclusive_scan(s, got.as<uint32_t>(), ret_i.as<uint32_t>(), cur.U, nullptr, block_sums.as<uint32_t>(),
                           nullptr);
@@ -384,7 +402,10 @@ void Shard::write_back(float *dst) {
     launch_refresh(s, tv, cur.view(), a, stats.as<uint32_t>());
     HCTR_HIP(hipMemcpyAsync(mirror->stats, stats.p, 16, hipMemcpyDeviceToHost, s));
   }
-  if (dst != nullptr) launch_gather(s, tv, cur.view(), a);
+  if (dst != nullptr) {
+    StageScope st(*group, S_GATHER);
+    launch_gather(s, tv, cur.view(), a);
+  }
 }
 
 void Shard::finish_push_pull() {
@@ -495,6 +516,8 @@ Group::~Group() {
   if (desc_host) (void)hipHostFree(desc_host);
   if (ev0) (void)hipEventDestroy(ev0);
   if (ev1) (void)hipEventDestroy(ev1);
+  for (auto &m : marks) { (void)hipEventDestroy(m.a); (void)hipEventDestroy(m.b); }
+  for (auto e : event_pool) (void)hipEventDestroy(e);
   if (stream) (void)hipStreamDestroy(stream);
 }
 
@@ -515,8 +538,33 @@ bool Group::complete() const {
   return true;
 }
 
+hipEvent_t Group::take_event() {
+  if (!event_pool.empty()) {
+    hipEvent_t e = event_pool.back();
+    event_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e;
+  HCTR_HIP(hipEventCreate(&e));
+  return e;
+}
+
+void Group::collect_marks() {
+  for (auto &m : marks) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, m.a, m.b) == hipSuccess) {
+      stage_ms[m.stage] += ms;
+      stage_calls[m.stage]++;
+    }
+    event_pool.push_back(m.a);
+    event_pool.push_back(m.b);
+  }
+  marks.clear();
+}
+
 void Group::run_copies(std::vector<CopyDesc> &descs) {
   if (descs.empty()) return;
+  StageScope st(*this, S_EXCHANGE);
   if (descs.size() > desc_cap) {
     if (desc_host) HCTR_HIP(hipHostFree(desc_host));
     desc_host = nullptr;
@@ -625,6 +673,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
   HCTR_HIP(hipStreamSynchronize(stream));
   float ms = 0.f;
   HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+  collect_marks();
   std::string first_error;
   for (Shard *m : members) {
     m->last_pre_ms = ms;
@@ -657,6 +706,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
     for (Shard *m : members) m->handle_gradient();
     for (Shard *m : members) m->handle_query();
     HCTR_HIP(hipStreamSynchronize(stream)); // hetu_gpu_table.cu:33: the return counts size the next exchange
+    collect_marks();
     for (Shard *m : members) m->finish_handle_query();
     exchange_return();
   }
@@ -665,6 +715,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
   HCTR_HIP(hipStreamSynchronize(stream));
   float ms = 0.f;
   HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+  collect_marks();
   for (Shard *m : members) {
     m->last_pp_ms = ms;
     m->finish_push_pull();

@@ -102,6 +102,16 @@ int hctr_stream(hctr_table *t, void **stream_out);
  * that stream around the launched work (host-side waits excluded). */
 int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
 
+/* Per-stage device time.  hctr_stage_timing(t, 1) resets the accumulators and makes every later call bracket
+ * each stage's launches with HIP events on the table's stream; hctr_stage_times returns, per stage, the
+ * accumulated milliseconds and the number of bracketed intervals.  Stage i is named hctr_stage_name(i),
+ * 0 <= i < hctr_stage_count().  No counterpart in the reference, which is profiled from outside with nvprof
+ * (tests/run.sh:4). */
+int hctr_stage_timing(hctr_table *t, int on);
+int hctr_stage_count(void);
+const char *hctr_stage_name(int stage);
+int hctr_stage_times(hctr_table *t, double *ms_total, long long *launches, int cap);
+
 /* Version string of the library. */
 const char *hctr_version(void);
 

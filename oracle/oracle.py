@@ -44,6 +44,7 @@ def lib():
         _lib.orc_fetch.restype = C.c_longlong
         _lib.orc_fetch.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t]
         _lib.orc_last_error.restype = C.c_char_p
+        _lib.orc_num_threads.restype = C.c_int
         _lib.orc_init_values.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.c_float, C.c_uint]
     return _lib
 
@@ -100,6 +101,21 @@ class Oracle:
         if lib().orc_push_pull(self._h, _ptr_array(gs), _ptr_array(dsts)):
             raise RuntimeError(lib().orc_last_error().decode())
         return dsts
+
+    def push_pull_into(self, grads, dsts):
+        """Like push_pull with caller-provided float32 C-contiguous arrays (no allocation, no copies)."""
+        if lib().orc_push_pull(self._h, _ptr_array(grads), _ptr_array(dsts)):
+            raise RuntimeError(lib().orc_last_error().decode())
+
+    def preprocess_raw(self, keys):
+        """Like preprocess for int64 C-contiguous arrays, without conversions."""
+        ns = (C.c_size_t * self.R)(*[k.shape[0] for k in keys])
+        if lib().orc_preprocess(self._h, _ptr_array(keys), ns):
+            raise RuntimeError(lib().orc_last_error().decode())
+        self._n = [k.shape[0] for k in keys]
+
+    def num_threads(self):
+        return lib().orc_num_threads()
 
     def fetch(self, rank, which):
         n = lib().orc_fetch(self._h, rank, which, None, 0)
