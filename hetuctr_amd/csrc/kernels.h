@@ -26,7 +26,19 @@ struct BatchView {
   slot_t *uoff;              // [U]   resident offset of rank u or -1           (d_offset)
   uint32_t *bucket_lo;       // [R+1] first rank owned by each shard            (u_shape before :131)
   uint32_t *d_U;             // [1]   number of unique keys                     (unique_size)
+  uint32_t *long_list;       // [*d_nlong] unique ranks whose run is longer than kLongRun (any order)
+  uint32_t *d_nlong;         // [1]
 };
+
+// A run of equal keys longer than this is summed by a whole block that streams its gradient rows through
+// LDS; shorter runs are summed by a small group of lanes.  Occurrences of long runs carry kLongFlag in
+// rank_sorted.
+#ifndef HCTR_LONG_RUN
+#define HCTR_LONG_RUN 128
+#endif
+constexpr uint32_t kLongRun = HCTR_LONG_RUN;
+constexpr uint32_t kLongFlag = 0x80000000u;
+inline size_t long_list_capacity(uint32_t n) { return n / (kLongRun + 1) + 1; }
 
 struct TableView {
   int rank, nrank;
@@ -50,6 +62,9 @@ void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, co
 // sorted keys -> everything per unique key + inverse index.  block_heads: scratch of sort_blocks(n) words.
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
                    const BatchView &b, uint32_t *block_heads);
+
+// flags the occurrences of long runs in rank_sorted and lists those runs (after launch_unique)
+void launch_mark_long_runs(hipStream_t s, const BatchView &b);
 
 // device-wide exclusive scan of n (<= *d_n if d_n != nullptr) 32-bit values; block_sums: div_up(n_max,2048)+1 words.
 // total (optional) receives the sum.

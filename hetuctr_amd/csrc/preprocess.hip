@@ -105,6 +105,17 @@ __global__ __launch_bounds__(kBlock) void unique_emit(const K *__restrict__ sk, 
   }
 }
 
+__global__ __launch_bounds__(kBlock) void mark_long_runs(BatchView b) {
+  const uint32_t j = blockIdx.x * kBlock + threadIdx.x;
+  if (j >= b.n) return;
+  const uint32_t u = b.rank_sorted[j];
+  const uint32_t lo = b.run_start[u], hi = b.run_start[u + 1];
+  if (hi - lo > kLongRun) {
+    b.rank_sorted[j] = u | kLongFlag;
+    if (j == lo) b.long_list[atomicAdd(b.d_nlong, 1u)] = u;
+  }
+}
+
 // ---- generic device-wide exclusive scan (two launches, no inter-block waiting) ----------------------
 __global__ __launch_bounds__(kBlock) void scan_block_sums(const uint32_t *__restrict__ in, uint32_t n_max,
                                                           const uint32_t *__restrict__ d_n,
@@ -210,6 +221,13 @@ void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const
     hipLaunchKernelGGL(unique_emit<uint32_t>, dim3(nb), dim3(kBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
                        kl.id_bits, t.nrank, t.slot, block_heads, b);
   }
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_mark_long_runs(hipStream_t s, const BatchView &b) {
+  HCTR_HIP(hipMemsetAsync(b.d_nlong, 0, 4, s));
+  if (!b.n) return;
+  hipLaunchKernelGGL(mark_long_runs, dim3(div_up(b.n, kBlock)), dim3(kBlock), 0, s, b);
   HCTR_HIP(hipGetLastError());
 }
 

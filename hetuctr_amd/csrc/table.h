@@ -51,7 +51,7 @@ struct DeviceBuf {
 struct Batch {
   uint32_t n = 0;   // keys
   uint32_t U = 0;   // unique keys (host copy, valid after the preprocess call returned)
-  DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU;
+  DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong;
   std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
   std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
   void reserve(uint32_t n_keys, int nrank, bool wide);

@@ -38,6 +38,8 @@ void Batch::reserve(uint32_t n_keys, int nrank, bool wide) {
   uoff.reserve(n * sizeof(slot_t));
   bucket_lo.reserve((size_t)(nrank + 1) * 4);
   dU.reserve(4);
+  long_list.reserve(long_list_capacity((uint32_t)n) * 4);
+  dnlong.reserve(4);
 }
 
 BatchView Batch::view() const {
@@ -52,6 +54,8 @@ BatchView Batch::view() const {
   v.uoff = uoff.as<slot_t>();
   v.bucket_lo = bucket_lo.as<uint32_t>();
   v.d_U = dU.as<uint32_t>();
+  v.long_list = long_list.as<uint32_t>();
+  v.d_nlong = dnlong.as<uint32_t>();
   return v;
 }
 
@@ -135,6 +139,7 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   for (Batch *b : {&cur, &prev}) {
     b->reserve(1, c.nrank, kl.wide);
     HCTR_HIP(hipMemsetAsync(b->dU.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(b->dnlong.p, 0, 4, s));
     HCTR_HIP(hipMemsetAsync(b->bucket_lo.p, 0, b->bucket_lo.bytes, s));
     HCTR_HIP(hipMemsetAsync(b->run_start.p, 0, 4, s));
     b->send_cnt.assign(c.nrank + 1, 0);
@@ -196,6 +201,7 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
     HCTR_HIP(hipMemsetAsync(cur.dU.p, 0, 4, s));
     HCTR_HIP(hipMemsetAsync(cur.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
     HCTR_HIP(hipMemsetAsync(cur.run_start.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(cur.dnlong.p, 0, 4, s));
   } else {
     reserve_batch_scratch(cur.n);
     HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s)); // :98-99
@@ -225,6 +231,7 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
     delete sort_scope;
     StageScope st(*group, S_UNIQUE);
     launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>());
+    launch_mark_long_runs(s, cur.view());
   }
   launch_bucket_sizes(s, cur.view(), cfg.nrank, cnt_dev.as<uint64_t>());
 }
@@ -278,6 +285,7 @@ void Shard::generate_gradient(const float *grad) {
     prev.n = 0;
     prev.U = 0;
     HCTR_HIP(hipMemsetAsync(prev.dU.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(prev.dnlong.p, 0, 4, s));
     HCTR_HIP(hipMemsetAsync(prev.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
     std::fill(prev.push_cnt.begin(), prev.push_cnt.end(), 0);
     std::fill(prev.pushrecv_cnt.begin(), prev.pushrecv_cnt.end(), 0);
