@@ -20,7 +20,7 @@ struct BatchView {
   const index_t *keys;       // [n]   the ids as handed in                      (d_idx)
   uint32_t *sorted_arg;      // [n]   positions grouped by unique key, stable   (d_sorted_arg)
   uint32_t *rank_sorted;     // [n]   unique rank of sorted position j
-  uint32_t *idx_map;         // [n]   unique rank of position i                 (d_idx_map)
+  uint32_t *idx_map;         // [n]   unique rank of position i, filled on request only    (d_idx_map)
   void *ukey;                // [U]   sort key of unique rank u: id and owner   (d_unique_idx, d_root)
   uint32_t *run_start;       // [U+1] first sorted position of rank u           (d_run_length)
   slot_t *uoff;              // [U]   resident offset of rank u or -1           (d_offset)
@@ -57,12 +57,16 @@ struct TableView {
 
 // ---- preprocess ---------------------------------------------------------------------------------
 // ids -> sort keys; flags ids outside [0, id_max) in *err (and sorts them as id 0)
+// keys_copy (optional): the ids are also copied there (the reference's d_idx); nlong (optional) is zeroed
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err);
+                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong);
 // sorted keys -> everything per unique key + inverse index.  block_heads: scratch of sort_blocks(n) words.
+// u_copy (optional) receives the number of unique keys as well (b.d_U always does)
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
-                   const BatchView &b, uint32_t *block_heads);
+                   const BatchView &b, uint32_t *block_heads, uint32_t *u_copy);
 
+// batch-order inverse index from sorted_arg and rank_sorted (introspection; the hot path does not need it)
+void launch_idx_map(hipStream_t s, const BatchView &b);
 // flags the occurrences of long runs in rank_sorted and lists those runs (after launch_unique)
 void launch_mark_long_runs(hipStream_t s, const BatchView &b);
 

@@ -16,10 +16,13 @@ constexpr int kTile = kBlock * kItems; // == kSortTile, so sort_blocks(n) sizes 
 template <typename K>
 __global__ __launch_bounds__(kBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
                                                     int id_bits, int nrank, const worker_t *__restrict__ root,
-                                                    K *__restrict__ comp, uint32_t *__restrict__ err) {
+                                                    K *__restrict__ comp, uint32_t *__restrict__ err,
+                                                    index_t *__restrict__ keys_copy, uint32_t *__restrict__ nlong) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i == 0 && nlong) *nlong = 0;
   if (i >= n) return;
   uint64_t id = (uint64_t)keys[i];
+  if (keys_copy) keys_copy[i] = (index_t)id;
   if (id >= id_max) { // also catches negative ids
     atomicOr(err, 1u);
     id = 0;
@@ -28,25 +31,18 @@ __global__ __launch_bounds__(kBlock) void make_keys(const index_t *__restrict__ 
   comp[i] = (K)((r << id_bits) | id);
 }
 
-template <typename K>
-__device__ __forceinline__ void load_tile(const K *__restrict__ sk, uint32_t n, uint32_t j0, K (&key)[kItems], K &prev) {
-#pragma unroll
-  for (int k = 0; k < kItems; k++) key[k] = (j0 + k < n) ? sk[j0 + k] : (K)0;
-  prev = (j0 > 0 && j0 <= n) ? sk[j0 - 1] : (K)0;
-}
-
+// Sorted position j of a block's tile is handled by thread (j % kBlock) in round (j / kBlock): every load
+// and store below is coalesced across the wave.
 template <typename K>
 __global__ __launch_bounds__(kBlock) void head_count(const K *__restrict__ sk, uint32_t n,
                                                      uint32_t *__restrict__ block_heads) {
   __shared__ uint32_t sm[kBlock / kWave + 1];
-  const uint32_t j0 = blockIdx.x * kTile + threadIdx.x * kItems;
-  K key[kItems], prev;
-  load_tile(sk, n, j0, key, prev);
+  const uint32_t base = blockIdx.x * kTile;
   uint32_t c = 0;
 #pragma unroll
   for (int k = 0; k < kItems; k++) {
-    const uint32_t j = j0 + k;
-    c += (j < n) && (j == 0 || key[k] != (k ? key[k - 1] : prev));
+    const uint32_t j = base + k * kBlock + threadIdx.x;
+    if (j < n) c += (j == 0) || (sk[j] != sk[j - 1]);
   }
   uint32_t total;
   block_exclusive_scan<kBlock>(c, sm, total);
@@ -56,63 +52,107 @@ __global__ __launch_bounds__(kBlock) void head_count(const K *__restrict__ sk, u
 template <typename K>
 __global__ __launch_bounds__(kBlock) void unique_emit(const K *__restrict__ sk, uint32_t n, int id_bits, int nrank,
                                                       const slot_t *__restrict__ slot,
-                                                      const uint32_t *__restrict__ block_heads, BatchView b) {
-  __shared__ uint32_t sm[kBlock / kWave + 1];
-  // ranks before this block
+                                                      const uint32_t *__restrict__ block_heads, BatchView b,
+                                                      uint32_t *__restrict__ u_copy) {
+  constexpr int NW = kBlock / kWave;
+  __shared__ uint32_t sm[NW + 1];
+  __shared__ uint32_t wsum[kItems * NW + 1];
+  // unique ranks before this block
   uint32_t s = 0;
   for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlock) s += block_heads[i];
   uint32_t prefix;
   block_exclusive_scan<kBlock>(s, sm, prefix);
 
-  const uint32_t j0 = blockIdx.x * kTile + threadIdx.x * kItems;
-  K key[kItems], prev;
-  load_tile(sk, n, j0, key, prev);
+  const uint32_t base = blockIdx.x * kTile;
+  const unsigned lane = lane_id();
+  const int w = threadIdx.x / kWave;
+  K key[kItems], pk[kItems];
   bool head[kItems];
-  uint32_t c = 0;
+  uint32_t before[kItems];
 #pragma unroll
   for (int k = 0; k < kItems; k++) {
-    const uint32_t j = j0 + k;
-    head[k] = (j < n) && (j == 0 || key[k] != (k ? key[k - 1] : prev));
-    c += head[k];
+    const uint32_t j = base + k * kBlock + threadIdx.x;
+    const bool valid = j < n;
+    key[k] = valid ? sk[j] : (K)0;
+    pk[k] = (valid && j > 0) ? sk[j - 1] : (K)0;
+    head[k] = valid && (j == 0 || key[k] != pk[k]);
+    const uint64_t m = __ballot(head[k]);
+    before[k] = __popcll(m & ((1ull << lane) - 1ull));
+    if (lane == 0) wsum[k * NW + w] = __popcll(m);
   }
-  uint32_t total;
-  uint32_t run = prefix + block_exclusive_scan<kBlock>(c, sm, total); // heads before this thread's items
+  __syncthreads();
+  if (threadIdx.x == 0) { // 32 wave totals, in item order
+    uint32_t run = 0;
+#pragma unroll
+    for (int i = 0; i < kItems * NW; i++) {
+      const uint32_t v = wsum[i];
+      wsum[i] = run;
+      run += v;
+    }
+  }
+  __syncthreads();
   K *ukey = (K *)b.ukey;
   const K id_mask = (K)(((uint64_t)1 << id_bits) - 1);
+  slot_t off[kItems];
+#pragma unroll
+  // all lookups are issued before the first store (the compiler cannot prove that the output arrays do not
+  // alias the directory, so a store in between would serialise them)
+  for (int k = 0; k < kItems; k++) off[k] = head[k] ? slot[(uint64_t)(key[k] & id_mask)] : kNoSlot;
 #pragma unroll
   for (int k = 0; k < kItems; k++) {
-    const uint32_t j = j0 + k;
-    if (j >= n) break;
-    run += head[k];
-    const uint32_t rank = run - 1;
+    const uint32_t j = base + k * kBlock + threadIdx.x;
+    if (j >= n) continue;
+    const uint32_t rank = prefix + wsum[k * NW + w] + before[k] + (head[k] ? 1u : 0u) - 1u;
     const int r = (int)(key[k] >> id_bits);
     if (head[k]) {
       ukey[rank] = key[k];
       b.run_start[rank] = j;
-      b.uoff[rank] = slot[(uint64_t)(key[k] & id_mask)];
-      const K pk = k ? key[k - 1] : prev;
-      const int r_prev = j == 0 ? -1 : (int)(pk >> id_bits);
+      b.uoff[rank] = off[k];
+      const int r_prev = j == 0 ? -1 : (int)(pk[k] >> id_bits);
       for (int i = r_prev + 1; i <= r; i++) b.bucket_lo[i] = rank;
     }
     b.rank_sorted[j] = rank;
-    b.idx_map[b.sorted_arg[j]] = rank;
     if (j == n - 1) {
       const uint32_t U = rank + 1;
       *b.d_U = U;
+      if (u_copy) *u_copy = U;
       b.run_start[U] = n;
       for (int i = r + 1; i <= nrank; i++) b.bucket_lo[i] = U;
     }
   }
 }
 
-__global__ __launch_bounds__(kBlock) void mark_long_runs(BatchView b) {
+// The inverse index in batch order (the reference's d_idx_map).  The hot path works in sorted order
+// (sorted_arg + rank_sorted are the same mapping, grouped by key) and never reads this array; it is
+// materialised on request.
+__global__ __launch_bounds__(kBlock) void scatter_idx_map(BatchView b) {
   const uint32_t j = blockIdx.x * kBlock + threadIdx.x;
-  if (j >= b.n) return;
-  const uint32_t u = b.rank_sorted[j];
-  const uint32_t lo = b.run_start[u], hi = b.run_start[u + 1];
-  if (hi - lo > kLongRun) {
-    b.rank_sorted[j] = u | kLongFlag;
-    if (j == lo) b.long_list[atomicAdd(b.d_nlong, 1u)] = u;
+  if (j < b.n) b.idx_map[b.sorted_arg[j]] = b.rank_sorted[j] & ~kLongFlag;
+}
+
+__global__ __launch_bounds__(kBlock) void mark_long_runs(BatchView b) {
+  constexpr int kPer = 4;
+  const uint32_t base = blockIdx.x * (kBlock * kPer) + threadIdx.x;
+  uint32_t *__restrict__ rs = b.rank_sorted;
+  const uint32_t *__restrict__ run_start = b.run_start;
+  uint32_t u[kPer], lo[kPer], hi[kPer];
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    const uint32_t j = base + k * kBlock;
+    u[k] = j < b.n ? rs[j] : 0u;
+  }
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    lo[k] = run_start[u[k]];
+    hi[k] = run_start[u[k] + 1];
+  }
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    const uint32_t j = base + k * kBlock;
+    if (j < b.n && hi[k] - lo[k] > kLongRun) {
+      rs[j] = u[k] | kLongFlag;
+      if (j == lo[k]) b.long_list[atomicAdd(b.d_nlong, 1u)] = u[k];
+    }
   }
 }
 
@@ -195,39 +235,44 @@ __global__ void bucket_sizes(BatchView b, int nrank, uint64_t *__restrict__ cnt_
 } // namespace
 
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err) {
+                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong) {
   if (!n) return;
   if (kl.wide)
     hipLaunchKernelGGL(make_keys<uint64_t>, dim3(div_up(n, kBlock)), dim3(kBlock), 0, s, keys, n, t.id_max,
-                       kl.id_bits, t.nrank, t.root, (uint64_t *)comp_keys, err);
+                       kl.id_bits, t.nrank, t.root, (uint64_t *)comp_keys, err, keys_copy, nlong);
   else
     hipLaunchKernelGGL(make_keys<uint32_t>, dim3(div_up(n, kBlock)), dim3(kBlock), 0, s, keys, n, t.id_max,
-                       kl.id_bits, t.nrank, t.root, (uint32_t *)comp_keys, err);
+                       kl.id_bits, t.nrank, t.root, (uint32_t *)comp_keys, err, keys_copy, nlong);
   HCTR_HIP(hipGetLastError());
 }
 
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
-                   const BatchView &b, uint32_t *block_heads) {
+                   const BatchView &b, uint32_t *block_heads, uint32_t *u_copy) {
   if (!b.n) return;
   const unsigned nb = div_up(b.n, kTile);
   if (kl.wide) {
     hipLaunchKernelGGL(head_count<uint64_t>, dim3(nb), dim3(kBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
                        block_heads);
     hipLaunchKernelGGL(unique_emit<uint64_t>, dim3(nb), dim3(kBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
-                       kl.id_bits, t.nrank, t.slot, block_heads, b);
+                       kl.id_bits, t.nrank, t.slot, block_heads, b, u_copy);
   } else {
     hipLaunchKernelGGL(head_count<uint32_t>, dim3(nb), dim3(kBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
                        block_heads);
     hipLaunchKernelGGL(unique_emit<uint32_t>, dim3(nb), dim3(kBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
-                       kl.id_bits, t.nrank, t.slot, block_heads, b);
+                       kl.id_bits, t.nrank, t.slot, block_heads, b, u_copy);
   }
   HCTR_HIP(hipGetLastError());
 }
 
-void launch_mark_long_runs(hipStream_t s, const BatchView &b) {
-  HCTR_HIP(hipMemsetAsync(b.d_nlong, 0, 4, s));
+void launch_idx_map(hipStream_t s, const BatchView &b) {
   if (!b.n) return;
-  hipLaunchKernelGGL(mark_long_runs, dim3(div_up(b.n, kBlock)), dim3(kBlock), 0, s, b);
+  hipLaunchKernelGGL(scatter_idx_map, dim3(div_up(b.n, kBlock)), dim3(kBlock), 0, s, b);
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_mark_long_runs(hipStream_t s, const BatchView &b) { // *b.d_nlong was zeroed by make_keys
+  if (!b.n) return;
+  hipLaunchKernelGGL(mark_long_runs, dim3(div_up(b.n, kBlock * 4)), dim3(kBlock), 0, s, b);
   HCTR_HIP(hipGetLastError());
 }
 

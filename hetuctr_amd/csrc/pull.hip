@@ -116,25 +116,29 @@ __global__ __launch_bounds__(kBlock) void refresh(TableView t, int id_bits_unuse
         *(const V *)(a.in_val + (size_t)k * W + col) + *(const V *)(t.pend + (size_t)o * W + col);
 }
 
-// one group per kRows consecutive output rows; rows of the table are read with 16-byte lanes, the output
-// is written once and never re-read by this kernel: non-temporal stores
+// Gather in SORTED order: one group per kRows consecutive sorted positions.  Duplicates of a key are adjacent,
+// so a table row is fetched from HBM once and re-read from cache for its other occurrences; every output row is
+// written whole, once, with non-temporal stores, at the batch position sorted_arg names.
 constexpr int kRows = 4;
 template <int VEC, int LPR, bool kLocalOnly>
 __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullArgs a) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
   const uint32_t n = c.n, W = t.width;
-  const uint32_t i0 = (blockIdx.x * kGroups + threadIdx.x / LPR) * kRows;
-  if (i0 >= n) return;
+  const uint32_t j0 = (blockIdx.x * kGroups + threadIdx.x / LPR) * kRows;
+  if (j0 >= n) return;
   const uint32_t gl = threadIdx.x % LPR;
   const embed_t *src[kRows];
+  embed_t *dst[kRows];
 #pragma unroll
   for (int k = 0; k < kRows; k++) {
-    const uint32_t i = min(i0 + k, n - 1);
-    const uint32_t u = c.idx_map[i];
+    const uint32_t j = min(j0 + k, n - 1);
+    const uint32_t u = c.rank_sorted[j] & ~kLongFlag;
+    const uint32_t i = c.sorted_arg[j];
     const slot_t o = c.uoff[u];
     if (kLocalOnly || o != kNoSlot) src[k] = t.emb + (size_t)o * W;
     else src[k] = a.in_val + (size_t)a.ret_i[u] * W;
+    dst[k] = a.dst + (size_t)i * W;
   }
   for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
     V v[kRows];
@@ -142,7 +146,7 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
     for (int k = 0; k < kRows; k++) v[k] = *(const V *)(src[k] + col);
 #pragma unroll
     for (int k = 0; k < kRows; k++)
-      if (i0 + k < n) __builtin_nontemporal_store(v[k], (V *)(a.dst + (size_t)(i0 + k) * W + col));
+      if (j0 + k < n) __builtin_nontemporal_store(v[k], (V *)(dst[k] + col));
   }
 }
 

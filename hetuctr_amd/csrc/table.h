@@ -51,6 +51,7 @@ struct DeviceBuf {
 struct Batch {
   uint32_t n = 0;   // keys
   uint32_t U = 0;   // unique keys (host copy, valid after the preprocess call returned)
+  bool idx_map_valid = false;
   DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong;
   std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
   std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
@@ -58,15 +59,20 @@ struct Batch {
   BatchView view() const;
 };
 
-// values the host reads back after a call; lives in pinned host memory
-struct HostMirror {
+// What the host reads back after a preprocess call: written by kernels into one device block (DevStat) and
+// copied with ONE transfer into the pinned HostMirror.  A single shard only needs the first 16 bytes.
+struct DevStat {
   uint32_t U;
   uint32_t err;
   uint32_t push_total;
-  uint32_t ret_total;
-  uint32_t stats[4];
+  uint32_t pad;
   uint64_t send_cnt[257];
   uint64_t push_cnt[257];
+};
+struct HostMirror {
+  DevStat st;
+  uint32_t ret_total;
+  uint32_t stats[4];
   uint32_t ret_seg[258];
 };
 
@@ -109,8 +115,10 @@ class Shard {
   bool prev_active = false; // false: inference step or no previous batch, nothing is pushed
   DeviceBuf root, slot, emb, ver, pend, upd, store_ids;
   // scratch shared by the stages
-  DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, ghist, bintot, block_sums, err, stats;
-  DeviceBuf need, prefix, push_total, cnt_dev;
+  DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, ghist, bintot, block_sums, dstat, stats;
+  DeviceBuf need, prefix;
+  DevStat *dst_ = nullptr; // == dstat.p
+  uint32_t *err_ptr() const { return &dst_->err; }
   // send side
   DeviceBuf q_idx, q_ver, g_idx, g_cnt, g_val;
   // receive side (owner role)

@@ -126,16 +126,13 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   HCTR_HIP(hipMemsetAsync(pend.p, 0, pend.bytes, s));
   HCTR_HIP(hipMemsetAsync(upd.p, 0, upd.bytes, s));
 
-  err.reserve(4);
+  dstat.reserve(sizeof(DevStat));
+  dst_ = dstat.as<DevStat>();
   stats.reserve(16);
-  push_total.reserve(4);
   ret_total.reserve(4);
   ret_seg_dev.reserve(2 * 258 * 4);
-  cnt_dev.reserve(2 * 257 * sizeof(uint64_t));
-  HCTR_HIP(hipMemsetAsync(err.p, 0, 4, s));
+  HCTR_HIP(hipMemsetAsync(dstat.p, 0, dstat.bytes, s));
   HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
-  HCTR_HIP(hipMemsetAsync(push_total.p, 0, 4, s));
-  HCTR_HIP(hipMemsetAsync(cnt_dev.p, 0, cnt_dev.bytes, s));
   for (Batch *b : {&cur, &prev}) {
     b->reserve(1, c.nrank, kl.wide);
     HCTR_HIP(hipMemsetAsync(b->dU.p, 0, 4, s));
@@ -196,6 +193,7 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
   hipStream_t s = group->stream;
   cur.n = (uint32_t)n;
   cur.U = 0;
+  cur.idx_map_valid = false;
   cur.reserve(cur.n, cfg.nrank, kl.wide);
   if (n == 0) { // :93-95
     HCTR_HIP(hipMemsetAsync(cur.dU.p, 0, 4, s));
@@ -204,10 +202,19 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
     HCTR_HIP(hipMemsetAsync(cur.dnlong.p, 0, 4, s));
   } else {
     reserve_batch_scratch(cur.n);
-    HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s)); // :98-99
     {
+      // ids -> device copy (:98-99) and sort keys.  When the caller's pointer is device-visible the copy is
+      // written by the same kernel that reads the ids; a pageable host buffer goes through a transfer first.
       StageScope st(*group, S_KEYS);
-      launch_make_keys(s, tv, kl, cur.keys.as<index_t>(), cur.n, comp.p, err.as<uint32_t>());
+      hipPointerAttribute_t attr;
+      const bool visible = hipPointerGetAttributes(&attr, keys) == hipSuccess &&
+                           (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged);
+      if (!visible) {
+        (void)hipGetLastError(); // an unregistered host pointer leaves a sticky "invalid value"
+        HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
+      }
+      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, comp.p, err_ptr(),
+                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>());
     }
     SortScratch sc;
     sc.ghist = ghist.as<uint32_t>();
@@ -230,19 +237,20 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
     }
     delete sort_scope;
     StageScope st(*group, S_UNIQUE);
-    launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>());
+    launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>(), &dst_->U);
     launch_mark_long_runs(s, cur.view());
   }
-  launch_bucket_sizes(s, cur.view(), cfg.nrank, cnt_dev.as<uint64_t>());
+  if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt);
 }
 
 // csrc/core/preprocess.cu:148-182
 void Shard::preprocess_gradient() {
   hipStream_t s = group->stream;
-  uint64_t *cnt = cnt_dev.as<uint64_t>() + 257;
-  if (cfg.nrank == 1 || prev.n == 0) { // single shard: every key is owned, nothing is ever pushed
+  uint64_t *cnt = dst_->push_cnt;
+  if (cfg.nrank == 1) return; // single shard: every key is owned, nothing is ever pushed
+  if (prev.n == 0) {
     HCTR_HIP(hipMemsetAsync(cnt, 0, (size_t)(cfg.nrank + 1) * sizeof(uint64_t), s));
-    HCTR_HIP(hipMemsetAsync(push_total.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(&dst_->push_total, 0, 4, s));
     return;
   }
   need.reserve((size_t)prev.n * 4);
@@ -251,30 +259,33 @@ void Shard::preprocess_gradient() {
   StageScope st(*group, S_PLAN);
   launch_decide_update(s, tv, kl, prev.view(), need.as<uint32_t>());
   launch_exclusive_scan(s, need.as<uint32_t>(), prefix.as<uint32_t>(), prev.n, prev.dU.as<uint32_t>(),
-                        block_sums.as<uint32_t>(), push_total.as<uint32_t>());
-  launch_bucket_counts(s, prev.view(), prefix.as<uint32_t>(), push_total.as<uint32_t>(), cfg.nrank, cnt);
+                        block_sums.as<uint32_t>(), &dst_->push_total);
+  launch_bucket_counts(s, prev.view(), prefix.as<uint32_t>(), &dst_->push_total, cfg.nrank, cnt);
 }
 
 void Shard::enqueue_readback_preprocess() {
   hipStream_t s = group->stream;
-  const size_t r1 = (size_t)(cfg.nrank + 1) * sizeof(uint64_t);
-  HCTR_HIP(hipMemcpyAsync(&mirror->U, cur.dU.p, 4, hipMemcpyDeviceToHost, s));
-  HCTR_HIP(hipMemcpyAsync(&mirror->err, err.p, 4, hipMemcpyDeviceToHost, s));
-  HCTR_HIP(hipMemcpyAsync(&mirror->push_total, push_total.p, 4, hipMemcpyDeviceToHost, s));
-  HCTR_HIP(hipMemcpyAsync(mirror->send_cnt, cnt_dev.p, r1, hipMemcpyDeviceToHost, s));
-  HCTR_HIP(hipMemcpyAsync(mirror->push_cnt, cnt_dev.as<uint64_t>() + 257, r1, hipMemcpyDeviceToHost, s));
+  if (cur.n == 0) HCTR_HIP(hipMemsetAsync(&dst_->U, 0, 4, s));
+  const size_t bytes = cfg.nrank == 1 ? 16 : sizeof(DevStat);
+  HCTR_HIP(hipMemcpyAsync(&mirror->st, dstat.p, bytes, hipMemcpyDeviceToHost, s));
 }
 
 void Shard::finish_preprocess() {
-  cur.U = mirror->U;
+  cur.U = mirror->st.U;
   prev_active = prev.n > 0;
-  for (int i = 0; i <= cfg.nrank; i++) {
-    cur.send_cnt[i] = mirror->send_cnt[i];
-    prev.push_cnt[i] = mirror->push_cnt[i];
+  if (cfg.nrank == 1) {
+    cur.send_cnt[0] = cur.U;
+    prev.push_cnt[0] = 0;
+  } else {
+    for (int i = 0; i <= cfg.nrank; i++) {
+      cur.send_cnt[i] = mirror->st.send_cnt[i];
+      prev.push_cnt[i] = mirror->st.push_cnt[i];
+    }
   }
-  if (mirror->err) {
-    HCTR_HIP(hipMemsetAsync(err.p, 0, 4, group->stream));
-    HCTR_CHECK(!(mirror->err & 1u), "preprocess: a key lies outside [0, length) (it was treated as id 0)");
+  if (mirror->st.err) {
+    const uint32_t e = mirror->st.err;
+    HCTR_HIP(hipMemsetAsync(err_ptr(), 0, 4, group->stream));
+    HCTR_CHECK(!(e & 1u), "preprocess: a key lies outside [0, length) (it was treated as id 0)");
   }
 }
 
@@ -336,7 +347,7 @@ void Shard::handle_gradient() {
   StageScope st(*group, S_OWNER);
   for (int src = 0; src < cfg.nrank; src++)
     launch_apply_remote(s, tv, rg_idx.as<index_t>(), rg_cnt.as<version_t>(), rg_val.as<embed_t>(),
-                        (uint32_t)rg_seg[src], (uint32_t)rg_seg[src + 1], err.as<uint32_t>());
+                        (uint32_t)rg_seg[src], (uint32_t)rg_seg[src + 1], err_ptr());
 }
 
 __global__ void segment_bounds(const uint32_t *__restrict__ out_pos, const uint32_t *__restrict__ total,
@@ -359,7 +370,7 @@ void Shard::handle_query() {
   reserve_batch_scratch(Q);
   StageScope st(*group, S_OWNER);
   launch_decide_outdated(s, tv, rq_idx.as<index_t>(), rq_ver.as<version_t>(), Q, (uint32_t)rq_seg[cfg.rank],
-                         (uint32_t)rq_seg[cfg.rank + 1], outdated.as<uint32_t>(), err.as<uint32_t>());
+                         (uint32_t)rq_seg[cfg.rank + 1], outdated.as<uint32_t>(), err_ptr());
   launch_exclusive_scan(s, outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q, nullptr, block_sums.as<uint32_t>(),
                         ret_total.as<uint32_t>());
   launch_pack_rows(s, tv, rq_idx.as<index_t>(), outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q,
@@ -373,15 +384,15 @@ void Shard::handle_query() {
                      seg_d, R, Q, seg_d + 258);
   HCTR_HIP(hipGetLastError());
   HCTR_HIP(hipMemcpyAsync(seg_h, seg_d + 258, (size_t)(R + 1) * 4, hipMemcpyDeviceToHost, s));
-  HCTR_HIP(hipMemcpyAsync(&mirror->err, err.p, 4, hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipMemcpyAsync(&mirror->st.err, err_ptr(), 4, hipMemcpyDeviceToHost, s));
 }
 
 void Shard::finish_handle_query() {
   for (int i = 0; i <= cfg.nrank; i++) ret_seg[i] = mirror->ret_seg[i];
   last_stats[4] = (long long)ret_seg[cfg.nrank];
-  if (mirror->err) {
-    const uint32_t e = mirror->err;
-    HCTR_HIP(hipMemsetAsync(err.p, 0, 4, group->stream));
+  if (mirror->st.err) {
+    const uint32_t e = mirror->st.err;
+    HCTR_HIP(hipMemsetAsync(err_ptr(), 0, 4, group->stream));
     HCTR_CHECK(!(e & 2u), "a pushed row reached a shard that does not own it");
     HCTR_CHECK(!(e & 4u), "a queried row reached a shard that does not own it");
   }
@@ -460,7 +471,14 @@ size_t Shard::fetch(int which, void *out, size_t cap) {
     case HCTR_F_ROOT: { auto k = ukeys(cur); for (auto &x : k) x >>= kl.id_bits; return put64(k, cur.U, out, cap); }
     case HCTR_F_SORTED_ARG: return put64(download<uint32_t>(cur.sorted_arg.p, cur.n), cur.n, out, cap);
     case HCTR_F_RUN_START: return put64(download<uint32_t>(cur.run_start.p, (size_t)cur.U + 1), (size_t)cur.U + 1, out, cap);
-    case HCTR_F_IDX_MAP: return put64(download<uint32_t>(cur.idx_map.p, cur.n), cur.n, out, cap);
+    case HCTR_F_IDX_MAP: {
+      if (!cur.idx_map_valid) {
+        launch_idx_map(group->stream, cur.view());
+        HCTR_HIP(hipStreamSynchronize(group->stream));
+        cur.idx_map_valid = true;
+      }
+      return put64(download<uint32_t>(cur.idx_map.p, cur.n), cur.n, out, cap);
+    }
     case HCTR_F_OFFSET: return put64(download<slot_t>(cur.uoff.p, cur.U), cur.U, out, cap);
     case HCTR_F_SEND_CNT: return put64(cur.send_cnt, R, out, cap);
     case HCTR_F_RECV_CNT: return put64(cur.recv_cnt, R, out, cap);
