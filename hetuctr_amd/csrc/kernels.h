@@ -26,19 +26,33 @@ struct BatchView {
   slot_t *uoff;              // [U]   resident offset of rank u or -1           (d_offset)
   uint32_t *bucket_lo;       // [R+1] first rank owned by each shard            (u_shape before :131)
   uint32_t *d_U;             // [1]   number of unique keys                     (unique_size)
-  uint32_t *long_list;       // [*d_nlong] unique ranks whose run is longer than kLongRun (any order)
-  uint32_t *d_nlong;         // [1]
+  uint32_t *long_list;       // [kLongBuckets][long_cap] unique ranks whose run is longer than kLongRun, by length class
+  uint32_t *d_nlong;         // [kLongBuckets] entries per class, then [kLongBuckets]: work counter of the push
+  uint32_t long_cap;         // capacity of one class
+  uint32_t *med_list;        // [d_nlong[kMedCount]] unique ranks with kTinyRun < run length <= kLongRun (any order)
 };
 
+// d_nlong layout: [0, kLongBuckets) long runs per class, then the long work counter, the number of medium runs
+// and the medium work counter
+constexpr int kLongWork = 8, kMedCount = 9, kMedWork = 10, kRunCounters = 11;
+
 // A run of equal keys longer than this is summed by a whole block that streams its gradient rows through
-// LDS; shorter runs are summed by a small group of lanes.  Occurrences of long runs carry kLongFlag in
-// rank_sorted.
+// LDS; shorter runs are summed by a small group of lanes.
 #ifndef HCTR_LONG_RUN
 #define HCTR_LONG_RUN 128
 #endif
 constexpr uint32_t kLongRun = HCTR_LONG_RUN;
-constexpr uint32_t kLongFlag = 0x80000000u;
+#ifndef HCTR_TINY_RUN
+#define HCTR_TINY_RUN 8
+#endif
+constexpr uint32_t kTinyRun = HCTR_TINY_RUN; // runs up to this length are summed by the group that owns their rank
+// Long runs are listed by length class (class 0 = longest) so that the push can start the longest chains first.
+constexpr int kLongBuckets = 8;
 inline size_t long_list_capacity(uint32_t n) { return n / (kLongRun + 1) + 1; }
+inline size_t med_list_capacity(uint32_t n) { return n / (kTinyRun + 1) + 1; }
+__host__ __device__ inline int long_bucket(uint32_t len) {
+  return len >= 8192 ? 0 : len >= 4096 ? 1 : len >= 2048 ? 2 : len >= 1024 ? 3 : len >= 512 ? 4 : len >= 256 ? 5 : 6;
+}
 
 struct TableView {
   int rank, nrank;
@@ -67,8 +81,8 @@ void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const
 
 // batch-order inverse index from sorted_arg and rank_sorted (introspection; the hot path does not need it)
 void launch_idx_map(hipStream_t s, const BatchView &b);
-// flags the occurrences of long runs in rank_sorted and lists those runs (after launch_unique)
-void launch_mark_long_runs(hipStream_t s, const BatchView &b);
+// lists the runs longer than kLongRun by length class (after launch_unique)
+void launch_list_long_runs(hipStream_t s, const BatchView &b);
 
 // device-wide exclusive scan of n (<= *d_n if d_n != nullptr) 32-bit values; block_sums: div_up(n_max,2048)+1 words.
 // total (optional) receives the sum.
@@ -92,8 +106,16 @@ struct PushArgs {
   version_t *g_cnt;
   embed_t *g_val;
 };
-size_t push_tiles(uint32_t n_prev);
-void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &prev, const PushArgs &a);
+// The push runs as three kernels (long, medium and short runs of duplicates) on three streams of default
+// priority; everything before it on `main` happens before all three, everything after it on `main` after them.
+struct PushStreams {
+  hipStream_t main, aux1, aux2;
+  hipEvent_t fork, join1, join2;
+  bool main_idle; // nothing is pending on `main` when the push is launched: the fork event is not needed
+};
+// n_unique: number of unique keys of `prev` (host copy)
+void launch_push(const PushStreams &ps, const TableView &t, const KeyLayout &kl, const BatchView &prev,
+                 uint32_t n_unique, const PushArgs &a);
 
 // ---- query / owner side / pull -------------------------------------------------------------------------
 void launch_lookup_version(hipStream_t s, const TableView &t, const BatchView &cur, version_t *q_ver);

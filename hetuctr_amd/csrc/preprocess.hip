@@ -19,7 +19,7 @@ __global__ __launch_bounds__(kBlock) void make_keys(const index_t *__restrict__ 
                                                     K *__restrict__ comp, uint32_t *__restrict__ err,
                                                     index_t *__restrict__ keys_copy, uint32_t *__restrict__ nlong) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i == 0 && nlong) *nlong = 0;
+  if (i < kRunCounters && nlong) nlong[i] = 0; // run-list counters and work counters of this batch
   if (i >= n) return;
   uint64_t id = (uint64_t)keys[i];
   if (keys_copy) keys_copy[i] = (index_t)id;
@@ -127,32 +127,27 @@ __global__ __launch_bounds__(kBlock) void unique_emit(const K *__restrict__ sk, 
 // materialised on request.
 __global__ __launch_bounds__(kBlock) void scatter_idx_map(BatchView b) {
   const uint32_t j = blockIdx.x * kBlock + threadIdx.x;
-  if (j < b.n) b.idx_map[b.sorted_arg[j]] = b.rank_sorted[j] & ~kLongFlag;
+  if (j < b.n) b.idx_map[b.sorted_arg[j]] = b.rank_sorted[j];
 }
 
-__global__ __launch_bounds__(kBlock) void mark_long_runs(BatchView b) {
-  constexpr int kPer = 4;
-  const uint32_t base = blockIdx.x * (kBlock * kPer) + threadIdx.x;
-  uint32_t *__restrict__ rs = b.rank_sorted;
-  const uint32_t *__restrict__ run_start = b.run_start;
-  uint32_t u[kPer], lo[kPer], hi[kPer];
-#pragma unroll
-  for (int k = 0; k < kPer; k++) {
-    const uint32_t j = base + k * kBlock;
-    u[k] = j < b.n ? rs[j] : 0u;
+// one thread per unique rank: long runs are listed by length class, medium runs in one list, for the push.
+// Medium runs are many: a wave reserves its list entries with ONE atomic.
+__global__ __launch_bounds__(kBlock) void list_long_runs(BatchView b) {
+  const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
+  const bool valid = u < *b.d_U;
+  const uint32_t len = valid ? b.run_start[u + 1] - b.run_start[u] : 0u;
+  if (len > kLongRun) {
+    const int c = long_bucket(len);
+    b.long_list[(size_t)c * b.long_cap + atomicAdd(&b.d_nlong[c], 1u)] = u;
   }
-#pragma unroll
-  for (int k = 0; k < kPer; k++) {
-    lo[k] = run_start[u[k]];
-    hi[k] = run_start[u[k] + 1];
-  }
-#pragma unroll
-  for (int k = 0; k < kPer; k++) {
-    const uint32_t j = base + k * kBlock;
-    if (j < b.n && hi[k] - lo[k] > kLongRun) {
-      rs[j] = u[k] | kLongFlag;
-      if (j == lo[k]) b.long_list[atomicAdd(b.d_nlong, 1u)] = u[k];
-    }
+  const bool med = len > kTinyRun && len <= kLongRun;
+  const uint64_t m = __ballot(med);
+  if (m) {
+    const unsigned lane = lane_id();
+    uint32_t base = 0;
+    if (lane == (unsigned)__ffsll((long long)m) - 1u) base = atomicAdd(&b.d_nlong[kMedCount], (uint32_t)__popcll(m));
+    base = __shfl(base, __ffsll((long long)m) - 1, kWave);
+    if (med) b.med_list[base + __popcll(m & ((1ull << lane) - 1ull))] = u;
   }
 }
 
@@ -270,9 +265,9 @@ void launch_idx_map(hipStream_t s, const BatchView &b) {
   HCTR_HIP(hipGetLastError());
 }
 
-void launch_mark_long_runs(hipStream_t s, const BatchView &b) { // *b.d_nlong was zeroed by make_keys
+void launch_list_long_runs(hipStream_t s, const BatchView &b) { // the class counters were zeroed by make_keys
   if (!b.n) return;
-  hipLaunchKernelGGL(mark_long_runs, dim3(div_up(b.n, kBlock * 4)), dim3(kBlock), 0, s, b);
+  hipLaunchKernelGGL(list_long_runs, dim3(div_up(b.n, kBlock)), dim3(kBlock), 0, s, b);
   HCTR_HIP(hipGetLastError());
 }
 

@@ -133,7 +133,7 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
 #pragma unroll
   for (int k = 0; k < kRows; k++) {
     const uint32_t j = min(j0 + k, n - 1);
-    const uint32_t u = c.rank_sorted[j] & ~kLongFlag;
+    const uint32_t u = c.rank_sorted[j];
     const uint32_t i = c.sorted_arg[j];
     const slot_t o = c.uoff[u];
     if (kLocalOnly || o != kNoSlot) src[k] = t.emb + (size_t)o * W;

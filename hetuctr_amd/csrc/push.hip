@@ -9,15 +9,15 @@
 // every run of equal keys is summed by ONE chain of additions per column, in exactly that order: sums are
 // bit-identical to the reference's order (compiled without fused multiply-add contraction), for any skew.
 //
-// One launch, two roles (block index decides):
-//  * long role (first blocks): a run longer than kLongRun is streamed by a whole block.  All 512 threads
-//    keep kDepth 16-byte loads of gradient rows in flight each and stage them through a ring of LDS slots;
-//    the first wave adds the staged rows in order, one column per lane.  The serial chain costs one LDS read
-//    and one add per duplicate while the memory latency is covered by the whole block.  A run is split by
-//    column slices of kSlice floats over several blocks.
-//  * tile role: the sorted occurrence list is cut into tiles of kTileOcc occurrences; a group of LPR lanes
-//    (LPR*VEC floats = one row) sums the short runs that START in its tile, walking past the tile end to
-//    finish the last one.  Occurrences of long runs are flagged in rank_sorted and skipped.
+// Three kernels, one per class of run length, launched on three streams so that they overlap:
+//  * long (> kLongRun duplicates): a run is streamed by a whole block.  Seven loader waves keep several
+//    16-byte loads of gradient rows in flight each and stage them through a ring of LDS slots; the first wave
+//    adds the staged rows in order, one column per lane.  The serial chain costs one LDS read and one add per
+//    duplicate while the memory latency is covered by the whole block.  A run is split by column slices of
+//    kSlice floats over several blocks; the longest runs are started first.
+//  * medium (kTinyRun < duplicates <= kLongRun): one group of LPR lanes per run, kBatch rows in flight.
+//  * short (<= kTinyRun): a group of LPR lanes (LPR*VEC floats = one row) owns a few consecutive unique keys
+//    and sums their runs, all first loads of the group issued together.
 #include "kernels.h"
 
 namespace hctr {
@@ -27,26 +27,33 @@ namespace hctr {
 #define HCTR_TILE_BATCH 8
 #endif
 #ifndef HCTR_DEPTH
-#define HCTR_DEPTH 8
+#define HCTR_DEPTH 4
+#endif
+#ifndef HCTR_RPT
+#define HCTR_RPT 2
 #endif
 #ifndef HCTR_SLICE
 #define HCTR_SLICE 64
 #endif
 #ifndef HCTR_LONG_BLOCKS
-#define HCTR_LONG_BLOCKS 1024
+#define HCTR_LONG_BLOCKS 192
+#endif
+#ifndef HCTR_MED_BLOCKS
+#define HCTR_MED_BLOCKS 2048
 #endif
 #ifndef HCTR_ONLY_ROLE
-#define HCTR_ONLY_ROLE 0 // 1: long role only, 2: tile role only (timing experiments; results are incomplete)
+#define HCTR_ONLY_ROLE 0 // 1: long, 2: short, 3: medium role only (timing experiments; results are incomplete)
 #endif
-constexpr int kTileOcc = 32;
-constexpr int kPushBlock = 512;
-constexpr int kBatch = HCTR_TILE_BATCH;   // tile role: gradient rows in flight per group
-constexpr int kDepth = HCTR_DEPTH;        // long role: loads in flight per thread
-constexpr int kSlots = 4;                 // long role: LDS ring slots
+constexpr int kPushBlock = 512;  // long kernel
+constexpr int kSmallBlock = 256; // medium and short kernels
+constexpr int kBatch = HCTR_TILE_BATCH;   // short role: gradient rows in flight per group past the first two
+constexpr int kDepth = HCTR_DEPTH;        // long role: chunks in flight per loader thread
+constexpr int kRPT = HCTR_RPT;            // long role: rows per loader thread and chunk
+constexpr int kSlots = 3;                 // long role: LDS ring slots
 constexpr int kSlice = HCTR_SLICE;        // long role: columns per block
 constexpr int kLongBlocks = HCTR_LONG_BLOCKS;
+constexpr int kMedBlocks = HCTR_MED_BLOCKS;
 
-size_t push_tiles(uint32_t n_prev) { return (n_prev + kTileOcc - 1) / kTileOcc; }
 
 namespace {
 
@@ -120,182 +127,300 @@ __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const
   }
 }
 
-// ---- tile role -----------------------------------------------------------------------------------------
-template <int VEC, int LPR, typename K>
-__device__ __forceinline__ void tile_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
-                                          uint32_t block) {
+// ---- short role ----------------------------------------------------------------------------------------
+// A group of LPR lanes owns kRunsPerGroup consecutive unique ranks and sums every run among them that is not
+// long.  Everything the group needs first is requested before anything is waited for: the run bounds and
+// resident offsets, then the destination rows, the first two gradient-row indices of every run and those
+// gradient rows.  Nine runs out of ten are finished by that; longer ones continue eight rows at a time.
+#ifndef HCTR_RUNS_PER_GROUP
+#define HCTR_RUNS_PER_GROUP 4
+#endif
+constexpr int kRunsPerGroup = HCTR_RUNS_PER_GROUP;
+constexpr int kHead = 2; // occurrences per run fetched up front
+
+template <int VEC, int LPR, typename K, bool kSingle>
+__device__ __forceinline__ void short_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
+                                           uint32_t block, uint32_t U) {
   typedef typename Vec<VEC>::T V;
-  constexpr int kGroups = kPushBlock / LPR;
-  const uint32_t n = p.n, W = t.width;
-  const uint32_t tile = block * kGroups + threadIdx.x / LPR;
+  constexpr int G = kRunsPerGroup;
+  constexpr int kGroups = kSmallBlock / LPR;
+  const uint32_t W = t.width, n = p.n;
+  const uint32_t u0 = (block * kGroups + threadIdx.x / LPR) * G;
+  if (u0 >= U) return;
   const uint32_t gl = threadIdx.x % LPR;
-  const uint32_t j0 = tile * kTileOcc;
-  if (j0 >= n) return;
-  const uint32_t j1 = min(j0 + kTileOcc, n);
-  // a run that started before the tile belongs to the group of an earlier tile (or to the long role)
-  const uint32_t head = p.rank_sorted[j0];
-  const bool head_foreign = j0 > 0 && p.rank_sorted[j0 - 1] == head;
-  // the last run of the tile is finished past the tile end if it is short and continues
-  uint32_t je = j1;
-  {
-    const uint32_t ul = p.rank_sorted[j1 - 1];
-    if (!(ul & kLongFlag) && j1 < n && p.rank_sorted[j1] == ul && !(head_foreign && ul == head))
-      je = p.run_start[ul + 1];
-  }
+  const uint32_t *__restrict__ run_start = p.run_start;
+  const uint32_t *__restrict__ sorted_arg = p.sorted_arg;
+  const embed_t *__restrict__ grad = a.grad;
+  uint32_t rs[G + 1];
+  slot_t off[G];
+#pragma unroll
+  for (int i = 0; i <= G; i++) rs[i] = run_start[min(u0 + i, U)];
+#pragma unroll
+  for (int i = 0; i < G; i++) off[i] = p.uoff[min(u0 + i, U - 1)];
   const float neg_lr = t.neg_lr;
 
   for (uint32_t c0 = 0; c0 < W; c0 += LPR * VEC) {
     const uint32_t col = c0 + gl * VEC;
     const bool active = col < W;
-    V acc = Vec<VEC>::zero();
-    uint32_t cur_u = 0;
-    bool have = false;
-    for (uint32_t j = j0; j < je; j += kBatch) {
-      uint32_t su[kBatch], ru[kBatch];
-      bool use[kBatch];
-      V v[kBatch];
+    uint32_t len[G];
+    bool mine[G];
+    V e[G];
+    uint32_t si[G][kHead];
+    V v[G][kHead];
 #pragma unroll
-      for (int k = 0; k < kBatch; k++) {
-        const bool ok = j + k < je;
-        su[k] = ok ? p.sorted_arg[j + k] : 0u;
-        ru[k] = ok ? p.rank_sorted[j + k] : kLongFlag;
-      }
+    for (int i = 0; i < G; i++) {
+      len[i] = rs[i + 1] - rs[i];
+      mine[i] = u0 + i < U && len[i] <= kTinyRun && active;
+    }
+    if (kSingle) {
 #pragma unroll
-      for (int k = 0; k < kBatch; k++) {
-        use[k] = !(ru[k] & kLongFlag) && !(head_foreign && ru[k] == head);
-        v[k] = Vec<VEC>::zero();
-        if (use[k] && active) v[k] = *(const V *)(a.grad + (size_t)su[k] * W + col);
-      }
-#pragma unroll
-      for (int k = 0; k < kBatch; k++) {
-        if (!use[k]) continue;
-        if (have && ru[k] != cur_u) {
-          if (active) apply_row<VEC, K>(t, id_bits, p, a, cur_u, Vec<VEC>::scale(acc, neg_lr), col, c0 == 0 && gl == 0);
-          acc = Vec<VEC>::zero();
-        }
-        cur_u = ru[k];
-        have = true;
-        Vec<VEC>::add(acc, v[k]);
+      for (int i = 0; i < G; i++) {
+        e[i] = Vec<VEC>::zero();
+        if (mine[i]) e[i] = *(const V *)(t.emb + (size_t)off[i] * W + col);
       }
     }
-    if (have && active) apply_row<VEC, K>(t, id_bits, p, a, cur_u, Vec<VEC>::scale(acc, neg_lr), col, c0 == 0 && gl == 0);
+#pragma unroll
+    for (int i = 0; i < G; i++)
+#pragma unroll
+      for (int k = 0; k < kHead; k++) si[i][k] = sorted_arg[min(rs[i] + k, n - 1)];
+#pragma unroll
+    for (int i = 0; i < G; i++)
+#pragma unroll
+      for (int k = 0; k < kHead; k++) {
+        v[i][k] = Vec<VEC>::zero();
+        if (mine[i] && (uint32_t)k < len[i]) v[i][k] = *(const V *)(grad + (size_t)si[i][k] * W + col);
+      }
+    V acc[G];
+#pragma unroll
+    for (int i = 0; i < G; i++) { // heads of all runs first: their registers are free before the tails start
+      acc[i] = Vec<VEC>::zero();  // the reference starts every sum from 0
+#pragma unroll
+      for (int k = 0; k < kHead; k++)
+        if (mine[i] && (uint32_t)k < len[i]) Vec<VEC>::add(acc[i], v[i][k]);
+    }
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+      if (!mine[i]) continue;
+      if (len[i] > kHead) { // the rest of the run (at most kTinyRun - kHead rows), in order
+        constexpr int kTail = kTinyRun - kHead;
+        uint32_t sj[kTail];
+        V x[kTail];
+        const uint32_t j = rs[i] + kHead;
+#pragma unroll
+        for (int k = 0; k < kTail; k++) sj[k] = sorted_arg[min(j + k, rs[i + 1] - 1)];
+#pragma unroll
+        for (int k = 0; k < kTail; k++) x[k] = *(const V *)(grad + (size_t)sj[k] * W + col);
+#pragma unroll
+        for (int k = 0; k < kTail; k++)
+          if (j + k < rs[i + 1]) Vec<VEC>::add(acc[i], x[k]);
+      }
+      const V scaled = Vec<VEC>::scale(acc[i], neg_lr);
+      if (kSingle) {
+        V r = e[i];
+        Vec<VEC>::add(r, scaled);
+        *(V *)(t.emb + (size_t)off[i] * W + col) = r;
+        if (c0 == 0 && gl == 0) t.ver[off[i]] += (version_t)len[i];
+      } else {
+        apply_row<VEC, K>(t, id_bits, p, a, u0 + i, scaled, col, c0 == 0 && gl == 0);
+      }
+    }
+  }
+}
+
+// ---- medium role ---------------------------------------------------------------------------------------
+// Runs between kTinyRun and kLongRun occurrences: one group of LPR lanes per run of the list (groups stride
+// over it).  The group first copies the run's gradient-row indices into LDS with one coalesced load, so that no
+// later load waits for an index; then two batches of kBatch gradient rows are kept in flight while the rows are
+// added in order.
+template <int VEC, int LPR, typename K, bool kSingle>
+__device__ __forceinline__ void medium_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
+                                            uint32_t *lds_idx) {
+  typedef typename Vec<VEC>::T V;
+  constexpr int kGroups = kSmallBlock / LPR;
+  const uint32_t W = t.width;
+  const uint32_t gl = threadIdx.x % LPR;
+  uint32_t *my_idx = lds_idx + (threadIdx.x / LPR) * kLongRun; // this group's slice of the index staging area
+  const uint32_t n_med = p.d_nlong[kMedCount];
+  const uint32_t *__restrict__ sorted_arg = p.sorted_arg;
+  const embed_t *__restrict__ grad = a.grad;
+  const float neg_lr = t.neg_lr;
+  for (uint32_t item = blockIdx.x * kGroups + threadIdx.x / LPR; item < n_med; item += gridDim.x * kGroups) {
+    const uint32_t u = p.med_list[item];
+    const uint32_t lo = p.run_start[u], hi = p.run_start[u + 1];
+    const uint32_t len = hi - lo; // <= kLongRun
+    const slot_t off = p.uoff[u];
+    for (uint32_t q = gl; q < len; q += LPR) my_idx[q] = sorted_arg[lo + q];
+    // a group never spans waves: the LDS writes above are ordered before the reads below in hardware; the
+    // fence keeps the compiler from moving them
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (uint32_t c0 = 0; c0 < W; c0 += LPR * VEC) {
+      const uint32_t col = c0 + gl * VEC;
+      const bool active = col < W;
+      const embed_t *gcol = grad + (active ? col : 0);
+      V e = Vec<VEC>::zero();
+      if (kSingle && active) e = *(const V *)(t.emb + (size_t)off * W + col);
+      V acc = Vec<VEC>::zero();
+      V xa[kBatch], xb[kBatch];
+      auto fetch = [&](V(&x)[kBatch], uint32_t q0) { // rows q0 .. q0+kBatch-1 of the run (clamped to its end)
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) x[k] = *(const V *)(gcol + (size_t)my_idx[min(q0 + k, len - 1)] * W);
+      };
+      auto add = [&](const V(&x)[kBatch], uint32_t q0) {
+#pragma unroll
+        for (int k = 0; k < kBatch; k++)
+          if (q0 + k < len) Vec<VEC>::add(acc, x[k]);
+      };
+      fetch(xa, 0);
+      for (uint32_t q = 0; q < len; q += 2 * kBatch) {
+        if (q + kBatch < len) fetch(xb, q + kBatch);
+        add(xa, q);
+        if (q + 2 * kBatch < len) fetch(xa, q + 2 * kBatch);
+        if (q + kBatch < len) add(xb, q + kBatch);
+      }
+      if (!active) continue;
+      const V scaled = Vec<VEC>::scale(acc, neg_lr);
+      if (kSingle) {
+        Vec<VEC>::add(e, scaled);
+        *(V *)(t.emb + (size_t)off * W + col) = e;
+        if (c0 == 0 && gl == 0) t.ver[off] += (version_t)len;
+      } else {
+        apply_row<VEC, K>(t, id_bits, p, a, u, scaled, col, c0 == 0 && gl == 0);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier(); // the staging area is rewritten for the next run
   }
 }
 
 // ---- long role -----------------------------------------------------------------------------------------
-// Work item = (long run, column slice of CS columns).  Wave 0 of the block only sums; the other 7 waves
-// ("loaders") only move gradient rows global -> registers -> LDS ring.  A row slice is read by CS/VEC loader
-// lanes, so one block-wide load covers RPL = 448 / (CS/VEC) consecutive occurrences ("chunk").
-// Loaders and the summing wave meet at one barrier per chunk: barrier m says "chunk m is in LDS".
+// Work item = (long run, column slice of CS columns), handed out longest class first through a counter.
+// Wave 0 of the block only sums; the other 7 waves ("loaders") only move gradient rows global -> registers ->
+// LDS ring.  A row slice is read by CS/VEC loader lanes; one block-wide load covers RPL = 448 / (CS/VEC)
+// consecutive occurrences and a chunk is kRPT such loads.  Loaders and the summing wave meet at one barrier
+// per chunk: barrier m says "chunk m is in LDS".  A slot is overwritten kSlots barriers later, after the
+// summing wave has passed the barrier that follows its reads.
 constexpr int kLoaders = kPushBlock - kWave;
 
 template <int VEC, typename K, int CSC> // CSC: columns per slice if known at compile time (64), else 0
 __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
-                                          uint32_t first_item, float *lds) {
+                                          float *lds, uint32_t *next_item) {
   typedef typename Vec<VEC>::T V;
   const uint32_t W = t.width;
   const uint32_t CS = CSC ? (uint32_t)CSC : min((uint32_t)kSlice, (W + VEC - 1) / VEC * VEC);
   uint32_t lanes = (CS + VEC - 1) / VEC; // loader lanes per row slice, rounded up to a power of two
   lanes = lanes <= 1 ? 1 : lanes <= 2 ? 2 : lanes <= 4 ? 4 : lanes <= 8 ? 8 : lanes <= 16 ? 16 : lanes <= 32 ? 32 : 64;
   const uint32_t RPL = CSC ? (uint32_t)(kLoaders / (CSC / VEC)) : kLoaders / lanes;
-  constexpr int kRows = CSC ? kLoaders / (CSC / VEC) : 1; // RPL as a constant on the fast path
+  const uint32_t CR = RPL * kRPT;                                   // rows per chunk
+  constexpr int kChunkRows = CSC ? kRPT * (kLoaders / (CSC / VEC)) : 1; // CR as a constant on the fast path
   const uint32_t slices = (W + CS - 1) / CS;
-  const uint32_t slot_floats = RPL * CS;
-  const uint32_t items = *p.d_nlong * slices;
+  const uint32_t slot_floats = CR * CS;
   const float neg_lr = t.neg_lr;
   const bool summer = threadIdx.x < kWave;
   const uint32_t lt = threadIdx.x - kWave; // loader thread number (meaningless on the summing wave)
   const uint32_t my_row = lt / lanes, my_lane = lt % lanes;
+  uint32_t class_end[kLongBuckets]; // items up to and including each length class
+  {
+    uint32_t run = 0;
+#pragma unroll
+    for (int c = 0; c < kLongBuckets; c++) {
+      run += p.d_nlong[c] * slices;
+      class_end[c] = run;
+    }
+  }
+  const uint32_t items = class_end[kLongBuckets - 1];
 
-  for (uint32_t item = first_item; item < items; item += kLongBlocks) {
-    const uint32_t u = p.long_list[item / slices];
-    const uint32_t slice = item % slices;
+  for (;;) {
+    if (threadIdx.x == 0) *next_item = atomicAdd(&p.d_nlong[kLongWork], 1u);
+    __syncthreads();
+    const uint32_t item = *next_item;
+    __syncthreads();
+    if (item >= items) break;
+    int cls = 0;
+    uint32_t first = 0;
+#pragma unroll
+    for (int c = 0; c < kLongBuckets - 1; c++)
+      if (item >= class_end[c]) {
+        cls = c + 1;
+        first = class_end[c];
+      }
+    const uint32_t u = p.long_list[(size_t)cls * p.long_cap + (item - first) / slices];
+    const uint32_t slice = (item - first) % slices;
     const uint32_t lo = p.run_start[u], hi = p.run_start[u + 1];
     const uint32_t L = hi - lo;
-    const uint32_t nchunks = (L + RPL - 1) / RPL;
+    const uint32_t nchunks = (L + CR - 1) / CR;
     if (!summer) {
       // ---------------- loaders ----------------
       const uint32_t lcol = my_lane * VEC; // column inside the slice
       const uint32_t col = slice * CS + lcol;
       const bool in_slice = lcol < CS && my_row < RPL;
-      // Loads are unconditional and branch-free so that kDepth of them stay in flight per thread: positions
+      // Loads are unconditional and branch-free so that kDepth chunks stay in flight per thread: positions
       // past the end of the run re-read its last row (never summed), lanes outside the slice read column 0.
       const embed_t *gbase = a.grad + ((in_slice && col < W) ? col : 0);
-      auto row_index = [&](uint32_t c) -> uint32_t { return p.sorted_arg[min(lo + c * RPL + my_row, hi - 1)]; };
+      auto row_index = [&](uint32_t c, int q) -> uint32_t {
+        return p.sorted_arg[min(lo + c * CR + q * RPL + my_row, hi - 1)];
+      };
       auto row_load = [&](uint32_t idx) -> V { return *(const V *)(gbase + (size_t)idx * W); };
-      uint32_t idx_a[kDepth], idx_b[kDepth];
-      V val[kDepth];
+      uint32_t idx_a[kDepth][kRPT], idx_b[kDepth][kRPT];
+      V val[kDepth][kRPT];
 #pragma unroll
-      for (int k = 0; k < kDepth; k++) idx_a[k] = row_index(k);
+      for (int k = 0; k < kDepth; k++)
 #pragma unroll
-      for (int k = 0; k < kDepth; k++) idx_b[k] = row_index(kDepth + k);
+        for (int q = 0; q < kRPT; q++) idx_a[k][q] = row_index(k, q);
 #pragma unroll
-      for (int k = 0; k < kDepth; k++) val[k] = row_load(idx_a[k]);
-      // invariant at the top of a round: val[k] holds chunk c0+k, idx_b[k] the row index of chunk c0+kDepth+k
+      for (int k = 0; k < kDepth; k++)
+#pragma unroll
+        for (int q = 0; q < kRPT; q++) idx_b[k][q] = row_index(kDepth + k, q);
+#pragma unroll
+      for (int k = 0; k < kDepth; k++)
+#pragma unroll
+        for (int q = 0; q < kRPT; q++) val[k][q] = row_load(idx_a[k][q]);
+      // invariant at the top of a round: val[k] holds chunk c0+k, idx_b[k] the row indices of chunk c0+kDepth+k
       for (uint32_t c0 = 0; c0 < nchunks; c0 += kDepth) {
 #pragma unroll
-        for (int k = 0; k < kDepth; k++) idx_a[k] = idx_b[k];
+        for (int k = 0; k < kDepth; k++)
 #pragma unroll
-        for (int k = 0; k < kDepth; k++) idx_b[k] = row_index(c0 + 2 * kDepth + k);
+          for (int q = 0; q < kRPT; q++) idx_a[k][q] = idx_b[k][q];
+#pragma unroll
+        for (int k = 0; k < kDepth; k++)
+#pragma unroll
+          for (int q = 0; q < kRPT; q++) idx_b[k][q] = row_index(c0 + 2 * kDepth + k, q);
 #pragma unroll
         for (int k = 0; k < kDepth; k++) {
           const uint32_t c = c0 + k;
           if (c < nchunks) { // uniform over the block: the summing wave makes the same number of barriers
             float *slot = lds + (c % kSlots) * slot_floats;
-            if (in_slice) *(V *)(slot + my_row * CS + lcol) = val[k];
-            val[k] = row_load(idx_a[k]); // chunk c + kDepth
-            __syncthreads();             // barrier c
+#pragma unroll
+            for (int q = 0; q < kRPT; q++) {
+              if (in_slice) *(V *)(slot + (q * RPL + my_row) * CS + lcol) = val[k][q];
+              val[k][q] = row_load(idx_a[k][q]); // chunk c + kDepth
+            }
+            __syncthreads(); // barrier c
           }
         }
       }
     } else {
       // ---------------- summing wave: one column per lane, rows strictly in order ----------------
       float acc = 0.f;
-      const uint32_t nfull = L / RPL; // chunks with all RPL rows
+      const uint32_t nfull = L / CR; // chunks with all CR rows
       uint32_t c = 0;
       if (CSC) {
-        // software pipeline: the LDS reads of chunk c+1 are issued before the adds of chunk c
-        float xa[kRows], xb[kRows];
-        if (nfull > 0) {
-          __syncthreads(); // barrier 0
-          const float *sp = lds + threadIdx.x;
+        for (; c < nfull; c++) {
+          __syncthreads(); // barrier c
+          const float *sp = lds + (c % kSlots) * slot_floats + threadIdx.x;
+          float x[kChunkRows];
 #pragma unroll
-          for (int q = 0; q < kRows; q++) xa[q] = sp[q * CSC];
-          for (c = 1; c + 1 < nfull; c += 2) {
-            __syncthreads(); // barrier c
-            const float *s1 = lds + (c % kSlots) * slot_floats + threadIdx.x;
+          for (int q = 0; q < kChunkRows; q++) x[q] = sp[q * CSC];
 #pragma unroll
-            for (int q = 0; q < kRows; q++) xb[q] = s1[q * CSC];
-#pragma unroll
-            for (int q = 0; q < kRows; q++) acc += xa[q];
-            __syncthreads(); // barrier c + 1
-            const float *s2 = lds + ((c + 1) % kSlots) * slot_floats + threadIdx.x;
-#pragma unroll
-            for (int q = 0; q < kRows; q++) xa[q] = s2[q * CSC];
-#pragma unroll
-            for (int q = 0; q < kRows; q++) acc += xb[q];
-          }
-          if (c < nfull) { // one more full chunk
-            __syncthreads(); // barrier c
-            const float *s1 = lds + (c % kSlots) * slot_floats + threadIdx.x;
-#pragma unroll
-            for (int q = 0; q < kRows; q++) xb[q] = s1[q * CSC];
-#pragma unroll
-            for (int q = 0; q < kRows; q++) acc += xa[q];
-#pragma unroll
-            for (int q = 0; q < kRows; q++) acc += xb[q];
-            c++;
-          } else {
-#pragma unroll
-            for (int q = 0; q < kRows; q++) acc += xa[q];
-          }
+          for (int q = 0; q < kChunkRows; q++) acc += x[q];
         }
       }
       for (; c < nchunks; c++) { // generic path, and the partial last chunk of the fast path
         __syncthreads();         // barrier c
         if (threadIdx.x < CS) {
           const float *col_ptr = lds + (c % kSlots) * slot_floats + threadIdx.x;
-          const uint32_t rows = min(RPL, L - c * RPL);
+          const uint32_t rows = min(CR, L - c * CR);
           uint32_t r = 0;
           for (; r + 8 <= rows; r += 8) {
             float x[8];
@@ -310,54 +435,87 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       if (threadIdx.x < CS && slice * CS + threadIdx.x < W)
         apply_row<1, K>(t, id_bits, p, a, u, acc * neg_lr, slice * CS + threadIdx.x, slice == 0 && threadIdx.x == 0);
     }
-    __syncthreads(); // the ring is reused by the next item
   }
-}
-
-template <int VEC, int LPR, typename K>
-__global__ __launch_bounds__(kPushBlock) void segment_sum_apply(TableView t, int id_bits, BatchView p, PushArgs a) {
-  __shared__ __align__(16) float lds[kSlots * kPushBlock * VEC];
-  if (blockIdx.x < kLongBlocks) {
-    if (HCTR_ONLY_ROLE != 2) {
-      if (VEC == 4 && t.width % 64 == 0) long_role<VEC, K, (VEC == 4 ? 64 : 0)>(t, id_bits, p, a, blockIdx.x, lds);
-      else long_role<VEC, K, 0>(t, id_bits, p, a, blockIdx.x, lds);
-    }
-  } else {
-    if (HCTR_ONLY_ROLE != 1) tile_role<VEC, LPR, K>(t, id_bits, p, a, blockIdx.x - kLongBlocks);
-  }
-}
-
-template <int VEC, int LPR, typename K>
-void launch_push_t(hipStream_t s, const TableView &t, int id_bits, const BatchView &p, const PushArgs &a) {
-  constexpr int kGroups = kPushBlock / LPR;
-  const unsigned tiles = (unsigned)push_tiles(p.n);
-  hipLaunchKernelGGL((segment_sum_apply<VEC, LPR, K>), dim3(kLongBlocks + div_up(tiles, kGroups)), dim3(kPushBlock),
-                     0, s, t, id_bits, p, a);
 }
 
 template <int VEC, typename K>
-void launch_push_v(hipStream_t s, const TableView &t, int id_bits, const BatchView &p, const PushArgs &a) {
+__global__ __launch_bounds__(kPushBlock) void push_long(TableView t, int id_bits, BatchView p, PushArgs a) {
+  __shared__ __align__(16) float lds[kSlots * kRPT * kPushBlock * VEC];
+  __shared__ uint32_t next_item;
+  if (VEC == 4 && t.width % kSlice == 0) long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, &next_item);
+  else long_role<VEC, K, 0>(t, id_bits, p, a, lds, &next_item);
+}
+
+template <int VEC, int LPR, typename K, bool kSingle>
+__global__ __launch_bounds__(kSmallBlock) void push_medium(TableView t, int id_bits, BatchView p, PushArgs a) {
+  __shared__ uint32_t lds_idx[(kSmallBlock / LPR) * kLongRun];
+  medium_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, lds_idx);
+}
+
+template <int VEC, int LPR, typename K, bool kSingle>
+__global__ __launch_bounds__(kSmallBlock) void push_short(TableView t, int id_bits, BatchView p, PushArgs a, uint32_t U) {
+  short_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, blockIdx.x, U);
+}
+
+template <int VEC, int LPR, typename K, bool kSingle>
+void launch_push_t(const PushStreams &ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
+                   const PushArgs &a) {
+  constexpr int kGroups = kSmallBlock / LPR;
+  // the long chains are the critical path: they go first, on the main stream; the other two overlap with them
+  if (HCTR_ONLY_ROLE == 0 || HCTR_ONLY_ROLE == 1)
+    hipLaunchKernelGGL((push_long<VEC, K>), dim3(kLongBlocks), dim3(kPushBlock), 0, ps.main, t, id_bits, p, a);
+  if (HCTR_ONLY_ROLE == 0 || HCTR_ONLY_ROLE == 2)
+    hipLaunchKernelGGL((push_short<VEC, LPR, K, kSingle>), dim3(div_up(U, kGroups * kRunsPerGroup)), dim3(kSmallBlock),
+                       0, ps.aux1, t, id_bits, p, a, U);
+  if (HCTR_ONLY_ROLE == 0 || HCTR_ONLY_ROLE == 3)
+    hipLaunchKernelGGL((push_medium<VEC, LPR, K, kSingle>), dim3(kMedBlocks), dim3(kSmallBlock), 0, ps.aux2, t, id_bits,
+                       p, a);
+}
+
+template <int VEC, typename K, bool kSingle>
+void launch_push_v(const PushStreams &ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
+                   const PushArgs &a) {
   const uint32_t lanes = (t.width + VEC - 1) / VEC;
-  if (lanes <= 4) launch_push_t<VEC, 4, K>(s, t, id_bits, p, a);
-  else if (lanes <= 8) launch_push_t<VEC, 8, K>(s, t, id_bits, p, a);
-  else if (lanes <= 16) launch_push_t<VEC, 16, K>(s, t, id_bits, p, a);
-  else if (lanes <= 32) launch_push_t<VEC, 32, K>(s, t, id_bits, p, a);
-  else launch_push_t<VEC, 64, K>(s, t, id_bits, p, a);
+  if (lanes <= 4) launch_push_t<VEC, 4, K, kSingle>(ps, t, id_bits, p, U, a);
+  else if (lanes <= 8) launch_push_t<VEC, 8, K, kSingle>(ps, t, id_bits, p, U, a);
+  else if (lanes <= 16) launch_push_t<VEC, 16, K, kSingle>(ps, t, id_bits, p, U, a);
+  else if (lanes <= 32) launch_push_t<VEC, 32, K, kSingle>(ps, t, id_bits, p, U, a);
+  else launch_push_t<VEC, 64, K, kSingle>(ps, t, id_bits, p, U, a);
+}
+
+template <int VEC, typename K>
+void launch_push_k(const PushStreams &ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
+                   const PushArgs &a) {
+  if (t.nrank == 1) launch_push_v<VEC, K, true>(ps, t, id_bits, p, U, a);
+  else launch_push_v<VEC, K, false>(ps, t, id_bits, p, U, a);
 }
 
 } // namespace
 
-void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &prev, const PushArgs &a) {
-  if (!prev.n) return;
+void launch_push(const PushStreams &ps, const TableView &t, const KeyLayout &kl, const BatchView &prev,
+                 uint32_t n_unique, const PushArgs &a) {
+  if (!prev.n || !n_unique) return;
+  // fork: the two auxiliary streams start after everything queued on the main stream so far (nothing is, when
+  // the caller knows the main stream to be idle)
+  if (!ps.main_idle) {
+    HCTR_HIP(hipEventRecord(ps.fork, ps.main));
+    HCTR_HIP(hipStreamWaitEvent(ps.aux1, ps.fork, 0));
+    HCTR_HIP(hipStreamWaitEvent(ps.aux2, ps.fork, 0));
+  }
   const bool vec4 = t.width % 4 == 0 && ((uintptr_t)a.grad % 16) == 0;
   if (vec4) {
-    if (kl.wide) launch_push_v<4, uint64_t>(s, t, kl.id_bits, prev, a);
-    else launch_push_v<4, uint32_t>(s, t, kl.id_bits, prev, a);
+    if (kl.wide) launch_push_k<4, uint64_t>(ps, t, kl.id_bits, prev, n_unique, a);
+    else launch_push_k<4, uint32_t>(ps, t, kl.id_bits, prev, n_unique, a);
   } else {
-    if (kl.wide) launch_push_v<1, uint64_t>(s, t, kl.id_bits, prev, a);
-    else launch_push_v<1, uint32_t>(s, t, kl.id_bits, prev, a);
+    if (kl.wide) launch_push_k<1, uint64_t>(ps, t, kl.id_bits, prev, n_unique, a);
+    else launch_push_k<1, uint32_t>(ps, t, kl.id_bits, prev, n_unique, a);
   }
   HCTR_HIP(hipGetLastError());
+  // join: the main stream continues when all three kernels are done
+  HCTR_HIP(hipEventRecord(ps.join1, ps.aux1));
+  HCTR_HIP(hipEventRecord(ps.join2, ps.aux2));
+  HCTR_HIP(hipStreamWaitEvent(ps.main, ps.join1, 0));
+  HCTR_HIP(hipStreamWaitEvent(ps.main, ps.join2, 0));
 }
 
 } // namespace hctr

@@ -52,7 +52,7 @@ struct Batch {
   uint32_t n = 0;   // keys
   uint32_t U = 0;   // unique keys (host copy, valid after the preprocess call returned)
   bool idx_map_valid = false;
-  DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong;
+  DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong, med_list;
   std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
   std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
   void reserve(uint32_t n_keys, int nrank, bool wide);
@@ -147,11 +147,14 @@ class Group {
   const std::string key;
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  PushStreams push_streams{};
   std::vector<Shard *> members;
   DeviceBuf desc_dev;
   CopyDesc *desc_host = nullptr;
   size_t desc_cap = 0;
   double wait_seconds = 120.0;
+  bool stream_idle = false; // true between a completed call and the next work queued on `stream`
+  void sync_stream();
 
   // per-stage device time, accumulated over calls while stage_timing is on
   bool stage_timing = false;

@@ -38,8 +38,9 @@ void Batch::reserve(uint32_t n_keys, int nrank, bool wide) {
   uoff.reserve(n * sizeof(slot_t));
   bucket_lo.reserve((size_t)(nrank + 1) * 4);
   dU.reserve(4);
-  long_list.reserve(long_list_capacity((uint32_t)n) * 4);
-  dnlong.reserve(4);
+  long_list.reserve(long_list_capacity((uint32_t)n) * 4 * kLongBuckets);
+  dnlong.reserve(4 * kRunCounters);
+  med_list.reserve(med_list_capacity((uint32_t)n) * 4);
 }
 
 BatchView Batch::view() const {
@@ -56,6 +57,8 @@ BatchView Batch::view() const {
   v.d_U = dU.as<uint32_t>();
   v.long_list = long_list.as<uint32_t>();
   v.d_nlong = dnlong.as<uint32_t>();
+  v.long_cap = (uint32_t)long_list_capacity(std::max<uint32_t>(n, 1));
+  v.med_list = med_list.as<uint32_t>();
   return v;
 }
 
@@ -136,7 +139,7 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   for (Batch *b : {&cur, &prev}) {
     b->reserve(1, c.nrank, kl.wide);
     HCTR_HIP(hipMemsetAsync(b->dU.p, 0, 4, s));
-    HCTR_HIP(hipMemsetAsync(b->dnlong.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(b->dnlong.p, 0, 4 * kRunCounters, s));
     HCTR_HIP(hipMemsetAsync(b->bucket_lo.p, 0, b->bucket_lo.bytes, s));
     HCTR_HIP(hipMemsetAsync(b->run_start.p, 0, 4, s));
     b->send_cnt.assign(c.nrank + 1, 0);
@@ -199,7 +202,7 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
     HCTR_HIP(hipMemsetAsync(cur.dU.p, 0, 4, s));
     HCTR_HIP(hipMemsetAsync(cur.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
     HCTR_HIP(hipMemsetAsync(cur.run_start.p, 0, 4, s));
-    HCTR_HIP(hipMemsetAsync(cur.dnlong.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(cur.dnlong.p, 0, 4 * kRunCounters, s));
   } else {
     reserve_batch_scratch(cur.n);
     {
@@ -238,7 +241,7 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
     delete sort_scope;
     StageScope st(*group, S_UNIQUE);
     launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>(), &dst_->U);
-    launch_mark_long_runs(s, cur.view());
+    launch_list_long_runs(s, cur.view());
   }
   if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt);
 }
@@ -296,7 +299,7 @@ void Shard::generate_gradient(const float *grad) {
     prev.n = 0;
     prev.U = 0;
     HCTR_HIP(hipMemsetAsync(prev.dU.p, 0, 4, s));
-    HCTR_HIP(hipMemsetAsync(prev.dnlong.p, 0, 4, s));
+    HCTR_HIP(hipMemsetAsync(prev.dnlong.p, 0, 4 * kRunCounters, s));
     HCTR_HIP(hipMemsetAsync(prev.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
     std::fill(prev.push_cnt.begin(), prev.push_cnt.end(), 0);
     std::fill(prev.pushrecv_cnt.begin(), prev.pushrecv_cnt.end(), 0);
@@ -326,7 +329,10 @@ void Shard::generate_gradient(const float *grad) {
     a.g_val = g_val.as<embed_t>();
   }
   StageScope st(*group, S_PUSH);
-  launch_push(s, tv, kl, prev.view(), a);
+  PushStreams ps = group->push_streams;
+  ps.main_idle = group->stream_idle && !group->stage_timing;
+  launch_push(ps, tv, kl, prev.view(), prev.U, a);
+  group->stream_idle = false;
 }
 
 // csrc/core/generate_query.cu:91-106
@@ -531,6 +537,12 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   HCTR_HIP(hipStreamCreate(&stream));
   HCTR_HIP(hipEventCreate(&ev0));
   HCTR_HIP(hipEventCreate(&ev1));
+  push_streams.main = stream;
+  HCTR_HIP(hipStreamCreateWithFlags(&push_streams.aux1, hipStreamNonBlocking));
+  HCTR_HIP(hipStreamCreateWithFlags(&push_streams.aux2, hipStreamNonBlocking));
+  HCTR_HIP(hipEventCreateWithFlags(&push_streams.fork, hipEventDisableTiming));
+  HCTR_HIP(hipEventCreateWithFlags(&push_streams.join1, hipEventDisableTiming));
+  HCTR_HIP(hipEventCreateWithFlags(&push_streams.join2, hipEventDisableTiming));
   a_keys_.resize(nr);
   a_n_.resize(nr);
   a_grad_.resize(nr);
@@ -544,6 +556,11 @@ Group::~Group() {
   if (ev1) (void)hipEventDestroy(ev1);
   for (auto &m : marks) { (void)hipEventDestroy(m.a); (void)hipEventDestroy(m.b); }
   for (auto e : event_pool) (void)hipEventDestroy(e);
+  if (push_streams.fork) (void)hipEventDestroy(push_streams.fork);
+  if (push_streams.join1) (void)hipEventDestroy(push_streams.join1);
+  if (push_streams.join2) (void)hipEventDestroy(push_streams.join2);
+  if (push_streams.aux1) (void)hipStreamDestroy(push_streams.aux1);
+  if (push_streams.aux2) (void)hipStreamDestroy(push_streams.aux2);
   if (stream) (void)hipStreamDestroy(stream);
 }
 
@@ -685,9 +702,20 @@ void Group::exchange_return() {
 }
 
 // csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
+// Waits for the stream by polling: the calls are short and a blocking wait adds tens of microseconds of
+// wake-up latency to each of them.
+void Group::sync_stream() {
+  hipError_t e;
+  while ((e = hipStreamQuery(stream)) == hipErrorNotReady) {
+  }
+  HCTR_HIP(e);
+  stream_idle = true;
+}
+
 void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
+  stream_idle = false;
   HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) {
     m->swap_batches();
@@ -696,7 +724,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     m->enqueue_readback_preprocess();
   }
   HCTR_HIP(hipEventRecord(ev1, stream));
-  HCTR_HIP(hipStreamSynchronize(stream));
+  sync_stream();
   float ms = 0.f;
   HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
   collect_marks();
@@ -722,6 +750,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
 void Group::push_pull_all(const float *const *grads, float *const *dsts) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
+  if (stage_timing || nrank > 1) stream_idle = false; // an event record or another shard's work precedes the push
   HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) {
     m->generate_gradient(grads[m->cfg.rank]);
@@ -731,14 +760,15 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
     exchange_query();
     for (Shard *m : members) m->handle_gradient();
     for (Shard *m : members) m->handle_query();
-    HCTR_HIP(hipStreamSynchronize(stream)); // hetu_gpu_table.cu:33: the return counts size the next exchange
+    sync_stream(); // hetu_gpu_table.cu:33: the return counts size the next exchange
+    stream_idle = false;
     collect_marks();
     for (Shard *m : members) m->finish_handle_query();
     exchange_return();
   }
   for (Shard *m : members) m->write_back(dsts[m->cfg.rank]);
   HCTR_HIP(hipEventRecord(ev1, stream));
-  HCTR_HIP(hipStreamSynchronize(stream));
+  sync_stream();
   float ms = 0.f;
   HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
   collect_marks();
