@@ -70,7 +70,7 @@ def build_pymod(force=False, verbose=True):
     src = os.path.join(CSRC, "pybind_module.cpp")
     if not os.path.exists(src):
         return None
-    deps = [src, os.path.join(HERE, "..", "include", "hetuctr_hip.h"), os.path.join(CSRC, "thread_pool.h")]
+    deps = [src, os.path.join(HERE, "..", "include", "hetuctr_hip.h")]
     if force or not _newer(PYMOD, deps):
         import pybind11
         inc = ["-I" + sysconfig.get_paths()["include"], "-I" + pybind11.get_include(), "-I" + os.path.join(HERE, "..", "include")]
