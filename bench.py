@@ -115,8 +115,7 @@ def main():
             uniq[i] = int(table.fetch(capi.SIZES)[1])
             table.push_pull(grad.data_ptr(), dst.data_ptr())
     w0 = max(a.warmup, 1) + len(dkeys)
-    if not a.no_stage_timing:
-        table.stage_timing(True)
+    # ---- timed region: K full steps, nothing else on the GPU
     pre_ms = pp_ms = 0.0
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -127,8 +126,20 @@ def main():
         pp_ms += q
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    stages = table.stage_times() if not a.no_stage_timing else {}
-    table.stage_timing(False)
+    # ---- same K steps again with every stage bracketed by HIP events on the table's stream (the events cost a
+    # few microseconds per stage, so the throughput above is taken without them)
+    stages = {}
+    ms_step_ev = None
+    if not a.no_stage_timing:
+        table.stage_timing(True)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(a.steps):
+            step(w0 + a.steps + i)
+        torch.cuda.synchronize()
+        ms_step_ev = 1e3 * (time.perf_counter() - t1) / a.steps
+        stages = table.stage_times()
+        table.stage_timing(False)
 
     ms_step = 1e3 * dt / a.steps
     # distinct keys of the batches the timed steps used (current batch = pulled, previous = pushed)
@@ -137,15 +148,22 @@ def main():
     bytes_step = workloads.algorithmic_bytes(n, 0.5 * (u_cur + u_prev), width)
     step_gbs = bytes_step / (ms_step * 1e-3) / 1e9
 
-    roof = None
-    if stages:
-        wide = {k: v for k, v in stages.items() if k in ("segment_sum_apply", "gather") and v[1] > 0}
-        dom = max(wide, key=lambda k: wide[k][0])
-        avg_ms = wide[dom][0] / wide[dom][1]
-        b = workloads.stage_bytes(dom, n, u_cur, n, u_prev, width)
-        roof = dict(bound="hbm", kernel=dom, achieved=b / (avg_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=b / (avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, traffic=None, avg_ms=avg_ms,
-                    algorithmic_bytes=int(b))
+    # HBM traffic per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (committed
+    # under profiles/, scaled by what the counters read for a plain copy of known size)
+    traffic = {}
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath) and a.scale == 1.0:
+        traffic = json.load(open(tpath)).get(a.config, {})
+    kernel_names = {"segment_sum_apply": "push_long + push_short + push_medium (concurrent, one stage)", "gather": "gather"}
+    roof_all = {}
+    for k, (tot, cnt) in stages.items():
+        if k in kernel_names and cnt > 0:
+            avg_ms = tot / cnt
+            b = workloads.stage_bytes(k, n, u_cur, n, u_prev, width)
+            gbs = b / (avg_ms * 1e-3) / 1e9
+            roof_all[k] = dict(bound="hbm", kernel=kernel_names[k], achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s",
+                               frac=gbs / HBM_PEAK_GBS, traffic=traffic.get(k), avg_ms=avg_ms, algorithmic_bytes=int(b))
+    roof = roof_all[max(roof_all, key=lambda k: roof_all[k]["avg_ms"])] if roof_all else None
 
     out = {
         "metric": "sparse IDs/sec per train step (pull+push)", "value": n * a.steps / dt, "unit": "IDs/s",
@@ -160,7 +178,9 @@ def main():
         "device_ms_per_step": {"preprocess": pre_ms / a.steps, "push_pull": pp_ms / a.steps},
         "step_hbm": {"algorithmic_bytes": int(bytes_step), "achieved_GBps": step_gbs, "frac": step_gbs / HBM_PEAK_GBS},
         "stage_ms": {k: v[0] / max(v[1], 1) for k, v in stages.items() if v[1]},
+        "ms_per_step_with_stage_events": ms_step_ev,
         "roofline": roof,
+        "roofline_stages": roof_all,
     }
     if not a.no_cpu:
         del dst
