@@ -119,7 +119,13 @@ __global__ __launch_bounds__(kBlock) void refresh(TableView t, int id_bits_unuse
 // Gather in SORTED order: one group per kRows consecutive sorted positions.  Duplicates of a key are adjacent,
 // so a table row is fetched from HBM once and re-read from cache for its other occurrences; every output row is
 // written whole, once, with non-temporal stores, at the batch position sorted_arg names.
-constexpr int kRows = 4;
+#ifndef HCTR_GATHER_ROWS
+#define HCTR_GATHER_ROWS 8
+#endif
+#ifndef HCTR_GATHER_NT
+#define HCTR_GATHER_NT 0
+#endif
+constexpr int kRows = HCTR_GATHER_ROWS;
 template <int VEC, int LPR, bool kLocalOnly>
 __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullArgs a) {
   typedef typename RowVec<VEC>::T V;
@@ -146,7 +152,10 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
     for (int k = 0; k < kRows; k++) v[k] = *(const V *)(src[k] + col);
 #pragma unroll
     for (int k = 0; k < kRows; k++)
-      if (j0 + k < n) __builtin_nontemporal_store(v[k], (V *)(dst[k] + col));
+      if (j0 + k < n) {
+        if (HCTR_GATHER_NT) __builtin_nontemporal_store(v[k], (V *)(dst[k] + col));
+        else *(V *)(dst[k] + col) = v[k];
+      }
   }
 }
 

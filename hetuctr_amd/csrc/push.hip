@@ -27,10 +27,16 @@ namespace hctr {
 #define HCTR_TILE_BATCH 8
 #endif
 #ifndef HCTR_DEPTH
-#define HCTR_DEPTH 4
+#define HCTR_DEPTH 8
 #endif
 #ifndef HCTR_RPT
 #define HCTR_RPT 2
+#endif
+#ifndef HCTR_SUM_PRIO
+#define HCTR_SUM_PRIO 0
+#endif
+#ifndef HCTR_ABL
+#define HCTR_ABL 0 // ablation bits for timing experiments only: 1 no version update, 2 no row read, 4 no row store, 8 no gradient loads
 #endif
 #ifndef HCTR_SLICE
 #define HCTR_SLICE 64
@@ -176,7 +182,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
       for (int i = 0; i < G; i++) {
         e[i] = Vec<VEC>::zero();
-        if (mine[i]) e[i] = *(const V *)(t.emb + (size_t)off[i] * W + col);
+        if (mine[i] && !(HCTR_ABL & 2)) e[i] = *(const V *)(t.emb + (size_t)off[i] * W + col);
       }
     }
 #pragma unroll
@@ -188,7 +194,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
       for (int k = 0; k < kHead; k++) {
         v[i][k] = Vec<VEC>::zero();
-        if (mine[i] && (uint32_t)k < len[i]) v[i][k] = *(const V *)(grad + (size_t)si[i][k] * W + col);
+        if (mine[i] && (uint32_t)k < len[i] && !(HCTR_ABL & 8)) v[i][k] = *(const V *)(grad + (size_t)si[i][k] * W + col);
       }
     V acc[G];
 #pragma unroll
@@ -218,8 +224,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
       if (kSingle) {
         V r = e[i];
         Vec<VEC>::add(r, scaled);
-        *(V *)(t.emb + (size_t)off[i] * W + col) = r;
-        if (c0 == 0 && gl == 0) t.ver[off[i]] += (version_t)len[i];
+        if (!(HCTR_ABL & 4)) *(V *)(t.emb + (size_t)off[i] * W + col) = r; // versions: bump_versions
       } else {
         apply_row<VEC, K>(t, id_bits, p, a, u0 + i, scaled, col, c0 == 0 && gl == 0);
       }
@@ -283,8 +288,7 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
       const V scaled = Vec<VEC>::scale(acc, neg_lr);
       if (kSingle) {
         Vec<VEC>::add(e, scaled);
-        *(V *)(t.emb + (size_t)off * W + col) = e;
-        if (c0 == 0 && gl == 0) t.ver[off] += (version_t)len;
+        *(V *)(t.emb + (size_t)off * W + col) = e; // versions: bump_versions
       } else {
         apply_row<VEC, K>(t, id_bits, p, a, u, scaled, col, c0 == 0 && gl == 0);
       }
@@ -402,6 +406,9 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       }
     } else {
       // ---------------- summing wave: one column per lane, rows strictly in order ----------------
+#if HCTR_SUM_PRIO
+      __builtin_amdgcn_s_setprio(HCTR_SUM_PRIO); // the chain of this wave is the critical path of the whole push
+#endif
       float acc = 0.f;
       const uint32_t nfull = L / CR; // chunks with all CR rows
       uint32_t c = 0;
@@ -432,10 +439,21 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
           for (; r < rows; r++) acc += col_ptr[r * CS];
         }
       }
+      // single shard: the version counters are moved by bump_versions, not here
       if (threadIdx.x < CS && slice * CS + threadIdx.x < W)
-        apply_row<1, K>(t, id_bits, p, a, u, acc * neg_lr, slice * CS + threadIdx.x, slice == 0 && threadIdx.x == 0);
+        apply_row<1, K>(t, id_bits, p, a, u, acc * neg_lr, slice * CS + threadIdx.x,
+                        t.nrank > 1 && slice == 0 && threadIdx.x == 0);
     }
   }
+}
+
+// Single shard: every key is owned, so the only counter is the row version, which grows by the number of
+// duplicates (generate_query.cu:68-69).  One thread per unique key, independent of the row kernels.
+__global__ __launch_bounds__(kSmallBlock) void bump_versions(TableView t, BatchView p, uint32_t U) {
+  const uint32_t u = blockIdx.x * kSmallBlock + threadIdx.x;
+  if (u >= U) return;
+  const uint32_t len = p.run_start[u + 1] - p.run_start[u];
+  t.ver[p.uoff[u]] += (version_t)len;
 }
 
 template <int VEC, typename K>
@@ -470,6 +488,8 @@ void launch_push_t(const PushStreams &ps, const TableView &t, int id_bits, const
   if (HCTR_ONLY_ROLE == 0 || HCTR_ONLY_ROLE == 3)
     hipLaunchKernelGGL((push_medium<VEC, LPR, K, kSingle>), dim3(kMedBlocks), dim3(kSmallBlock), 0, ps.aux2, t, id_bits,
                        p, a);
+  if (kSingle && HCTR_ONLY_ROLE == 0)
+    hipLaunchKernelGGL(bump_versions, dim3(div_up(U, kSmallBlock)), dim3(kSmallBlock), 0, ps.aux2, t, p, U);
 }
 
 template <int VEC, typename K, bool kSingle>
