@@ -106,16 +106,9 @@ struct PushArgs {
   version_t *g_cnt;
   embed_t *g_val;
 };
-// The push runs as three kernels (long, medium and short runs of duplicates) on three streams of default
-// priority; everything before it on `main` happens before all three, everything after it on `main` after them.
-struct PushStreams {
-  hipStream_t main, aux1, aux2;
-  hipEvent_t fork, join1, join2;
-  bool main_idle; // nothing is pending on `main` when the push is launched: the fork event is not needed
-};
 // n_unique: number of unique keys of `prev` (host copy)
-void launch_push(const PushStreams &ps, const TableView &t, const KeyLayout &kl, const BatchView &prev,
-                 uint32_t n_unique, const PushArgs &a);
+void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &prev, uint32_t n_unique,
+                 const PushArgs &a);
 
 // ---- query / owner side / pull -------------------------------------------------------------------------
 void launch_lookup_version(hipStream_t s, const TableView &t, const BatchView &cur, version_t *q_ver);

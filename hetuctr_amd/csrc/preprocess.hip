@@ -131,23 +131,29 @@ __global__ __launch_bounds__(kBlock) void scatter_idx_map(BatchView b) {
 }
 
 // one thread per unique rank: long runs are listed by length class, medium runs in one list, for the push.
-// Medium runs are many: a wave reserves its list entries with ONE atomic.
+// Atomics on one address are served one after the other, so a block reserves its list entries with ONE atomic
+// per list: entries are counted and placed inside the block through LDS first.
 __global__ __launch_bounds__(kBlock) void list_long_runs(BatchView b) {
+  constexpr int kLists = kLongBuckets + 1; // length classes of long runs, then the medium list
+  __shared__ uint32_t cnt[kLists], base[kLists];
   const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
+  if (blockIdx.x * kBlock >= *b.d_U) return; // whole block past the last unique key
+  if (threadIdx.x < kLists) cnt[threadIdx.x] = 0;
+  __syncthreads();
   const bool valid = u < *b.d_U;
   const uint32_t len = valid ? b.run_start[u + 1] - b.run_start[u] : 0u;
-  if (len > kLongRun) {
-    const int c = long_bucket(len);
-    b.long_list[(size_t)c * b.long_cap + atomicAdd(&b.d_nlong[c], 1u)] = u;
-  }
-  const bool med = len > kTinyRun && len <= kLongRun;
-  const uint64_t m = __ballot(med);
-  if (m) {
-    const unsigned lane = lane_id();
-    uint32_t base = 0;
-    if (lane == (unsigned)__ffsll((long long)m) - 1u) base = atomicAdd(&b.d_nlong[kMedCount], (uint32_t)__popcll(m));
-    base = __shfl(base, __ffsll((long long)m) - 1, kWave);
-    if (med) b.med_list[base + __popcll(m & ((1ull << lane) - 1ull))] = u;
+  int list = -1;
+  if (len > kLongRun) list = long_bucket(len);
+  else if (len > kTinyRun) list = kLongBuckets;
+  uint32_t local = 0;
+  if (list >= 0) local = atomicAdd(&cnt[list], 1u); // LDS atomic: the order inside a list does not matter
+  __syncthreads();
+  if (threadIdx.x < kLists && cnt[threadIdx.x])
+    base[threadIdx.x] = atomicAdd(&b.d_nlong[threadIdx.x < kLongBuckets ? threadIdx.x : kMedCount], cnt[threadIdx.x]);
+  __syncthreads();
+  if (list >= 0) {
+    if (list < kLongBuckets) b.long_list[(size_t)list * b.long_cap + base[list] + local] = u;
+    else b.med_list[base[list] + local] = u;
   }
 }
 

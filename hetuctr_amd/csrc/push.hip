@@ -9,7 +9,8 @@
 // every run of equal keys is summed by ONE chain of additions per column, in exactly that order: sums are
 // bit-identical to the reference's order (compiled without fused multiply-add contraction), for any skew.
 //
-// Three kernels, one per class of run length, launched on three streams so that they overlap:
+// One launch, three ranges of blocks, one per class of run length (the long chains are dispatched first and the
+// other blocks fill the machine behind them):
 //  * long (> kLongRun duplicates): a run is streamed by a whole block.  Seven loader waves keep several
 //    16-byte loads of gradient rows in flight each and stage them through a ring of LDS slots; the first wave
 //    adds the staged rows in order, one column per lane.  The serial chain costs one LDS read and one add per
@@ -45,13 +46,13 @@ namespace hctr {
 #define HCTR_LONG_BLOCKS 192
 #endif
 #ifndef HCTR_MED_BLOCKS
-#define HCTR_MED_BLOCKS 2048
+#define HCTR_MED_BLOCKS 512
 #endif
 #ifndef HCTR_ONLY_ROLE
 #define HCTR_ONLY_ROLE 0 // 1: long, 2: short, 3: medium role only (timing experiments; results are incomplete)
 #endif
-constexpr int kPushBlock = 512;  // long kernel
-constexpr int kSmallBlock = 256; // medium and short kernels
+constexpr int kPushBlock = 512;
+
 constexpr int kBatch = HCTR_TILE_BATCH;   // short role: gradient rows in flight per group past the first two
 constexpr int kDepth = HCTR_DEPTH;        // long role: chunks in flight per loader thread
 constexpr int kRPT = HCTR_RPT;            // long role: rows per loader thread and chunk
@@ -139,7 +140,7 @@ __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const
 // resident offsets, then the destination rows, the first two gradient-row indices of every run and those
 // gradient rows.  Nine runs out of ten are finished by that; longer ones continue eight rows at a time.
 #ifndef HCTR_RUNS_PER_GROUP
-#define HCTR_RUNS_PER_GROUP 4
+#define HCTR_RUNS_PER_GROUP 2
 #endif
 constexpr int kRunsPerGroup = HCTR_RUNS_PER_GROUP;
 constexpr int kHead = 2; // occurrences per run fetched up front
@@ -149,7 +150,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
                                            uint32_t block, uint32_t U) {
   typedef typename Vec<VEC>::T V;
   constexpr int G = kRunsPerGroup;
-  constexpr int kGroups = kSmallBlock / LPR;
+  constexpr int kGroups = kPushBlock / LPR;
   const uint32_t W = t.width, n = p.n;
   const uint32_t u0 = (block * kGroups + threadIdx.x / LPR) * G;
   if (u0 >= U) return;
@@ -239,9 +240,9 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 // added in order.
 template <int VEC, int LPR, typename K, bool kSingle>
 __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
-                                            uint32_t *lds_idx) {
+                                            uint32_t *lds_idx, uint32_t block, uint32_t nblocks) {
   typedef typename Vec<VEC>::T V;
-  constexpr int kGroups = kSmallBlock / LPR;
+  constexpr int kGroups = kPushBlock / LPR;
   const uint32_t W = t.width;
   const uint32_t gl = threadIdx.x % LPR;
   uint32_t *my_idx = lds_idx + (threadIdx.x / LPR) * kLongRun; // this group's slice of the index staging area
@@ -249,7 +250,7 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
   const uint32_t *__restrict__ sorted_arg = p.sorted_arg;
   const embed_t *__restrict__ grad = a.grad;
   const float neg_lr = t.neg_lr;
-  for (uint32_t item = blockIdx.x * kGroups + threadIdx.x / LPR; item < n_med; item += gridDim.x * kGroups) {
+  for (uint32_t item = block * kGroups + threadIdx.x / LPR; item < n_med; item += nblocks * kGroups) {
     const uint32_t u = p.med_list[item];
     const uint32_t lo = p.run_start[u], hi = p.run_start[u + 1];
     const uint32_t len = hi - lo; // <= kLongRun
@@ -449,51 +450,45 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
 
 // Single shard: every key is owned, so the only counter is the row version, which grows by the number of
 // duplicates (generate_query.cu:68-69).  One thread per unique key, independent of the row kernels.
-__global__ __launch_bounds__(kSmallBlock) void bump_versions(TableView t, BatchView p, uint32_t U) {
-  const uint32_t u = blockIdx.x * kSmallBlock + threadIdx.x;
+__global__ __launch_bounds__(256) void bump_versions(TableView t, BatchView p, uint32_t U) {
+  const uint32_t u = blockIdx.x * 256 + threadIdx.x;
   if (u >= U) return;
   const uint32_t len = p.run_start[u + 1] - p.run_start[u];
   t.ver[p.uoff[u]] += (version_t)len;
 }
 
-template <int VEC, typename K>
-__global__ __launch_bounds__(kPushBlock) void push_long(TableView t, int id_bits, BatchView p, PushArgs a) {
-  __shared__ __align__(16) float lds[kSlots * kRPT * kPushBlock * VEC];
+// all three roles in one launch: the long chains start first, medium and short blocks fill the machine behind them
+template <int VEC, int LPR, typename K, bool kSingle>
+__global__ __launch_bounds__(kPushBlock) void push_fused(TableView t, int id_bits, BatchView p, PushArgs a, uint32_t U) {
+  // one LDS area for whichever role the block plays: the row ring of the long role or the index staging of the
+  // medium role (one slice of kLongRun indices per group)
+  constexpr int kRingWords = kSlots * kRPT * kPushBlock * VEC;
+  constexpr int kStageWords = (kPushBlock / LPR) * (int)kLongRun;
+  __shared__ __align__(16) float lds[kRingWords > kStageWords ? kRingWords : kStageWords];
   __shared__ uint32_t next_item;
-  if (VEC == 4 && t.width % kSlice == 0) long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, &next_item);
-  else long_role<VEC, K, 0>(t, id_bits, p, a, lds, &next_item);
+  if (blockIdx.x < kLongBlocks) {
+    if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 1) return;
+    if (VEC == 4 && t.width % kSlice == 0) long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, &next_item);
+    else long_role<VEC, K, 0>(t, id_bits, p, a, lds, &next_item);
+  } else if (blockIdx.x < kLongBlocks + kMedBlocks) {
+    if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 3) return;
+    medium_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, (uint32_t *)lds, blockIdx.x - kLongBlocks, kMedBlocks);
+  } else {
+    if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 2) return;
+    short_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, blockIdx.x - kLongBlocks - kMedBlocks, U);
+  }
 }
 
 template <int VEC, int LPR, typename K, bool kSingle>
-__global__ __launch_bounds__(kSmallBlock) void push_medium(TableView t, int id_bits, BatchView p, PushArgs a) {
-  __shared__ uint32_t lds_idx[(kSmallBlock / LPR) * kLongRun];
-  medium_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, lds_idx);
-}
-
-template <int VEC, int LPR, typename K, bool kSingle>
-__global__ __launch_bounds__(kSmallBlock) void push_short(TableView t, int id_bits, BatchView p, PushArgs a, uint32_t U) {
-  short_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, blockIdx.x, U);
-}
-
-template <int VEC, int LPR, typename K, bool kSingle>
-void launch_push_t(const PushStreams &ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
-                   const PushArgs &a) {
-  constexpr int kGroups = kSmallBlock / LPR;
-  // the long chains are the critical path: they go first, on the main stream; the other two overlap with them
-  if (HCTR_ONLY_ROLE == 0 || HCTR_ONLY_ROLE == 1)
-    hipLaunchKernelGGL((push_long<VEC, K>), dim3(kLongBlocks), dim3(kPushBlock), 0, ps.main, t, id_bits, p, a);
-  if (HCTR_ONLY_ROLE == 0 || HCTR_ONLY_ROLE == 2)
-    hipLaunchKernelGGL((push_short<VEC, LPR, K, kSingle>), dim3(div_up(U, kGroups * kRunsPerGroup)), dim3(kSmallBlock),
-                       0, ps.aux1, t, id_bits, p, a, U);
-  if (HCTR_ONLY_ROLE == 0 || HCTR_ONLY_ROLE == 3)
-    hipLaunchKernelGGL((push_medium<VEC, LPR, K, kSingle>), dim3(kMedBlocks), dim3(kSmallBlock), 0, ps.aux2, t, id_bits,
-                       p, a);
-  if (kSingle && HCTR_ONLY_ROLE == 0)
-    hipLaunchKernelGGL(bump_versions, dim3(div_up(U, kSmallBlock)), dim3(kSmallBlock), 0, ps.aux2, t, p, U);
+void launch_push_t(hipStream_t st, const TableView &t, int id_bits, const BatchView &p, uint32_t U, const PushArgs &a) {
+  constexpr int kGroups = kPushBlock / LPR;
+  hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle>), dim3(kLongBlocks + kMedBlocks + div_up(U, kGroups * kRunsPerGroup)),
+                     dim3(kPushBlock), 0, st, t, id_bits, p, a, U);
+  if (kSingle) hipLaunchKernelGGL(bump_versions, dim3(div_up(U, 256)), dim3(256), 0, st, t, p, U);
 }
 
 template <int VEC, typename K, bool kSingle>
-void launch_push_v(const PushStreams &ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
+void launch_push_v(hipStream_t ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
                    const PushArgs &a) {
   const uint32_t lanes = (t.width + VEC - 1) / VEC;
   if (lanes <= 4) launch_push_t<VEC, 4, K, kSingle>(ps, t, id_bits, p, U, a);
@@ -504,7 +499,7 @@ void launch_push_v(const PushStreams &ps, const TableView &t, int id_bits, const
 }
 
 template <int VEC, typename K>
-void launch_push_k(const PushStreams &ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
+void launch_push_k(hipStream_t ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
                    const PushArgs &a) {
   if (t.nrank == 1) launch_push_v<VEC, K, true>(ps, t, id_bits, p, U, a);
   else launch_push_v<VEC, K, false>(ps, t, id_bits, p, U, a);
@@ -512,16 +507,9 @@ void launch_push_k(const PushStreams &ps, const TableView &t, int id_bits, const
 
 } // namespace
 
-void launch_push(const PushStreams &ps, const TableView &t, const KeyLayout &kl, const BatchView &prev,
-                 uint32_t n_unique, const PushArgs &a) {
+void launch_push(hipStream_t ps, const TableView &t, const KeyLayout &kl, const BatchView &prev, uint32_t n_unique,
+                 const PushArgs &a) {
   if (!prev.n || !n_unique) return;
-  // fork: the two auxiliary streams start after everything queued on the main stream so far (nothing is, when
-  // the caller knows the main stream to be idle)
-  if (!ps.main_idle) {
-    HCTR_HIP(hipEventRecord(ps.fork, ps.main));
-    HCTR_HIP(hipStreamWaitEvent(ps.aux1, ps.fork, 0));
-    HCTR_HIP(hipStreamWaitEvent(ps.aux2, ps.fork, 0));
-  }
   const bool vec4 = t.width % 4 == 0 && ((uintptr_t)a.grad % 16) == 0;
   if (vec4) {
     if (kl.wide) launch_push_k<4, uint64_t>(ps, t, kl.id_bits, prev, n_unique, a);
@@ -531,11 +519,6 @@ void launch_push(const PushStreams &ps, const TableView &t, const KeyLayout &kl,
     else launch_push_k<1, uint32_t>(ps, t, kl.id_bits, prev, n_unique, a);
   }
   HCTR_HIP(hipGetLastError());
-  // join: the main stream continues when all three kernels are done
-  HCTR_HIP(hipEventRecord(ps.join1, ps.aux1));
-  HCTR_HIP(hipEventRecord(ps.join2, ps.aux2));
-  HCTR_HIP(hipStreamWaitEvent(ps.main, ps.join1, 0));
-  HCTR_HIP(hipStreamWaitEvent(ps.main, ps.join2, 0));
 }
 
 } // namespace hctr

@@ -4,7 +4,8 @@
 //   digit_histogram   per-block digit counts (LDS atomics) -> ghist[bin][block]
 //   scan_bins         one block per digit value: exclusive scan of its row over the blocks + row total
 //   scatter           per block: global base of every bin, stable rank of every key inside the block
-//                     (wave-level match by ballots, wave-private LDS counters), scatter to the output
+//                     (wave-level match by ballots, wave-private LDS counters), the tile sorted by digit in
+//                     LDS, then stores that are contiguous per bin
 // Stability: a block's tile is split into 4 contiguous sub-tiles, one per wave; a wave walks its
 // sub-tile 64 keys at a time in ascending position; inside such a group the rank among equal digits is
 // the lane order.  Wave-private counters make the result independent of wave scheduling.
@@ -61,22 +62,24 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
                                                       const uint32_t *__restrict__ ghist, uint32_t nblocks,
                                                       const uint32_t *__restrict__ bintot) {
   __shared__ uint32_t cnt[kWaves][1 << kSortMaxDigitBits];
-  __shared__ uint32_t base[1 << kSortMaxDigitBits];
+  __shared__ uint32_t base[1 << kSortMaxDigitBits];      // global position of the bin's first key of this block
+  __shared__ uint32_t bin_start[1 << kSortMaxDigitBits]; // position of the bin inside the block's sorted tile
+  __shared__ K skey[kSortTile];
+  __shared__ uint32_t sval[kSortTile];
   __shared__ uint32_t sm[kWaves + 1];
   const uint32_t nb = 1u << dbits, mask = nb - 1;
   const int w = threadIdx.x / kWave;
   const unsigned lane = lane_id();
+  const uint32_t per = (nb + kSortBlock - 1) / kSortBlock; // consecutive bins per thread in the two bin scans
+  const uint32_t blo = min(threadIdx.x * per, nb), bhi = min(blo + per, nb);
 
-  // global base of each bin for this block: sum of the totals of lower bins + this bin's lower blocks.
-  // 256 threads, up to 1024 bins: 4 consecutive bins per thread.
+  // global base of each bin for this block: sum of the totals of lower bins + this bin's lower blocks
   {
-    const uint32_t per = (nb + kSortBlock - 1) / kSortBlock;
-    const uint32_t lo = min(threadIdx.x * per, nb), hi = min(lo + per, nb);
     uint32_t s = 0;
-    for (uint32_t i = lo; i < hi; i++) s += bintot[i];
+    for (uint32_t i = blo; i < bhi; i++) s += bintot[i];
     uint32_t total;
     uint32_t off = block_exclusive_scan<kSortBlock>(s, sm, total);
-    for (uint32_t i = lo; i < hi; i++) {
+    for (uint32_t i = blo; i < bhi; i++) {
       base[i] = off + ghist[(size_t)i * nblocks + blockIdx.x];
       off += bintot[i];
     }
@@ -84,9 +87,10 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
   for (uint32_t i = threadIdx.x; i < kWaves * nb; i += kSortBlock) cnt[i / nb][i % nb] = 0;
   __syncthreads();
 
+  // stable rank of every key among the keys of its wave with the same digit
   K key[kRounds];
   uint32_t val[kRounds];
-  uint32_t dig[kRounds];  // digit | local rank << 10 would overflow for rank up to 512: keep separate
+  uint32_t dig[kRounds];
   uint32_t rnk[kRounds];
   const uint32_t wbase = blockIdx.x * kSortTile + w * kSub;
 #pragma unroll
@@ -95,6 +99,11 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
     const bool valid = idx < n;
     key[r] = valid ? keys_in[idx] : (K)0;
     val[r] = kFirst ? idx : (valid ? vals_in[idx] : 0u);
+  }
+#pragma unroll
+  for (int r = 0; r < kRounds; r++) {
+    const uint32_t idx = wbase + r * kWave + lane;
+    const bool valid = idx < n;
     const uint32_t d = (uint32_t)(key[r] >> shift) & mask;
     uint64_t m = __ballot(valid);
     for (int b = 0; b < dbits; b++) {
@@ -114,24 +123,51 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
     rnk[r] = prior + before;
   }
   __syncthreads();
-  // wave-private counts -> start of each wave's keys inside the bin, plus the bin's global base
-  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) {
-    uint32_t run = base[i];
+  // wave-private counts -> offset of each wave's keys inside the bin; bin totals -> start of the bin in the tile
+  {
+    uint32_t s = 0;
+    for (uint32_t i = blo; i < bhi; i++) {
+      uint32_t run = 0;
 #pragma unroll
-    for (int ww = 0; ww < kWaves; ww++) {
-      uint32_t t = cnt[ww][i];
-      cnt[ww][i] = run;
-      run += t;
+      for (int ww = 0; ww < kWaves; ww++) {
+        const uint32_t t = cnt[ww][i];
+        cnt[ww][i] = run;
+        run += t;
+      }
+      bin_start[i] = run; // total of the bin for now
+      s += run;
+    }
+    uint32_t total;
+    uint32_t off = block_exclusive_scan<kSortBlock>(s, sm, total);
+    for (uint32_t i = blo; i < bhi; i++) {
+      const uint32_t t = bin_start[i];
+      bin_start[i] = off;
+      off += t;
     }
   }
   __syncthreads();
+  // the tile, sorted by digit, in LDS
 #pragma unroll
   for (int r = 0; r < kRounds; r++) {
     const uint32_t idx = wbase + r * kWave + lane;
     if (idx < n) {
-      const uint32_t pos = cnt[w][dig[r]] + rnk[r];
-      keys_out[pos] = key[r];
-      vals_out[pos] = val[r];
+      const uint32_t lp = bin_start[dig[r]] + cnt[w][dig[r]] + rnk[r];
+      skey[lp] = key[r];
+      sval[lp] = val[r];
+    }
+  }
+  __syncthreads();
+  // neighbouring threads now hold neighbouring keys of a bin: the global stores of a bin are contiguous
+  const uint32_t tile_n = min((uint32_t)kSortTile, n - blockIdx.x * kSortTile);
+#pragma unroll
+  for (int k = 0; k < kSortItems; k++) {
+    const uint32_t i = k * kSortBlock + threadIdx.x;
+    if (i < tile_n) {
+      const K kk = skey[i];
+      const uint32_t d = (uint32_t)(kk >> shift) & mask;
+      const uint32_t pos = base[d] + (i - bin_start[d]);
+      keys_out[pos] = kk;
+      vals_out[pos] = sval[i];
     }
   }
 }

@@ -147,13 +147,11 @@ class Group {
   const std::string key;
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  PushStreams push_streams{};
   std::vector<Shard *> members;
   DeviceBuf desc_dev;
   CopyDesc *desc_host = nullptr;
   size_t desc_cap = 0;
   double wait_seconds = 120.0;
-  bool stream_idle = false; // true between a completed call and the next work queued on `stream`
   void sync_stream();
 
   // per-stage device time, accumulated over calls while stage_timing is on

@@ -329,10 +329,7 @@ void Shard::generate_gradient(const float *grad) {
     a.g_val = g_val.as<embed_t>();
   }
   StageScope st(*group, S_PUSH);
-  PushStreams ps = group->push_streams;
-  ps.main_idle = group->stream_idle && !group->stage_timing;
-  launch_push(ps, tv, kl, prev.view(), prev.U, a);
-  group->stream_idle = false;
+  launch_push(s, tv, kl, prev.view(), prev.U, a);
 }
 
 // csrc/core/generate_query.cu:91-106
@@ -537,12 +534,6 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   HCTR_HIP(hipStreamCreate(&stream));
   HCTR_HIP(hipEventCreate(&ev0));
   HCTR_HIP(hipEventCreate(&ev1));
-  push_streams.main = stream;
-  HCTR_HIP(hipStreamCreateWithFlags(&push_streams.aux1, hipStreamNonBlocking));
-  HCTR_HIP(hipStreamCreateWithFlags(&push_streams.aux2, hipStreamNonBlocking));
-  HCTR_HIP(hipEventCreateWithFlags(&push_streams.fork, hipEventDisableTiming));
-  HCTR_HIP(hipEventCreateWithFlags(&push_streams.join1, hipEventDisableTiming));
-  HCTR_HIP(hipEventCreateWithFlags(&push_streams.join2, hipEventDisableTiming));
   a_keys_.resize(nr);
   a_n_.resize(nr);
   a_grad_.resize(nr);
@@ -556,11 +547,6 @@ Group::~Group() {
   if (ev1) (void)hipEventDestroy(ev1);
   for (auto &m : marks) { (void)hipEventDestroy(m.a); (void)hipEventDestroy(m.b); }
   for (auto e : event_pool) (void)hipEventDestroy(e);
-  if (push_streams.fork) (void)hipEventDestroy(push_streams.fork);
-  if (push_streams.join1) (void)hipEventDestroy(push_streams.join1);
-  if (push_streams.join2) (void)hipEventDestroy(push_streams.join2);
-  if (push_streams.aux1) (void)hipStreamDestroy(push_streams.aux1);
-  if (push_streams.aux2) (void)hipStreamDestroy(push_streams.aux2);
   if (stream) (void)hipStreamDestroy(stream);
 }
 
@@ -709,13 +695,11 @@ void Group::sync_stream() {
   while ((e = hipStreamQuery(stream)) == hipErrorNotReady) {
   }
   HCTR_HIP(e);
-  stream_idle = true;
 }
 
 void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
-  stream_idle = false;
   HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) {
     m->swap_batches();
@@ -750,7 +734,6 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
 void Group::push_pull_all(const float *const *grads, float *const *dsts) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
-  if (stage_timing || nrank > 1) stream_idle = false; // an event record or another shard's work precedes the push
   HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) {
     m->generate_gradient(grads[m->cfg.rank]);
@@ -761,7 +744,6 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
     for (Shard *m : members) m->handle_gradient();
     for (Shard *m : members) m->handle_query();
     sync_stream(); // hetu_gpu_table.cu:33: the return counts size the next exchange
-    stream_idle = false;
     collect_marks();
     for (Shard *m : members) m->finish_handle_query();
     exchange_return();
