@@ -64,6 +64,8 @@ constexpr int kMedBlocks = HCTR_MED_BLOCKS;
 
 namespace {
 
+__device__ __forceinline__ uint32_t div_up_dev(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
 template <int VEC> struct Vec;
 template <> struct Vec<4> {
   typedef float4 T;
@@ -448,16 +450,8 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
   }
 }
 
-// Single shard: every key is owned, so the only counter is the row version, which grows by the number of
-// duplicates (generate_query.cu:68-69).  One thread per unique key, independent of the row kernels.
-__global__ __launch_bounds__(256) void bump_versions(TableView t, BatchView p, uint32_t U) {
-  const uint32_t u = blockIdx.x * 256 + threadIdx.x;
-  if (u >= U) return;
-  const uint32_t len = p.run_start[u + 1] - p.run_start[u];
-  t.ver[p.uoff[u]] += (version_t)len;
-}
-
-// all three roles in one launch: the long chains start first, medium and short blocks fill the machine behind them
+// all roles in one launch: the long chains start first, medium and short blocks fill the machine behind them, the
+// version counters of a single shard come last
 template <int VEC, int LPR, typename K, bool kSingle>
 __global__ __launch_bounds__(kPushBlock) void push_fused(TableView t, int id_bits, BatchView p, PushArgs a, uint32_t U) {
   // one LDS area for whichever role the block plays: the row ring of the long role or the index staging of the
@@ -474,17 +468,28 @@ __global__ __launch_bounds__(kPushBlock) void push_fused(TableView t, int id_bit
     if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 3) return;
     medium_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, (uint32_t *)lds, blockIdx.x - kLongBlocks, kMedBlocks);
   } else {
-    if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 2) return;
-    short_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, blockIdx.x - kLongBlocks - kMedBlocks, U);
+    constexpr int kGroups = kPushBlock / LPR;
+    const uint32_t short_blocks = div_up_dev(U, kGroups * kRunsPerGroup);
+    const uint32_t b = blockIdx.x - kLongBlocks - kMedBlocks;
+    if (b < short_blocks) {
+      if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 2) return;
+      short_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, b, U);
+    } else if (kSingle) {
+      // Single shard: every key is owned, so the only counter is the row version, which grows by the number of
+      // duplicates (generate_query.cu:68-69).  One thread per unique key, in the last blocks of the grid.
+      const uint32_t u = (b - short_blocks) * kPushBlock + threadIdx.x;
+      if (u < U) t.ver[p.uoff[u]] += (version_t)(p.run_start[u + 1] - p.run_start[u]);
+    }
   }
 }
 
 template <int VEC, int LPR, typename K, bool kSingle>
 void launch_push_t(hipStream_t st, const TableView &t, int id_bits, const BatchView &p, uint32_t U, const PushArgs &a) {
   constexpr int kGroups = kPushBlock / LPR;
-  hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle>), dim3(kLongBlocks + kMedBlocks + div_up(U, kGroups * kRunsPerGroup)),
-                     dim3(kPushBlock), 0, st, t, id_bits, p, a, U);
-  if (kSingle) hipLaunchKernelGGL(bump_versions, dim3(div_up(U, 256)), dim3(256), 0, st, t, p, U);
+  const unsigned ver_blocks = kSingle ? div_up(U, kPushBlock) : 0; // version counters of a single shard
+  hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle>),
+                     dim3(kLongBlocks + kMedBlocks + div_up(U, kGroups * kRunsPerGroup) + ver_blocks), dim3(kPushBlock), 0,
+                     st, t, id_bits, p, a, U);
 }
 
 template <int VEC, typename K, bool kSingle>
