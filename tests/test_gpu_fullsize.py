@@ -1,0 +1,121 @@
+"""The BASELINE.json configurations at their full sizes on the GPU.
+
+cfg2 (headline) runs next to the CPU oracle and must agree bit for bit.  The larger ones are checked through
+properties that do not need an oracle of that size: the integer outputs against numpy's own unique / lexsort on
+the same keys, and the update arithmetic with integer-valued gradients, whose sums are exact in any order, against
+a float64 scatter-add (np.add.at)."""
+import numpy as np
+import pytest
+import torch
+
+from hetuctr_amd import capi, workloads
+from oracle import oracle as orc
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def single_table(rows, width, init, lr):
+    capi.seed(0)
+    return capi.Table(0, 1, 0, "127.0.0.1", 0, rows, width, 0, 0, np.zeros(rows, np.uint8),
+                      np.arange(rows, dtype=np.int64), init, lr, 0)
+
+
+def check_integers(t, keys):
+    """unique / sorted_arg / run_start / idx_map of the table's current batch against numpy on the same keys."""
+    n = keys.shape[0]
+    uniq, first, inverse, counts = np.unique(keys, return_index=True, return_inverse=True, return_counts=True)
+    assert np.array_equal(t.fetch(capi.UNIQUE), uniq)
+    run_start = np.concatenate([[0], np.cumsum(counts)])
+    assert np.array_equal(t.fetch(capi.RUN_START), run_start)
+    assert np.array_equal(t.fetch(capi.IDX_MAP), inverse.reshape(-1))
+    sa = t.fetch(capi.SORTED_ARG)
+    assert np.array_equal(sa, np.argsort(keys, kind="stable"))   # stable: equal keys in ascending position
+    assert np.array_equal(t.fetch(capi.OFFSET), uniq)            # identity storage: offset == id
+    assert t.fetch(capi.SIZES)[:2].tolist() == [n, uniq.shape[0]]
+    return uniq, counts
+
+
+def test_cfg2_headline_bit_exact_against_oracle():
+    cfg = workloads.CONFIGS["cfg2"]
+    ks = workloads.KeyStream(cfg, seed=0)
+    rows, width, n = ks.rows, cfg["width"], ks.n
+    say("cfg2 full size: %d rows x %d, %d keys" % (rows, width, n))
+    t = single_table(rows, width, ("Zero", 0.0, 0.0), cfg["lr"])
+    o = orc.Oracle(1, rows, width, 0, 0, np.zeros(rows, np.uint8), [np.arange(rows, dtype=np.int64)],
+                   init=("Zero", 0.0, 0.0), learning_rate=cfg["lr"])
+    o.set_parallel(True)
+    rng = np.random.default_rng(3)
+    dst = torch.empty((n, width), device="cuda")
+    ref = np.empty((n, width), np.float32)
+    grad = None
+    for step in range(3):
+        keys = ks.batch()
+        dk = torch.from_numpy(keys).cuda()
+        dg = None if grad is None else torch.from_numpy(grad).cuda()
+        torch.cuda.synchronize()
+        t.preprocess(dk.data_ptr(), n)
+        t.push_pull(0 if dg is None else dg.data_ptr(), dst.data_ptr())
+        o.preprocess_raw([keys])
+        o.push_pull_into([grad], [ref])
+        for item in (capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.OFFSET):
+            assert np.array_equal(t.fetch(item), o.fetch(0, item)), "item %d step %d" % (item, step)
+        got = dst.cpu().numpy()
+        assert np.array_equal(got, ref), "step %d: %d rows differ" % (step, int((got != ref).any(axis=1).sum()))
+        assert_close(got, ref, 1e-5, "cfg2 step %d" % step)
+        grad = rng.normal(0, 1e-3, size=(n, width)).astype(np.float32)
+    u = o.fetch(0, orc.UNIQUE)
+    ver_gpu = t.fetch(capi.VERSION)
+    assert np.array_equal(ver_gpu, o.fetch(0, orc.VERSION))
+    t.close(); o.close()
+
+
+@pytest.mark.parametrize("name", ["cfg4", "cfg5_zipf", "cfg5_uniform"])
+def test_large_configs_by_properties(name):
+    cfg = workloads.CONFIGS[name]
+    ks = workloads.KeyStream(cfg, seed=0)
+    rows, width, n = ks.rows, cfg["width"], ks.n
+    say("%s full size: %d rows x %d, %d keys" % (name, rows, width, n))
+    t = single_table(rows, width, ("Zero", 0.0, 0.0), -1.0)      # lr = -1: rows accumulate the gradients
+    dst = torch.empty((n, width), device="cuda")
+    rng = np.random.default_rng(5)
+    total = {}                                                   # id -> accumulated column-0 value (float64)
+    acc = np.zeros(0)
+    prev_keys, prev_g = None, None
+    table_sum = np.zeros(width)
+    for step in range(3):
+        keys = ks.batch()
+        dk = torch.from_numpy(keys).cuda()
+        if prev_keys is None:
+            dg = None
+        else:
+            # integer-valued gradients in [-3, 3]: every partial sum is exact in fp32, in any order
+            g_int = rng.integers(-3, 4, size=(prev_keys.shape[0], 1)).astype(np.float32)
+            prev_g = g_int
+            dg = (torch.from_numpy(g_int).cuda() * torch.arange(1, width + 1, device="cuda", dtype=torch.float32)).contiguous()
+        torch.cuda.synchronize()
+        t.preprocess(dk.data_ptr(), n)
+        t.push_pull(0 if dg is None else dg.data_ptr(), dst.data_ptr())
+        uniq, counts = check_integers(t, keys)
+        if prev_keys is not None:
+            u_prev, inv = np.unique(prev_keys, return_inverse=True)
+            s = np.zeros(u_prev.shape[0])
+            np.add.at(s, inv.reshape(-1), prev_g[:, 0].astype(np.float64))
+            for k, v in zip(u_prev[s != 0].tolist(), s[s != 0].tolist()):
+                total[k] = total.get(k, 0.0) + v
+        got = dst.cpu().numpy()
+        expect0 = np.array([total.get(k, 0.0) for k in uniq.tolist()])[np.searchsorted(uniq, keys)]
+        assert np.array_equal(got[:, 0], expect0.astype(np.float32)), "%s step %d column 0" % (name, step)
+        # column w holds (w+1) times column 0, exactly
+        assert np.array_equal(got[:, width - 1], (expect0 * width).astype(np.float32))
+        # equal keys pulled equal rows
+        first_pos = np.unique(keys, return_index=True)[1]
+        assert np.array_equal(got, got[first_pos][np.searchsorted(uniq, keys)])
+        prev_keys = keys
+    ver = t.fetch(capi.VERSION)
+    assert int(ver.sum()) == 2 * n                               # two batches were pushed, one count per key
+    t.close()
