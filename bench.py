@@ -154,7 +154,7 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath) and a.scale == 1.0:
         traffic = json.load(open(tpath)).get(a.config, {})
-    kernel_names = {"segment_sum_apply": "push_long + push_short + push_medium (concurrent, one stage)", "gather": "gather"}
+    kernel_names = {"segment_sum_apply": "push_fused", "gather": "gather"}
     roof_all = {}
     for k, (tot, cnt) in stages.items():
         if k in kernel_names and cnt > 0:
