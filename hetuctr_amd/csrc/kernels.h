@@ -74,7 +74,7 @@ struct TableView {
 // keys_copy (optional): the ids are also copied there (the reference's d_idx); nlong (optional) is zeroed
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
                       void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong);
-// sorted keys -> everything per unique key + inverse index.  block_heads: scratch of sort_blocks(n) words.
+// sorted keys -> everything per unique key + inverse index.  block_heads: scratch of scan_blocks(n) words.
 // u_copy (optional) receives the number of unique keys as well (b.d_U always does)
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
                    const BatchView &b, uint32_t *block_heads, uint32_t *u_copy);

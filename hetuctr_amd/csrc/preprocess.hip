@@ -11,7 +11,7 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kItems = 8;
-constexpr int kTile = kBlock * kItems; // == kSortTile, so sort_blocks(n) sizes the scratch
+constexpr int kTile = kBlock * kItems; // 2048: scan_blocks(n) sizes the scratch
 
 template <typename K>
 __global__ __launch_bounds__(kBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,

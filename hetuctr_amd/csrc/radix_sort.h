@@ -6,7 +6,10 @@
 namespace hctr {
 
 constexpr int kSortBlock = 256;                 // threads per block (4 waves)
-constexpr int kSortItems = 8;                   // keys per thread
+#ifndef HCTR_SORT_ITEMS
+#define HCTR_SORT_ITEMS 16
+#endif
+constexpr int kSortItems = HCTR_SORT_ITEMS;     // keys per thread
 constexpr int kSortTile = kSortBlock * kSortItems;
 constexpr int kSortMaxDigitBits = 10;           // up to 1024 bins: 4 wave-private rows of 4 KiB in LDS
 
@@ -17,6 +20,8 @@ struct SortScratch {
 };
 
 inline size_t sort_blocks(size_t n) { return (n + kSortTile - 1) / kSortTile; }
+// tiles of the scan / unique kernels of the preprocess (256 threads x 8 items), whatever the sort tile is
+inline size_t scan_blocks(size_t n) { return (n + 2047) / 2048; }
 
 // Sorts n pairs by the low `bits` bits of the key.  The value of element i is its position i (never
 // materialised as an input).  keys_in is left untouched; tmp_k0/tmp_k1 and tmp_v0/tmp_v1 are ping-pong

@@ -186,7 +186,7 @@ void Shard::reserve_batch_scratch(uint32_t n) {
   const size_t blocks = sort_blocks(m);
   ghist.reserve(((size_t)1 << kSortMaxDigitBits) * blocks * 4);
   bintot.reserve(((size_t)1 << kSortMaxDigitBits) * 4);
-  block_sums.reserve((blocks + 2) * 4);
+  block_sums.reserve((scan_blocks(m) + 2) * 4);
 }
 
 // csrc/core/preprocess.cu:92-141
