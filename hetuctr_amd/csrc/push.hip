@@ -56,7 +56,10 @@ constexpr int kPushBlock = 512;
 constexpr int kBatch = HCTR_TILE_BATCH;   // short role: gradient rows in flight per group past the first two
 constexpr int kDepth = HCTR_DEPTH;        // long role: chunks in flight per loader thread
 constexpr int kRPT = HCTR_RPT;            // long role: rows per loader thread and chunk
-constexpr int kSlots = 3;                 // long role: LDS ring slots
+#ifndef HCTR_SLOTS
+#define HCTR_SLOTS 3
+#endif
+constexpr int kSlots = HCTR_SLOTS;        // long role: LDS ring slots
 constexpr int kSlice = HCTR_SLICE;        // long role: columns per block
 constexpr int kLongBlocks = HCTR_LONG_BLOCKS;
 constexpr int kMedBlocks = HCTR_MED_BLOCKS;
@@ -453,7 +456,10 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
 // all roles in one launch: the long chains start first, medium and short blocks fill the machine behind them, the
 // version counters of a single shard come last
 template <int VEC, int LPR, typename K, bool kSingle>
-__global__ __launch_bounds__(kPushBlock) void push_fused(TableView t, int id_bits, BatchView p, PushArgs a, uint32_t U) {
+#ifndef HCTR_PUSH_WAVES
+#define HCTR_PUSH_WAVES 4
+#endif
+__global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR_PUSH_WAVES, 8))) void push_fused(TableView t, int id_bits, BatchView p, PushArgs a, uint32_t U) {
   // one LDS area for whichever role the block plays: the row ring of the long role or the index staging of the
   // medium role (one slice of kLongRun indices per group)
   constexpr int kRingWords = kSlots * kRPT * kPushBlock * VEC;
