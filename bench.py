@@ -31,6 +31,10 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=3)
     ap.add_argument("--no-stage-timing", action="store_true")
+    ap.add_argument("--active-peers", action="store_true",
+                    help="sharded configs: every rank caches hot rows and feeds batches (default: rank 0 only)")
+    ap.add_argument("--pull-bound", type=int, default=0, help="sharded configs: staleness bound of pulls")
+    ap.add_argument("--push-bound", type=int, default=0, help="sharded configs: staleness bound of pushes")
     return ap.parse_args()
 
 
@@ -64,6 +68,104 @@ def cpu_baseline(cfg, ks, batches, width, lr, steps):
                        "OpenMP oracle, warm" % (steps, n, rows, width))
 
 
+def main_sharded(a, cfg):
+    """cfg3: the shards of an 8-way partition live on this one GPU behind the loopback.  By default only rank 0 feeds
+    batches and holds the hot-row cache; the seven peers own their rows and serve rank 0's pushes and queries with
+    the real owner-side kernels (in a deployment that work runs on the other GPUs, here it is inside the step
+    time).  With --active-peers every rank has a cache and feeds its own batches, so rows do go stale and get
+    refreshed; the GPU then does the work of all eight ranks in turn and `value` counts all their keys."""
+    import torch
+    from hetuctr_amd import capi, workloads
+    R, width, lr = cfg["nrank"], cfg["width"], cfg["lr"]
+    active = list(range(R)) if a.active_peers else [0]
+    ks = workloads.KeyStream(cfg, seed=0, scale=a.scale)
+    nb = max(2, a.batches)
+    batches = {r: [ks.batch() for _ in range(nb)] for r in active}
+    ks.release_tables()
+    n = batches[0][0].shape[0]
+    root, storage = workloads.shard_layout(ks, R, cfg["cache_frac"], cached_ranks=active)
+    print("[bench] %s: %d rows x %d over %d shards, rank 0 owns %d and caches %d rows, %d keys/batch, ranks with "
+          "batches: %s" % (a.config, ks.rows, width, R, int((root == 0).sum()),
+                           storage[0].shape[0] - int((root == 0).sum()), n, active), file=sys.stderr, flush=True)
+    torch.cuda.set_device(0)
+    capi.seed(0)
+    bounds = (a.pull_bound, a.push_bound)
+    tables = [capi.Table(r, R, 0, "127.0.0.1", 23456, ks.rows, width, bounds[0], bounds[1], root, storage[r],
+                         cfg["init"], lr, 0) for r in range(R)]
+    dkeys = {r: [torch.from_numpy(b).cuda() for b in batches[r]] for r in active}
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    grad = torch.randn((n, width), device="cuda", generator=gen) * 1e-3
+    dsts = {r: torch.empty((n, width), device="cuda") for r in active}
+    torch.cuda.synchronize()
+    counts = [n if r in dkeys else 0 for r in range(R)]
+    gptr = [grad.data_ptr() if r in dkeys else 0 for r in range(R)]
+    dptr = [dsts[r].data_ptr() if r in dkeys else 0 for r in range(R)]
+
+    def step(i):
+        capi.group_preprocess(tables, [dkeys[r][i % nb].data_ptr() if r in dkeys else 0 for r in range(R)], counts)
+        capi.group_push_pull(tables, gptr, dptr)
+
+    w0 = max(a.warmup, 2) + nb
+    for i in range(w0):
+        step(i)
+    pre_ms = pp_ms = 0.0
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(w0 + i)
+        p, q = tables[0].last_times()
+        pre_ms += p
+        pp_ms += q
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    stages = None
+    if not a.no_stage_timing:
+        tables[0].stage_timing(True)
+        for i in range(a.steps):
+            step(w0 + a.steps + i)
+        stages = {k: {"ms_per_step": v[0] / a.steps, "intervals_per_step": v[1] / a.steps}
+                  for k, v in tables[0].stage_times().items() if v[1]}
+        tables[0].stage_timing(False)
+    k = min(a.steps, nb)                     # counters of a few more steps, outside the timed region
+    acc = np.zeros(6)                        # per step, summed over the ranks: hit, miss, refreshed, pushed, returned, received
+    us = 0.0
+    for i in range(k):
+        step(w0 + 2 * a.steps + i)
+        for t in tables:
+            acc += np.asarray(t.fetch(capi.STATS)[:6], dtype=np.float64) / k
+        us += sum(float(tables[r].fetch(capi.SIZES)[1]) for r in active) / k
+    hit, miss, refresh, pushed, served, received = acc
+    ms_step = 1e3 * dt / a.steps
+    keys_step = n * len(active)
+    bytes_step = workloads.algorithmic_bytes(keys_step, us, width) + workloads.sharded_extra_bytes(
+        width, hit + refresh, pushed, received, us, served, refresh)
+    gbs = bytes_step / (ms_step * 1e-3) / 1e9
+    out = {
+        "metric": "sparse IDs/sec per train step (pull+push)", "value": keys_step * a.steps / dt, "unit": "IDs/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: %d shards of a %d-row x %d fp32 table (uniform owners) on one GPU behind the "
+                               "loopback, ranks %s feed batches of %d keys (per-field Zipf %.2f) and cache the hottest "
+                               "%.0f%% of their remote rows, bounds pull/push %d/%d; the other ranks only serve" %
+                               (a.config, R, ks.rows, width, active, n, cfg["alpha"], 100 * cfg["cache_frac"],
+                                bounds[0], bounds[1]),
+                   "keys_per_step": keys_step, "unique_keys_per_step": us, "width": width, "rows": ks.rows},
+        "cache_per_step_all_ranks": {"remote_unique_keys_hit": hit, "missed_not_cached": miss, "refreshed": refresh,
+                                     "rows_pushed_to_owners": pushed, "rows_returned_by_owners": served},
+        "device_ms_per_step": {"preprocess": pre_ms / a.steps, "push_pull": pp_ms / a.steps},
+        "step_hbm": {"algorithmic_bytes": int(bytes_step), "achieved_GBps": gbs, "frac": gbs / HBM_PEAK_GBS},
+        "roofline": {"bound": "hbm", "kernel": "whole step (all shards' kernels)", "achieved": gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None, "avg_ms": ms_step,
+                     "algorithmic_bytes": int(bytes_step)},
+        "stages_all_shards": stages,
+        "cpu_baseline": None,
+    }
+    for t in tables:
+        t.close()
+    print(json.dumps(out), flush=True)
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -77,6 +179,8 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     cfg = workloads.CONFIGS[a.config]
+    if cfg.get("nrank", 1) > 1:
+        return main_sharded(a, cfg)
     width, lr = cfg["width"], cfg["lr"]
     t_gen = time.perf_counter()
     ks = workloads.KeyStream(cfg, seed=0, scale=a.scale)

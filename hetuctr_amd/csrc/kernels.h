@@ -130,7 +130,8 @@ struct PullArgs {
   const embed_t *in_val;
   embed_t *dst;              // [n][width]
 };
-void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a, uint32_t *stats);
+void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
+                    uint32_t *stats);
 void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a);
 
 // ---- init -------------------------------------------------------------------------------------------------

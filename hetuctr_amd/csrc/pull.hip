@@ -91,10 +91,42 @@ __global__ __launch_bounds__(kBlock) void pack_rows(TableView t, const index_t *
     *(V *)(ret_val + (size_t)pos * W + col) = *(const V *)(t.emb + (size_t)o * W + col);
 }
 
+// Counts of the step's remote unique keys: [0] cached and fresh enough, [1] not stored here, [2] cached and
+// refreshed.  Atomics on one address are served one after the other, so every thread counts its strided share in
+// registers and a block adds its three totals once.
+constexpr int kCountBlocks = 128;
+__global__ __launch_bounds__(kBlock) void count_remote(TableView t, BatchView c, const uint32_t *__restrict__ got,
+                                                       uint32_t *__restrict__ stats) {
+  __shared__ uint32_t tot[3];
+  if (threadIdx.x < 3) tot[threadIdx.x] = 0;
+  __syncthreads();
+  const uint32_t U = *c.d_U;
+  uint32_t n0 = 0, n1 = 0, n2 = 0;
+  for (uint32_t u = blockIdx.x * kBlock + threadIdx.x; u < U; u += kCountBlocks * kBlock) {
+    const slot_t o = c.uoff[u];
+    if (o == kNoSlot) n1++;
+    else if ((uint32_t)o < t.n_cached) {
+      if (got[u]) n2++;
+      else n0++;
+    }
+  }
+  for (int d = 32; d; d >>= 1) {
+    n0 += __shfl_down(n0, d);
+    n1 += __shfl_down(n1, d);
+    n2 += __shfl_down(n2, d);
+  }
+  if (threadIdx.x % 64 == 0) {
+    atomicAdd(&tot[0], n0);
+    atomicAdd(&tot[1], n1);
+    atomicAdd(&tot[2], n2);
+  }
+  __syncthreads();
+  if (threadIdx.x < 3 && tot[threadIdx.x]) atomicAdd(&stats[threadIdx.x], tot[threadIdx.x]);
+}
+
 // one group per unique rank of the current batch
 template <int VEC, int LPR>
-__global__ __launch_bounds__(kBlock) void refresh(TableView t, int id_bits_unused, BatchView c, PullArgs a,
-                                                  uint32_t *__restrict__ stats) {
+__global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, PullArgs a, uint32_t *__restrict__ stats) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
   const uint32_t u = blockIdx.x * kGroups + threadIdx.x / LPR;
@@ -102,8 +134,6 @@ __global__ __launch_bounds__(kBlock) void refresh(TableView t, int id_bits_unuse
   const uint32_t gl = threadIdx.x % LPR, W = t.width;
   const slot_t o = c.uoff[u];
   const bool got = a.got[u] != 0;
-  const bool remote = o == kNoSlot || (uint32_t)o < t.n_cached;
-  if (gl == 0 && remote) atomicAdd(&stats[o == kNoSlot ? 1 : (got ? 2 : 0)], 1u);
   if (!got || o == kNoSlot) return;
   if ((uint32_t)o >= t.n_cached) { // an owned row can never come back as outdated
     if (gl == 0) atomicOr(&stats[3], 8u);
@@ -248,12 +278,14 @@ void launch_pack_rows(hipStream_t s, const TableView &t, const index_t *rq_idx, 
   HCTR_HIP(hipGetLastError());
 }
 
-void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a, uint32_t *stats) {
-  if (!cur.n || !a.got) return;
+void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
+                    uint32_t *stats) {
+  if (!n_unique || !a.got) return;
+  hipLaunchKernelGGL(count_remote, dim3(kCountBlocks), dim3(kBlock), 0, s, t, cur, a.got, stats);
   const bool vec4 = t.width % 4 == 0;
   const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
 #define CALL(V, L) \
-  hipLaunchKernelGGL((refresh<V, L>), dim3(div_up(cur.n, kBlock / L)), dim3(kBlock), 0, s, t, 0, cur, a, stats)
+  hipLaunchKernelGGL((refresh<V, L>), dim3(div_up(n_unique, kBlock / L)), dim3(kBlock), 0, s, t, cur, a, stats)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   HCTR_HIP(hipGetLastError());

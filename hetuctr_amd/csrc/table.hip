@@ -421,7 +421,7 @@ void Shard::write_back(float *dst) {
     a.ret_i = ret_i.as<uint32_t>();
     a.in_ver = in_ver.as<version_t>();
     a.in_val = in_val.as<embed_t>();
-    launch_refresh(s, tv, cur.view(), a, stats.as<uint32_t>());
+    launch_refresh(s, tv, cur.view(), cur.U, a, stats.as<uint32_t>());
     HCTR_HIP(hipMemcpyAsync(mirror->stats, stats.p, 16, hipMemcpyDeviceToHost, s));
   }
   if (dst != nullptr) {

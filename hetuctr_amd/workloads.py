@@ -15,6 +15,10 @@ CONFIGS = {
     # headline: ~33M rows in 26 log-uniform fields (10 .. 10M), dim 128
     "cfg2": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=1.05, lr=0.05,
                  init=("Normal", 0.0, 0.1), single_field=False),
+    # one GPU's shard of an 8-way partition of the cfg2 table: rank 0 owns 1/8 of the rows and caches the hottest
+    # 10 % of the others; the peers live on the same GPU behind the loopback and only serve rank 0
+    "cfg3": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=1.05, lr=0.05,
+                 init=("Normal", 0.0, 0.1), single_field=False, nrank=8, cache_frac=0.10),
     # large table: 100M rows dim 128 (51.2 GB)
     "cfg4": dict(rows=100_000_000, width=128, samples=131072, fields=26, hot=1, alpha=1.2, lr=0.05,
                  init=("Normal", 0.0, 0.1), single_field=False),
@@ -75,6 +79,35 @@ class KeyStream:
 
     def release_tables(self):
         self._cdf.clear()
+
+
+def shard_layout(ks, nrank, cache_frac, seed=0, cached_ranks=(0,)):
+    """Owner of every id (seeded uniform, as the reference's benchmark draws it, tests/benchmark.py:16) and the
+    resident ids of every rank: a rank in `cached_ranks` stores what it owns plus the hottest `cache_frac` of the ids
+    it does not own (per field the ids of lowest Zipf rank, i.e. the first ids of the field); the others store
+    what they own."""
+    rng = np.random.default_rng(seed + 100)
+    root = rng.integers(0, nrank, size=ks.rows, dtype=np.uint8)
+    storage = [np.flatnonzero(root == r).astype(np.int64) for r in range(nrank)]
+    for r in cached_ranks:
+        hot = []
+        for f in range(ks.fields):
+            lo, c = int(ks.base[f]), int(ks.card[f])
+            ids = np.arange(lo, lo + c, dtype=np.int64)
+            remote = ids[root[lo:lo + c] != r]
+            hot.append(remote[:int(np.ceil(cache_frac * remote.shape[0]))])
+        storage[r] = np.concatenate([storage[r]] + hot)
+    return root, storage
+
+
+def sharded_extra_bytes(width, touched_cached, pushed, received, queried, returned, refreshed):
+    """Bytes a step moves on top of algorithmic_bytes when rows are sharded and cached (same accounting): the
+    pending-gradient store and update counter of touched cached rows, the push buffer and its loopback copy,
+    applying received gradient rows, the query (id, version, directory slot, flag, both ways), packing and
+    returning rows, refreshing cached rows."""
+    row = 4 * width
+    return (touched_cached * (2 * row + 16) + pushed * (row + 2 * row + 32) + received * (2 * row + 32) +
+            queried * 2 * (8 + 8 + 16 + 8) + returned * (2 * row + 2 * row + 8) + refreshed * (3 * row + 8))
 
 
 def algorithmic_bytes(n_keys, n_unique, width):

@@ -107,6 +107,38 @@ def test_stepwise_parity_with_staleness(nrank, bounds, cache, width):
     p.close()
 
 
+@pytest.mark.parametrize("bounds,cached", [((0, 0), (0,)), ((2, 3), tuple(range(8)))])
+def test_partitioned_table_with_hot_row_cache(bounds, cached):
+    # the 8-way partition of the Criteo-like table at 1/100 scale: uniform owners, the hottest 10 % of the remote
+    # rows cached; either rank 0 alone feeds batches while the peers only serve, or every rank does
+    from hetuctr_amd import workloads
+    say("partitioned", bounds, cached)
+    cfg = workloads.CONFIGS["cfg3"]
+    ks = workloads.KeyStream(cfg, seed=0, scale=0.01)
+    R, width = cfg["nrank"], cfg["width"]
+    root, storage = workloads.shard_layout(ks, R, cfg["cache_frac"], cached_ranks=cached)
+    p = Pair(R, ks.rows, width, root, storage, init=("Uniform", -0.1, 0.1), lr=cfg["lr"], bounds=bounds, seed=0)
+    rng = np.random.default_rng(4)
+    prev_n = [0] * R
+    totals = np.zeros(6)
+    for step in range(5):
+        keys = [ks.batch() if r in cached else np.zeros(0, np.int64) for r in range(R)]
+        p.preprocess(keys, device_keys=True)
+        p.compare_ints(INT_ITEMS_PRE, "step %d" % step)
+        out, ref = p.push_pull([rng.normal(0, 1e-2, size=(prev_n[r], width)).astype(np.float32) for r in range(R)])
+        p.compare_ints(INT_ITEMS_POST, "step %d" % step)
+        for r in cached:
+            assert_close(out[r], ref[r], 1e-5, "dst step %d rank %d" % (step, r))
+        for r in range(R):
+            totals += p.tables[r].fetch(capi.STATS)[:6]
+        prev_n = [k.shape[0] for k in keys]
+    p.compare_state(1e-5, "end")
+    hit, miss, refreshed, pushed, returned, received = totals
+    assert hit > 0 and miss > 0 and pushed == received and returned == miss + refreshed
+    assert refreshed > 0                            # at least the first fetch of every touched cached row
+    p.close()
+
+
 def test_hand_computed_staleness_scenario():
     # same scenario as tests/test_oracle_update.py::test_staleness_scenario_both_update, on the GPU
     root = np.array([0, 1], np.uint8)
