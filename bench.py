@@ -31,6 +31,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=3)
     ap.add_argument("--no-stage-timing", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run the library's plain 1 GiB copy kernel (scale factor of the HBM byte counters)")
     ap.add_argument("--active-peers", action="store_true",
                     help="sharded configs: every rank caches hot rows and feeds batches (default: rank 0 only)")
     ap.add_argument("--pull-bound", type=int, default=0, help="sharded configs: staleness bound of pulls")
@@ -178,6 +180,17 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
+    if a.copy_probe:
+        # yardstick for hardware byte counters and for the memory system itself: 1 GiB read + 1 GiB written per launch
+        nbytes = 1 << 30
+        src = torch.ones(nbytes // 4, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        ms = capi.copy_probe(dst.data_ptr(), src.data_ptr(), nbytes, 5)
+        assert bool((dst[:: 1 << 16] == 1).all())
+        print(json.dumps({"probe": "plain_copy", "bytes_read": nbytes, "bytes_written": nbytes, "avg_ms": ms,
+                          "GBps": 2 * nbytes / (ms * 1e-3) / 1e9}), flush=True)
+        return
     cfg = workloads.CONFIGS[a.config]
     if cfg.get("nrank", 1) > 1:
         return main_sharded(a, cfg)

@@ -12,7 +12,7 @@ INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
 SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_push_pull", "hctr_group_preprocess",
            "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch",
            "hctr_stream", "hctr_last_times", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
-           "hctr_stage_times", "hctr_version"]
+           "hctr_stage_times", "hctr_copy_probe", "hctr_version"]
 
 # items of hctr_debug_fetch (HCTR_F_*)
 UNIQUE, SORTED_ARG, RUN_START, IDX_MAP, ROOT, OFFSET, SEND_CNT, RECV_CNT = range(8)
@@ -56,6 +56,7 @@ def lib():
         l.hctr_stage_name.argtypes = [C.c_int]
         l.hctr_stage_name.restype = C.c_char_p
         l.hctr_stage_times.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        l.hctr_copy_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
         _lib = l
     return _lib
 
@@ -67,6 +68,13 @@ def _check(rc):
 
 def seed(n):
     lib().hctr_seed(int(n))
+
+
+def copy_probe(dst_ptr, src_ptr, nbytes, repeats=5):
+    """Average ms of a plain device copy of nbytes (read nbytes + write nbytes per launch)."""
+    ms = C.c_float(0)
+    _check(lib().hctr_copy_probe(dst_ptr, src_ptr, nbytes, repeats, C.byref(ms)))
+    return ms.value
 
 
 class Table:

@@ -183,5 +183,24 @@ int hctr_stage_times(hctr_table *t, double *ms_total, long long *launches, int c
   });
 }
 
+int hctr_copy_probe(void *dst, const void *src, size_t bytes, int repeats, float *ms_avg) {
+  return guarded([&] {
+    HCTR_CHECK(dst && src && bytes % 16 == 0 && repeats >= 1, "copy probe: device pointers, bytes a multiple of 16");
+    hipEvent_t a, b;
+    HCTR_HIP(hipEventCreate(&a));
+    HCTR_HIP(hipEventCreate(&b));
+    launch_plain_copy(nullptr, src, dst, bytes); // untimed first launch
+    HCTR_HIP(hipEventRecord(a, nullptr));
+    for (int i = 0; i < repeats; i++) launch_plain_copy(nullptr, src, dst, bytes);
+    HCTR_HIP(hipEventRecord(b, nullptr));
+    HCTR_HIP(hipEventSynchronize(b));
+    float ms = 0.f;
+    HCTR_HIP(hipEventElapsedTime(&ms, a, b));
+    if (ms_avg) *ms_avg = ms / repeats;
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+  });
+}
+
 #pragma GCC visibility pop
 } // extern "C"

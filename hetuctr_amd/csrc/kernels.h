@@ -142,5 +142,6 @@ void launch_build_directory(hipStream_t s, const index_t *store_ids, uint32_t n_
 // segmented copies of an exchange: n descriptors {src, dst, bytes}
 struct CopyDesc { const void *src; void *dst; size_t bytes; };
 void launch_copies(hipStream_t s, const CopyDesc *descs_device, uint32_t n, size_t max_bytes);
+void launch_plain_copy(hipStream_t s, const void *src, void *dst, size_t bytes); // bytes % 16 == 0
 
 } // namespace hctr

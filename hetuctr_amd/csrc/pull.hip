@@ -204,6 +204,12 @@ __global__ __launch_bounds__(kBlock) void copy_segments(const CopyDesc *__restri
   }
 }
 
+// plain 16-byte-lane copy of known size: the yardstick the HBM byte counters are scaled with
+__global__ __launch_bounds__(kBlock) void plain_copy(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 inline int lanes_for(uint32_t width, int vec) {
   const uint32_t lanes = (width + vec - 1) / vec;
   return lanes <= 4 ? 4 : lanes <= 8 ? 8 : lanes <= 16 ? 16 : lanes <= 32 ? 32 : 64;
@@ -304,6 +310,11 @@ void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, cons
   } while (0)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_plain_copy(hipStream_t s, const void *src, void *dst, size_t bytes) {
+  hipLaunchKernelGGL(plain_copy, dim3(256 * 16), dim3(kBlock), 0, s, (const uint4 *)src, (uint4 *)dst, bytes / 16);
   HCTR_HIP(hipGetLastError());
 }
 

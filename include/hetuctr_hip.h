@@ -112,6 +112,11 @@ int hctr_stage_count(void);
 const char *hctr_stage_name(int stage);
 int hctr_stage_times(hctr_table *t, double *ms_total, long long *launches, int cap);
 
+/* Measurement aid without a counterpart in the reference: copies `bytes` (a multiple of 16) of device memory with a
+ * plain 16-byte-lane kernel on the default stream, 1 + repeats times, and reports the average duration.  A launch
+ * reads and writes exactly `bytes`, which is what hardware byte counters are scaled against. */
+int hctr_copy_probe(void *dst, const void *src, size_t bytes, int repeats, float *ms_avg);
+
 /* Version string of the library. */
 const char *hctr_version(void);
 
