@@ -26,7 +26,7 @@ struct BatchView {
   slot_t *uoff;              // [U]   resident offset of rank u or -1           (d_offset)
   uint32_t *bucket_lo;       // [R+1] first rank owned by each shard            (u_shape before :131)
   uint32_t *d_U;             // [1]   number of unique keys                     (unique_size)
-  uint32_t *long_list;       // [kLongBuckets][long_cap] unique ranks whose run is longer than kLongRun, by length class
+  uint4 *long_list;          // [kLongBuckets][long_cap] runs longer than kLongRun by length class: {unique rank, first sorted position, length, resident offset}
   uint32_t *d_nlong;         // [kLongBuckets] entries per class, then [kLongBuckets]: work counter of the push
   uint32_t long_cap;         // capacity of one class
   uint32_t *med_list;        // [d_nlong[kMedCount]] unique ranks with kTinyRun < run length <= kLongRun (any order)
@@ -34,7 +34,7 @@ struct BatchView {
 
 // d_nlong layout: [0, kLongBuckets) long runs per class, then the long work counter, the number of medium runs
 // and the medium work counter
-constexpr int kLongWork = 8, kMedCount = 9, kMedWork = 10, kRunCounters = 11;
+constexpr int kLongWork = 8, kMedCount = 9, kMedWork = 10, kTicketBase = 11, kTicketLanes = 16, kRunCounters = kTicketBase + 2 * kTicketLanes;
 
 // A run of equal keys longer than this is summed by a whole block that streams its gradient rows through
 // LDS; shorter runs are summed by a small group of lanes.

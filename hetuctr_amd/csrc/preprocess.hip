@@ -152,7 +152,8 @@ __global__ __launch_bounds__(kBlock) void list_long_runs(BatchView b) {
     base[threadIdx.x] = atomicAdd(&b.d_nlong[threadIdx.x < kLongBuckets ? threadIdx.x : kMedCount], cnt[threadIdx.x]);
   __syncthreads();
   if (list >= 0) {
-    if (list < kLongBuckets) b.long_list[(size_t)list * b.long_cap + base[list] + local] = u;
+    if (list < kLongBuckets)
+      b.long_list[(size_t)list * b.long_cap + base[list] + local] = make_uint4(u, b.run_start[u], len, (uint32_t)b.uoff[u]);
     else b.med_list[base[list] + local] = u;
   }
 }

@@ -19,6 +19,7 @@
 //  * medium (kTinyRun < duplicates <= kLongRun): one group of LPR lanes per run, kBatch rows in flight.
 //  * short (<= kTinyRun): a group of LPR lanes (LPR*VEC floats = one row) owns a few consecutive unique keys
 //    and sums their runs, all first loads of the group issued together.
+#include <algorithm>
 #include "kernels.h"
 
 namespace hctr {
@@ -62,7 +63,21 @@ constexpr int kRPT = HCTR_RPT;            // long role: rows per loader thread a
 constexpr int kSlots = HCTR_SLOTS;        // long role: LDS ring slots
 constexpr int kSlice = HCTR_SLICE;        // long role: columns per block
 constexpr int kLongBlocks = HCTR_LONG_BLOCKS;
+#ifndef HCTR_GIANT_BLOCKS
+#define HCTR_GIANT_BLOCKS 96
+#endif
+#ifndef HCTR_GIANT_SLICE
+#define HCTR_GIANT_SLICE 32
+#endif
+#ifndef HCTR_GIANT_CLASSES
+#define HCTR_GIANT_CLASSES 2
+#endif
+constexpr int kGiantBlocks = HCTR_GIANT_BLOCKS;   // long role: blocks for the longest runs ...
+constexpr int kGiantSlice = HCTR_GIANT_SLICE;     // ... which are cut into slices of this many columns
+constexpr int kGiantClasses = HCTR_GIANT_CLASSES; // ... and are the runs of the first length classes (>= 4096)
+static_assert(kSlice % kGiantSlice == 0 && kGiantBlocks < kLongBlocks, "tiers of the long role");
 constexpr int kMedBlocks = HCTR_MED_BLOCKS;
+
 
 
 namespace {
@@ -305,17 +320,29 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
 }
 
 // ---- long role -----------------------------------------------------------------------------------------
-// Work item = (long run, column slice of CS columns), handed out longest class first through a counter.
+// A block works on ONE column slice (CS columns) of a bundle of long runs at a time and treats the bundle as one
+// stream of chunks, so that the loads of the next run are in flight while the current one is summed.  Runs are
+// listed by length class, longest first; a bundle is 1..kTable runs of one class holding at least ~2048
+// occurrences.  Tickets (bundle, slice) are handed out through one counter per group of blocks that share slices;
+// the summing wave draws the next ticket and requests its run descriptors while the current bundle streams, so a
+// change of bundle costs only the refill of the load pipeline.
 // Wave 0 of the block only sums; the other 7 waves ("loaders") only move gradient rows global -> registers ->
 // LDS ring.  A row slice is read by CS/VEC loader lanes; one block-wide load covers RPL = 448 / (CS/VEC)
-// consecutive occurrences and a chunk is kRPT such loads.  Loaders and the summing wave meet at one barrier
-// per chunk: barrier m says "chunk m is in LDS".  A slot is overwritten kSlots barriers later, after the
-// summing wave has passed the barrier that follows its reads.
+// consecutive occurrences and a chunk is kRPT such loads (chunks never span two runs).  Loaders and the summing
+// wave meet at one barrier per chunk: barrier m says "chunk m is in LDS".  A slot is overwritten kSlots
+// barriers later, after the summing wave has passed the barrier that follows its reads.
 constexpr int kLoaders = kPushBlock - kWave;
+constexpr int kTable = 16;     // runs per bundle at most
+constexpr int kSumBatch = 56;  // rows the summing wave reads from LDS in one go
 
-template <int VEC, typename K, int CSC> // CSC: columns per slice if known at compile time (64), else 0
+__device__ __forceinline__ uint32_t bundle_runs(int cls) { // runs per bundle: classes halve in length
+  return cls <= 2 ? 1u : min(1u << (cls - 2), (uint32_t)kTable);
+}
+
+template <int VEC, typename K, int CSC> // CSC: columns per slice if known at compile time, else 0
 __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
-                                          float *lds, uint32_t *next_item) {
+                                          float *lds, uint4 *table, uint32_t *shared, int c_lo, int c_hi,
+                                          uint32_t bidx, uint32_t nblk, uint32_t *counters) {
   typedef typename Vec<VEC>::T V;
   const uint32_t W = t.width;
   const uint32_t CS = CSC ? (uint32_t)CSC : min((uint32_t)kSlice, (W + VEC - 1) / VEC * VEC);
@@ -324,89 +351,142 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
   const uint32_t RPL = CSC ? (uint32_t)(kLoaders / (CSC / VEC)) : kLoaders / lanes;
   const uint32_t CR = RPL * kRPT;                                   // rows per chunk
   constexpr int kChunkRows = CSC ? kRPT * (kLoaders / (CSC / VEC)) : 1; // CR as a constant on the fast path
+  static_assert(!CSC || kChunkRows % kSumBatch == 0, "a chunk of the fast path is a whole number of sum batches");
   const uint32_t slices = (W + CS - 1) / CS;
   const uint32_t slot_floats = CR * CS;
   const float neg_lr = t.neg_lr;
   const bool summer = threadIdx.x < kWave;
   const uint32_t lt = threadIdx.x - kWave; // loader thread number (meaningless on the summing wave)
   const uint32_t my_row = lt / lanes, my_lane = lt % lanes;
-  uint32_t class_end[kLongBuckets]; // items up to and including each length class
-  {
-    uint32_t run = 0;
+  const uint32_t *__restrict__ sorted_arg = p.sorted_arg;
+
+  // tickets of this block's group: (bundle, slice) with the bundle changing slowest, so the longest runs go first
+  const uint32_t share = min(min(slices, nblk), (uint32_t)kTicketLanes);
+  const uint32_t lane_id = bidx % share;
+  const uint32_t n_sl = (slices - lane_id + share - 1) / share; // slices lane_id, lane_id + share, ...
+  uint32_t cnt[kLongBuckets];
+  uint32_t nbundles = 0;
+#pragma unroll
+  for (int c = 0; c < kLongBuckets; c++) {
+    cnt[c] = (c >= c_lo && c < c_hi) ? p.d_nlong[c] : 0u;
+    nbundles += (cnt[c] + bundle_runs(c) - 1) / bundle_runs(c);
+  }
+  if (!nbundles) return;
+  const uint32_t tickets = nbundles * n_sl;
+
+  // summing wave: draws a ticket and requests the descriptors of its runs (one lane per run)
+  uint4 pend = make_uint4(0, 0, 0, 0);
+  uint32_t pend_runs = 0, pend_slice = 0;
+  auto draw = [&]() {
+    uint32_t tk = 0;
+    if (threadIdx.x == 0) tk = atomicAdd(counters + lane_id, 1u);
+    tk = (uint32_t)__builtin_amdgcn_readfirstlane((int)tk);
+    pend_runs = 0;
+    if (tk >= tickets) return;
+    uint32_t bundle = tk / n_sl;
+    pend_slice = lane_id + (tk % n_sl) * share;
+    int cls = 0;
+    uint32_t run0 = 0;
+    bool found = false;
 #pragma unroll
     for (int c = 0; c < kLongBuckets; c++) {
-      run += p.d_nlong[c] * slices;
-      class_end[c] = run;
-    }
-  }
-  const uint32_t items = class_end[kLongBuckets - 1];
-
-  for (;;) {
-    if (threadIdx.x == 0) *next_item = atomicAdd(&p.d_nlong[kLongWork], 1u);
-    __syncthreads();
-    const uint32_t item = *next_item;
-    __syncthreads();
-    if (item >= items) break;
-    int cls = 0;
-    uint32_t first = 0;
-#pragma unroll
-    for (int c = 0; c < kLongBuckets - 1; c++)
-      if (item >= class_end[c]) {
-        cls = c + 1;
-        first = class_end[c];
+      const uint32_t bs = bundle_runs(c), nb = (cnt[c] + bs - 1) / bs;
+      if (!found) {
+        if (bundle < nb) {
+          found = true;
+          cls = c;
+          run0 = bundle * bs;
+          pend_runs = min(bs, cnt[c] - run0);
+        } else {
+          bundle -= nb;
+        }
       }
-    const uint32_t u = p.long_list[(size_t)cls * p.long_cap + (item - first) / slices];
-    const uint32_t slice = (item - first) % slices;
-    const uint32_t lo = p.run_start[u], hi = p.run_start[u + 1];
-    const uint32_t L = hi - lo;
-    const uint32_t nchunks = (L + CR - 1) / CR;
+    }
+    if (threadIdx.x < pend_runs) pend = p.long_list[(size_t)cls * p.long_cap + run0 + threadIdx.x];
+  };
+  // ... and makes them the block's current bundle: descriptors, number of runs, chunks and the slice
+  auto publish = [&]() {
+    uint32_t chunks = threadIdx.x < pend_runs ? (pend.z + CR - 1) / CR : 0u;
+    if (threadIdx.x < pend_runs) table[threadIdx.x] = pend; // rank, first position, length, offset
+#pragma unroll
+    for (int d = kTable / 2; d; d >>= 1) chunks += __shfl_down(chunks, d);
+    if (threadIdx.x == 0) {
+      shared[0] = pend_runs;
+      shared[1] = chunks;
+      shared[2] = pend_slice;
+    }
+  };
+
+  if (summer) draw();
+  for (;;) {
+    if (summer) publish();
+    __syncthreads();
+    const uint32_t J = shared[0], G = shared[1], slice = shared[2]; // runs, chunks and slice of this bundle
+    if (!J) break;
+    if (summer) draw(); // the requests stay in flight while this bundle streams
+
     if (!summer) {
       // ---------------- loaders ----------------
       const uint32_t lcol = my_lane * VEC; // column inside the slice
       const uint32_t col = slice * CS + lcol;
       const bool in_slice = lcol < CS && my_row < RPL;
       // Loads are unconditional and branch-free so that kDepth chunks stay in flight per thread: positions
-      // past the end of the run re-read its last row (never summed), lanes outside the slice read column 0.
+      // past the end of a run re-read its last row (never summed), lanes outside the slice read column 0.
       const embed_t *gbase = a.grad + ((in_slice && col < W) ? col : 0);
-      auto row_index = [&](uint32_t c, int q) -> uint32_t {
-        return p.sorted_arg[min(lo + c * CR + q * RPL + my_row, hi - 1)];
-      };
       auto row_load = [&](uint32_t idx) -> V { return *(const V *)(gbase + (size_t)idx * W); };
+      // cursor of the index stage, 2 * kDepth chunks ahead of the LDS stage; past the end of the stream it
+      // stays on the last run
+      uint32_t cj = 0, cc = 0;
+      uint32_t clo, chi, cn;
+      {
+        const uint4 m = table[0];
+        clo = m.y;
+        chi = m.y + m.z;
+        cn = (m.z + CR - 1) / CR;
+      }
+      auto next_chunk = [&](uint32_t(&dst)[kRPT]) {
+#pragma unroll
+        for (int q = 0; q < kRPT; q++) dst[q] = sorted_arg[min(clo + cc * CR + q * RPL + my_row, chi - 1)];
+        cc++;
+        if (cc >= cn && cj + 1 < J) {
+          cj++;
+          const uint4 m = table[cj];
+          clo = m.y;
+          chi = m.y + m.z;
+          cn = (m.z + CR - 1) / CR;
+          cc = 0;
+        }
+      };
       uint32_t idx_a[kDepth][kRPT], idx_b[kDepth][kRPT];
       V val[kDepth][kRPT];
 #pragma unroll
-      for (int k = 0; k < kDepth; k++)
+      for (int k = 0; k < kDepth; k++) next_chunk(idx_a[k]);
 #pragma unroll
-        for (int q = 0; q < kRPT; q++) idx_a[k][q] = row_index(k, q);
-#pragma unroll
-      for (int k = 0; k < kDepth; k++)
-#pragma unroll
-        for (int q = 0; q < kRPT; q++) idx_b[k][q] = row_index(kDepth + k, q);
+      for (int k = 0; k < kDepth; k++) next_chunk(idx_b[k]);
 #pragma unroll
       for (int k = 0; k < kDepth; k++)
 #pragma unroll
         for (int q = 0; q < kRPT; q++) val[k][q] = row_load(idx_a[k][q]);
-      // invariant at the top of a round: val[k] holds chunk c0+k, idx_b[k] the row indices of chunk c0+kDepth+k
-      for (uint32_t c0 = 0; c0 < nchunks; c0 += kDepth) {
+      // invariant at the top of a round: val[k] holds chunk g0+k, idx_b[k] the row indices of chunk g0+kDepth+k
+      uint32_t slot = 0;
+      for (uint32_t g0 = 0; g0 < G; g0 += kDepth) {
 #pragma unroll
         for (int k = 0; k < kDepth; k++)
 #pragma unroll
           for (int q = 0; q < kRPT; q++) idx_a[k][q] = idx_b[k][q];
 #pragma unroll
-        for (int k = 0; k < kDepth; k++)
-#pragma unroll
-          for (int q = 0; q < kRPT; q++) idx_b[k][q] = row_index(c0 + 2 * kDepth + k, q);
+        for (int k = 0; k < kDepth; k++) next_chunk(idx_b[k]);
 #pragma unroll
         for (int k = 0; k < kDepth; k++) {
-          const uint32_t c = c0 + k;
-          if (c < nchunks) { // uniform over the block: the summing wave makes the same number of barriers
-            float *slot = lds + (c % kSlots) * slot_floats;
+          if (g0 + k < G) { // uniform over the block: the summing wave makes the same number of barriers
+            float *sp = lds + slot * slot_floats;
+            slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
 #pragma unroll
             for (int q = 0; q < kRPT; q++) {
-              if (in_slice) *(V *)(slot + (q * RPL + my_row) * CS + lcol) = val[k][q];
-              val[k][q] = row_load(idx_a[k][q]); // chunk c + kDepth
+              if (in_slice) *(V *)(sp + (q * RPL + my_row) * CS + lcol) = val[k][q];
+              val[k][q] = row_load(idx_a[k][q]); // chunk g0 + k + kDepth
             }
-            __syncthreads(); // barrier c
+            __syncthreads(); // barrier g0 + k
           }
         }
       }
@@ -415,41 +495,58 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
 #if HCTR_SUM_PRIO
       __builtin_amdgcn_s_setprio(HCTR_SUM_PRIO); // the chain of this wave is the critical path of the whole push
 #endif
-      float acc = 0.f;
-      const uint32_t nfull = L / CR; // chunks with all CR rows
-      uint32_t c = 0;
-      if (CSC) {
-        for (; c < nfull; c++) {
-          __syncthreads(); // barrier c
-          const float *sp = lds + (c % kSlots) * slot_floats + threadIdx.x;
-          float x[kChunkRows];
+      const uint32_t mycol = slice * CS + threadIdx.x;
+      const bool col_ok = threadIdx.x < CS && mycol < W;
+      const bool direct = t.nrank == 1; // every key is owned and resident; the version counters move elsewhere
+      uint32_t slot = 0;
+      for (uint32_t j = 0; j < J; j++) {
+        const uint4 m = table[j];
+        const uint32_t L = m.z;
+        const uint32_t nfull = L / CR, nch = (L + CR - 1) / CR;
+        float e = 0.f;
+        if (direct && col_ok) e = t.emb[(size_t)m.w * W + mycol]; // needed only after the last chunk
+        float acc = 0.f; // the reference starts every sum from 0
+        uint32_t c = 0;
+        if (CSC) {
+          for (; c < nfull; c++) {
+            __syncthreads(); // barrier of this chunk
+            const float *sp = lds + slot * slot_floats + (threadIdx.x < CS ? threadIdx.x : 0);
+            slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
 #pragma unroll
-          for (int q = 0; q < kChunkRows; q++) x[q] = sp[q * CSC];
+            for (int r0 = 0; r0 < kChunkRows; r0 += kSumBatch) {
+              float x[kSumBatch];
 #pragma unroll
-          for (int q = 0; q < kChunkRows; q++) acc += x[q];
-        }
-      }
-      for (; c < nchunks; c++) { // generic path, and the partial last chunk of the fast path
-        __syncthreads();         // barrier c
-        if (threadIdx.x < CS) {
-          const float *col_ptr = lds + (c % kSlots) * slot_floats + threadIdx.x;
-          const uint32_t rows = min(CR, L - c * CR);
-          uint32_t r = 0;
-          for (; r + 8 <= rows; r += 8) {
-            float x[8];
+              for (int q = 0; q < kSumBatch; q++) x[q] = sp[(r0 + q) * (CSC ? CSC : 1)];
 #pragma unroll
-            for (int q = 0; q < 8; q++) x[q] = col_ptr[(r + q) * CS];
-#pragma unroll
-            for (int q = 0; q < 8; q++) acc += x[q];
+              for (int q = 0; q < kSumBatch; q++) acc += x[q];
+            }
           }
-          for (; r < rows; r++) acc += col_ptr[r * CS];
+        }
+        for (; c < nch; c++) { // generic path, and the partial last chunk of the fast path
+          __syncthreads();     // barrier of this chunk
+          const float *col_ptr = lds + slot * slot_floats + threadIdx.x;
+          slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
+          if (threadIdx.x < CS) {
+            const uint32_t rows = min(CR, L - c * CR);
+            uint32_t r = 0;
+            for (; r + 8 <= rows; r += 8) {
+              float x[8];
+#pragma unroll
+              for (int q = 0; q < 8; q++) x[q] = col_ptr[(r + q) * CS];
+#pragma unroll
+              for (int q = 0; q < 8; q++) acc += x[q];
+            }
+            for (; r < rows; r++) acc += col_ptr[r * CS];
+          }
+        }
+        if (col_ok) {
+          const float scaled = acc * neg_lr;
+          if (direct) t.emb[(size_t)m.w * W + mycol] = e + scaled;
+          else apply_row<1, K>(t, id_bits, p, a, m.x, scaled, mycol, slice == 0 && threadIdx.x == 0);
         }
       }
-      // single shard: the version counters are moved by bump_versions, not here
-      if (threadIdx.x < CS && slice * CS + threadIdx.x < W)
-        apply_row<1, K>(t, id_bits, p, a, u, acc * neg_lr, slice * CS + threadIdx.x,
-                        t.nrank > 1 && slice == 0 && threadIdx.x == 0);
     }
+    __syncthreads(); // everybody is done with the table and the ring
   }
 }
 
@@ -465,12 +562,25 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
   constexpr int kRingWords = kSlots * kRPT * kPushBlock * VEC;
   constexpr int kStageWords = (kPushBlock / LPR) * (int)kLongRun;
   __shared__ __align__(16) float lds[kRingWords > kStageWords ? kRingWords : kStageWords];
-  __shared__ uint32_t next_item;
+  __shared__ uint4 run_table[kTable];
+  __shared__ uint32_t run_totals[3];
   if (blockIdx.x < kLongBlocks) {
     if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 1) return;
-    if (VEC == 4 && t.width % kSlice == 0) long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, &next_item);
-    else long_role<VEC, K, 0>(t, id_bits, p, a, lds, &next_item);
-  } else if (blockIdx.x < kLongBlocks + kMedBlocks) {
+    // the longest runs are cut into narrower column slices, worked on by more blocks: the blocks of a saturated
+    // memory system get equal shares of it, and a chain advances with the share of the block that feeds it
+    uint32_t *tk = p.d_nlong + kTicketBase;
+    if (VEC == 4 && t.width % kSlice == 0) {
+      if (blockIdx.x < kGiantBlocks)
+        long_role<VEC, K, (VEC == 4 ? kGiantSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, 0, kGiantClasses,
+                                                        blockIdx.x, kGiantBlocks, tk);
+      else
+        long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, kGiantClasses,
+                                                   kLongBuckets, blockIdx.x - kGiantBlocks, kLongBlocks - kGiantBlocks,
+                                                   tk + kTicketLanes);
+    } else {
+      long_role<VEC, K, 0>(t, id_bits, p, a, lds, run_table, run_totals, 0, kLongBuckets, blockIdx.x, kLongBlocks, tk);
+    }
+  } else if (blockIdx.x < kLongBlocks + kMedBlocks) { // medium runs take long per block: they start early
     if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 3) return;
     medium_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, (uint32_t *)lds, blockIdx.x - kLongBlocks, kMedBlocks);
   } else {
@@ -493,9 +603,9 @@ template <int VEC, int LPR, typename K, bool kSingle>
 void launch_push_t(hipStream_t st, const TableView &t, int id_bits, const BatchView &p, uint32_t U, const PushArgs &a) {
   constexpr int kGroups = kPushBlock / LPR;
   const unsigned ver_blocks = kSingle ? div_up(U, kPushBlock) : 0; // version counters of a single shard
-  hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle>),
-                     dim3(kLongBlocks + kMedBlocks + div_up(U, kGroups * kRunsPerGroup) + ver_blocks), dim3(kPushBlock), 0,
-                     st, t, id_bits, p, a, U);
+  const unsigned rest = kMedBlocks + div_up(U, kGroups * kRunsPerGroup) + ver_blocks;
+  hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle>), dim3(kLongBlocks + rest), dim3(kPushBlock), 0, st, t, id_bits, p,
+                     a, U);
 }
 
 template <int VEC, typename K, bool kSingle>

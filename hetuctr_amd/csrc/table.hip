@@ -38,7 +38,7 @@ void Batch::reserve(uint32_t n_keys, int nrank, bool wide) {
   uoff.reserve(n * sizeof(slot_t));
   bucket_lo.reserve((size_t)(nrank + 1) * 4);
   dU.reserve(4);
-  long_list.reserve(long_list_capacity((uint32_t)n) * 4 * kLongBuckets);
+  long_list.reserve(long_list_capacity((uint32_t)n) * sizeof(uint4) * kLongBuckets);
   dnlong.reserve(4 * kRunCounters);
   med_list.reserve(med_list_capacity((uint32_t)n) * 4);
 }
@@ -55,7 +55,7 @@ BatchView Batch::view() const {
   v.uoff = uoff.as<slot_t>();
   v.bucket_lo = bucket_lo.as<uint32_t>();
   v.d_U = dU.as<uint32_t>();
-  v.long_list = long_list.as<uint32_t>();
+  v.long_list = long_list.as<uint4>();
   v.d_nlong = dnlong.as<uint32_t>();
   v.long_cap = (uint32_t)long_list_capacity(std::max<uint32_t>(n, 1));
   v.med_list = med_list.as<uint32_t>();
