@@ -27,14 +27,16 @@ struct BatchView {
   uint32_t *bucket_lo;       // [R+1] first rank owned by each shard            (u_shape before :131)
   uint32_t *d_U;             // [1]   number of unique keys                     (unique_size)
   uint4 *long_list;          // [kLongBuckets][long_cap] runs longer than kLongRun by length class: {unique rank, first sorted position, length, resident offset}
-  uint32_t *d_nlong;         // [kLongBuckets] entries per class, then [kLongBuckets]: work counter of the push
+  uint32_t *d_nlong;         // [kRunCounters] entries per class of long runs, then counters of the push
   uint32_t long_cap;         // capacity of one class
   uint32_t *med_list;        // [d_nlong[kMedCount]] unique ranks with kTinyRun < run length <= kLongRun (any order)
 };
 
-// d_nlong layout: [0, kLongBuckets) long runs per class, then the long work counter, the number of medium runs
-// and the medium work counter
-constexpr int kLongWork = 8, kMedCount = 9, kMedWork = 10, kTicketBase = 11, kTicketLanes = 16, kRunCounters = kTicketBase + 2 * kTicketLanes;
+// d_nlong layout: [0, kLongBuckets) long runs per class, then the number of medium runs, the medium work counter
+// and the ticket counters of the long role
+constexpr int kLongBuckets = 12;
+constexpr int kMedCount = kLongBuckets, kMedWork = kLongBuckets + 1, kTicketBase = kLongBuckets + 2, kTicketLanes = 16,
+              kRunCounters = kTicketBase + 2 * kTicketLanes;
 
 // A run of equal keys longer than this is summed by a whole block that streams its gradient rows through
 // LDS; shorter runs are summed by a small group of lanes.
@@ -47,11 +49,13 @@ constexpr uint32_t kLongRun = HCTR_LONG_RUN;
 #endif
 constexpr uint32_t kTinyRun = HCTR_TINY_RUN; // runs up to this length are summed by the group that owns their rank
 // Long runs are listed by length class (class 0 = longest) so that the push can start the longest chains first.
-constexpr int kLongBuckets = 8;
 inline size_t long_list_capacity(uint32_t n) { return n / (kLongRun + 1) + 1; }
 inline size_t med_list_capacity(uint32_t n) { return n / (kTinyRun + 1) + 1; }
 __host__ __device__ inline int long_bucket(uint32_t len) {
-  return len >= 8192 ? 0 : len >= 4096 ? 1 : len >= 2048 ? 2 : len >= 1024 ? 3 : len >= 512 ? 4 : len >= 256 ? 5 : 6;
+  // class c holds lengths in [2^(17-c), 2^(18-c)), the first everything from 2^17 up, the last everything below 256
+  int c = 0;
+  for (uint32_t lim = 1u << 17; c < kLongBuckets - 1 && len < lim; lim >>= 1) c++;
+  return c;
 }
 
 struct TableView {

@@ -63,19 +63,15 @@ constexpr int kRPT = HCTR_RPT;            // long role: rows per loader thread a
 constexpr int kSlots = HCTR_SLOTS;        // long role: LDS ring slots
 constexpr int kSlice = HCTR_SLICE;        // long role: columns per block
 constexpr int kLongBlocks = HCTR_LONG_BLOCKS;
-#ifndef HCTR_GIANT_BLOCKS
-#define HCTR_GIANT_BLOCKS 96
-#endif
 #ifndef HCTR_GIANT_SLICE
 #define HCTR_GIANT_SLICE 32
 #endif
 #ifndef HCTR_GIANT_CLASSES
-#define HCTR_GIANT_CLASSES 2
+#define HCTR_GIANT_CLASSES 6
 #endif
-constexpr int kGiantBlocks = HCTR_GIANT_BLOCKS;   // long role: blocks for the longest runs ...
-constexpr int kGiantSlice = HCTR_GIANT_SLICE;     // ... which are cut into slices of this many columns
-constexpr int kGiantClasses = HCTR_GIANT_CLASSES; // ... and are the runs of the first length classes (>= 4096)
-static_assert(kSlice % kGiantSlice == 0 && kGiantBlocks < kLongBlocks, "tiers of the long role");
+constexpr int kGiantSlice = HCTR_GIANT_SLICE;     // long role: the longest runs are cut into slices of this many columns;
+constexpr int kGiantClasses = HCTR_GIANT_CLASSES; // they are the runs of the first length classes (>= 4096)
+static_assert(kSlice % kGiantSlice == 0, "tiers of the long role");
 constexpr int kMedBlocks = HCTR_MED_BLOCKS;
 
 
@@ -333,10 +329,22 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
 // barriers later, after the summing wave has passed the barrier that follows its reads.
 constexpr int kLoaders = kPushBlock - kWave;
 constexpr int kTable = 16;     // runs per bundle at most
-constexpr int kSumBatch = 56;  // rows the summing wave reads from LDS in one go
+#ifndef HCTR_SUM_BATCH
+#define HCTR_SUM_BATCH 28
+#endif
+constexpr int kSumBatch = HCTR_SUM_BATCH; // rows the summing wave reads from LDS in one go (two such batches are live)
+
+// the four floats of v to dst[0], dst[stride], dst[2 * stride], dst[3 * stride]
+__device__ __forceinline__ void store_transposed(float *dst, uint32_t stride, const float4 &v) {
+  dst[0] = v.x, dst[stride] = v.y, dst[2 * stride] = v.z, dst[3 * stride] = v.w;
+}
+__device__ __forceinline__ void store_transposed(float *, uint32_t, const float &) {} // generic path: never called
+
+// a value that is the same in every lane, moved to a scalar register
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
 __device__ __forceinline__ uint32_t bundle_runs(int cls) { // runs per bundle: classes halve in length
-  return cls <= 2 ? 1u : min(1u << (cls - 2), (uint32_t)kTable);
+  return cls <= 6 ? 1u : min(1u << (cls - 6), (uint32_t)kTable); // one run of 2048 or more, 2 of 1024.., 4, 8, 16
 }
 
 template <int VEC, typename K, int CSC> // CSC: columns per slice if known at compile time, else 0
@@ -351,9 +359,15 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
   const uint32_t RPL = CSC ? (uint32_t)(kLoaders / (CSC / VEC)) : kLoaders / lanes;
   const uint32_t CR = RPL * kRPT;                                   // rows per chunk
   constexpr int kChunkRows = CSC ? kRPT * (kLoaders / (CSC / VEC)) : 1; // CR as a constant on the fast path
-  static_assert(!CSC || kChunkRows % kSumBatch == 0, "a chunk of the fast path is a whole number of sum batches");
+  static_assert(!CSC || (kChunkRows % kSumBatch == 0 && kSumBatch % 4 == 0), "a chunk of the fast path is a whole number of sum batches");
+  static_assert(!CSC || kSlots * CSC * (kChunkRows + 4) <= kSlots * kRPT * kPushBlock * VEC, "ring slots of the fast path fit the LDS area");
   const uint32_t slices = (W + CS - 1) / CS;
-  const uint32_t slot_floats = CR * CS;
+  // LDS layout of a ring slot.  Generic path: row-major [row][CS].  Fast path (CSC): column-major with the row
+  // index fastest, [column place][pitch], pitch = rows + 4, so that the summing lane gets four consecutive rows of
+  // its column with one 16-byte read; column c sits at place (c % 4) * (CSC / 4) + c / 4, which makes both the
+  // loaders' 4-byte writes and the 16-byte reads free of bank conflicts (pitch % 8 == 4).
+  const uint32_t pitch = CR + 4;
+  const uint32_t slot_floats = CSC ? CS * pitch : CR * CS;
   const float neg_lr = t.neg_lr;
   const bool summer = threadIdx.x < kWave;
   const uint32_t lt = threadIdx.x - kWave; // loader thread number (meaningless on the summing wave)
@@ -368,7 +382,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
   uint32_t nbundles = 0;
 #pragma unroll
   for (int c = 0; c < kLongBuckets; c++) {
-    cnt[c] = (c >= c_lo && c < c_hi) ? p.d_nlong[c] : 0u;
+    cnt[c] = (c >= c_lo && c < c_hi) ? uni(p.d_nlong[c]) : 0u;
     nbundles += (cnt[c] + bundle_runs(c) - 1) / bundle_runs(c);
   }
   if (!nbundles) return;
@@ -421,7 +435,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
   for (;;) {
     if (summer) publish();
     __syncthreads();
-    const uint32_t J = shared[0], G = shared[1], slice = shared[2]; // runs, chunks and slice of this bundle
+    const uint32_t J = uni(shared[0]), G = uni(shared[1]), slice = uni(shared[2]); // runs, chunks and slice of this bundle
     if (!J) break;
     if (summer) draw(); // the requests stay in flight while this bundle streams
 
@@ -440,9 +454,9 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       uint32_t clo, chi, cn;
       {
         const uint4 m = table[0];
-        clo = m.y;
-        chi = m.y + m.z;
-        cn = (m.z + CR - 1) / CR;
+        clo = uni(m.y);
+        chi = clo + uni(m.z);
+        cn = (uni(m.z) + CR - 1) / CR;
       }
       auto next_chunk = [&](uint32_t(&dst)[kRPT]) {
 #pragma unroll
@@ -451,31 +465,25 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
         if (cc >= cn && cj + 1 < J) {
           cj++;
           const uint4 m = table[cj];
-          clo = m.y;
-          chi = m.y + m.z;
-          cn = (m.z + CR - 1) / CR;
+          clo = uni(m.y);
+          chi = clo + uni(m.z);
+          cn = (uni(m.z) + CR - 1) / CR;
           cc = 0;
         }
       };
-      uint32_t idx_a[kDepth][kRPT], idx_b[kDepth][kRPT];
+      uint32_t idx[kDepth][kRPT];
       V val[kDepth][kRPT];
 #pragma unroll
-      for (int k = 0; k < kDepth; k++) next_chunk(idx_a[k]);
-#pragma unroll
-      for (int k = 0; k < kDepth; k++) next_chunk(idx_b[k]);
+      for (int k = 0; k < kDepth; k++) next_chunk(idx[k]);
 #pragma unroll
       for (int k = 0; k < kDepth; k++)
 #pragma unroll
-        for (int q = 0; q < kRPT; q++) val[k][q] = row_load(idx_a[k][q]);
-      // invariant at the top of a round: val[k] holds chunk g0+k, idx_b[k] the row indices of chunk g0+kDepth+k
+        for (int q = 0; q < kRPT; q++) val[k][q] = row_load(idx[k][q]);
+#pragma unroll
+      for (int k = 0; k < kDepth; k++) next_chunk(idx[k]);
+      // invariant at step k of a round: val[k] holds chunk g0+k, idx[k] the row indices of chunk g0+k+kDepth
       uint32_t slot = 0;
       for (uint32_t g0 = 0; g0 < G; g0 += kDepth) {
-#pragma unroll
-        for (int k = 0; k < kDepth; k++)
-#pragma unroll
-          for (int q = 0; q < kRPT; q++) idx_a[k][q] = idx_b[k][q];
-#pragma unroll
-        for (int k = 0; k < kDepth; k++) next_chunk(idx_b[k]);
 #pragma unroll
         for (int k = 0; k < kDepth; k++) {
           if (g0 + k < G) { // uniform over the block: the summing wave makes the same number of barriers
@@ -483,10 +491,14 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
             slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
 #pragma unroll
             for (int q = 0; q < kRPT; q++) {
-              if (in_slice) *(V *)(sp + (q * RPL + my_row) * CS + lcol) = val[k][q];
-              val[k][q] = row_load(idx_a[k][q]); // chunk g0 + k + kDepth
+              if (in_slice) {
+                if (CSC) store_transposed(sp + my_lane * pitch + (q * RPL + my_row), (CSC / 4) * pitch, val[k][q]);
+                else *(V *)(sp + (q * RPL + my_row) * CS + lcol) = val[k][q];
+              }
+              val[k][q] = row_load(idx[k][q]); // chunk g0 + k + kDepth
             }
-            __syncthreads(); // barrier g0 + k
+            next_chunk(idx[k]); // chunk g0 + k + 2 * kDepth
+            __syncthreads();    // barrier g0 + k
           }
         }
       }
@@ -495,7 +507,8 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
 #if HCTR_SUM_PRIO
       __builtin_amdgcn_s_setprio(HCTR_SUM_PRIO); // the chain of this wave is the critical path of the whole push
 #endif
-      const uint32_t mycol = slice * CS + threadIdx.x;
+      // the column this lane sums: lane = place in the fast path's layout
+      const uint32_t mycol = slice * CS + (CSC ? (threadIdx.x % (CSC ? CSC / 4 : 1)) * 4 + threadIdx.x / (CSC ? CSC / 4 : 1) : threadIdx.x);
       const bool col_ok = threadIdx.x < CS && mycol < W;
       const bool direct = t.nrank == 1; // every key is owned and resident; the version counters move elsewhere
       uint32_t slot = 0;
@@ -508,23 +521,48 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
         float acc = 0.f; // the reference starts every sum from 0
         uint32_t c = 0;
         if (CSC) {
-          for (; c < nfull; c++) {
-            __syncthreads(); // barrier of this chunk
-            const float *sp = lds + slot * slot_floats + (threadIdx.x < CS ? threadIdx.x : 0);
-            slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
+          // Full chunks, kSumBatch rows at a time, one batch ahead: the LDS reads of a batch are in flight while the
+          // previous batch is added.  Reading the first batch of a chunk passes that chunk's barrier, i.e. the wave
+          // is at most one barrier ahead of its adds, which the three ring slots allow.
+          constexpr int kBatches = kChunkRows / kSumBatch; // per chunk
+          const uint32_t total = nfull * kBatches;
+          const uint32_t lane_off = (threadIdx.x < CS ? threadIdx.x : 0) * pitch;
+          const float *sp = lds;
+          auto read_batch = [&](uint32_t b, float(&dst)[kSumBatch]) {
+            if (b % kBatches == 0) {
+              __syncthreads(); // barrier of this chunk
+              sp = lds + slot * slot_floats + lane_off;
+              slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
+            }
+            const float4 *bp = (const float4 *)(sp + (b % kBatches) * kSumBatch);
 #pragma unroll
-            for (int r0 = 0; r0 < kChunkRows; r0 += kSumBatch) {
-              float x[kSumBatch];
+            for (int q = 0; q < kSumBatch / 4; q++) {
+              const float4 v = bp[q];
+              dst[4 * q] = v.x, dst[4 * q + 1] = v.y, dst[4 * q + 2] = v.z, dst[4 * q + 3] = v.w;
+            }
+          };
+          if (total) {
+            float x0[kSumBatch], x1[kSumBatch];
+            read_batch(0, x0);
+            for (uint32_t b = 0;; b += 2) {
+              const bool more1 = b + 1 < total;
+              if (more1) read_batch(b + 1, x1);
 #pragma unroll
-              for (int q = 0; q < kSumBatch; q++) x[q] = sp[(r0 + q) * (CSC ? CSC : 1)];
+              for (int q = 0; q < kSumBatch; q++) acc += x0[q];
+              if (!more1) break;
+              const bool more2 = b + 2 < total;
+              if (more2) read_batch(b + 2, x0);
 #pragma unroll
-              for (int q = 0; q < kSumBatch; q++) acc += x[q];
+              for (int q = 0; q < kSumBatch; q++) acc += x1[q];
+              if (!more2) break;
             }
           }
+          c = nfull;
         }
         for (; c < nch; c++) { // generic path, and the partial last chunk of the fast path
           __syncthreads();     // barrier of this chunk
-          const float *col_ptr = lds + slot * slot_floats + threadIdx.x;
+          const uint32_t rstride = CSC ? 1u : CS; // distance between two rows of this lane's column
+          const float *col_ptr = lds + slot * slot_floats + threadIdx.x * (CSC ? pitch : 1u);
           slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
           if (threadIdx.x < CS) {
             const uint32_t rows = min(CR, L - c * CR);
@@ -532,11 +570,11 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
             for (; r + 8 <= rows; r += 8) {
               float x[8];
 #pragma unroll
-              for (int q = 0; q < 8; q++) x[q] = col_ptr[(r + q) * CS];
+              for (int q = 0; q < 8; q++) x[q] = col_ptr[(r + q) * rstride];
 #pragma unroll
               for (int q = 0; q < 8; q++) acc += x[q];
             }
-            for (; r < rows; r++) acc += col_ptr[r * CS];
+            for (; r < rows; r++) acc += col_ptr[r * rstride];
           }
         }
         if (col_ok) {
@@ -566,17 +604,15 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
   __shared__ uint32_t run_totals[3];
   if (blockIdx.x < kLongBlocks) {
     if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 1) return;
-    // the longest runs are cut into narrower column slices, worked on by more blocks: the blocks of a saturated
-    // memory system get equal shares of it, and a chain advances with the share of the block that feeds it
+    // Every block first takes tickets of the longest runs, which are cut into narrower column slices so that more
+    // blocks feed each of them (the blocks of a saturated memory system get equal shares of it, and a chain
+    // advances with the share of the block that feeds it), then tickets of the other long runs.
     uint32_t *tk = p.d_nlong + kTicketBase;
     if (VEC == 4 && t.width % kSlice == 0) {
-      if (blockIdx.x < kGiantBlocks)
-        long_role<VEC, K, (VEC == 4 ? kGiantSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, 0, kGiantClasses,
-                                                        blockIdx.x, kGiantBlocks, tk);
-      else
-        long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, kGiantClasses,
-                                                   kLongBuckets, blockIdx.x - kGiantBlocks, kLongBlocks - kGiantBlocks,
-                                                   tk + kTicketLanes);
+      long_role<VEC, K, (VEC == 4 ? kGiantSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, 0, kGiantClasses,
+                                                      blockIdx.x, kLongBlocks, tk);
+      long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, kGiantClasses, kLongBuckets,
+                                                 blockIdx.x, kLongBlocks, tk + kTicketLanes);
     } else {
       long_role<VEC, K, 0>(t, id_bits, p, a, lds, run_table, run_totals, 0, kLongBuckets, blockIdx.x, kLongBlocks, tk);
     }
