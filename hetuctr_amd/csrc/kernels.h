@@ -32,10 +32,10 @@ struct BatchView {
   uint32_t *med_list;        // [d_nlong[kMedCount]] unique ranks with kTinyRun < run length <= kLongRun (any order)
 };
 
-// d_nlong layout: [0, kLongBuckets) long runs per class, then the number of medium runs, the medium work counter
-// and the ticket counters of the long role
+// d_nlong layout: [0, kLongBuckets) long runs per class, then the number of medium runs and the ticket counters of
+// the long role
 constexpr int kLongBuckets = 12;
-constexpr int kMedCount = kLongBuckets, kMedWork = kLongBuckets + 1, kTicketBase = kLongBuckets + 2, kTicketLanes = 16,
+constexpr int kMedCount = kLongBuckets, kTicketBase = kLongBuckets + 1, kTicketLanes = 16,
               kRunCounters = kTicketBase + 2 * kTicketLanes;
 
 // A run of equal keys longer than this is summed by a whole block that streams its gradient rows through

@@ -37,9 +37,6 @@ namespace hctr {
 #ifndef HCTR_SUM_PRIO
 #define HCTR_SUM_PRIO 0
 #endif
-#ifndef HCTR_ABL
-#define HCTR_ABL 0 // ablation bits for timing experiments only: 1 no version update, 2 no row read, 4 no row store, 8 no gradient loads
-#endif
 #ifndef HCTR_SLICE
 #define HCTR_SLICE 64
 #endif
@@ -199,7 +196,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
       for (int i = 0; i < G; i++) {
         e[i] = Vec<VEC>::zero();
-        if (mine[i] && !(HCTR_ABL & 2)) e[i] = *(const V *)(t.emb + (size_t)off[i] * W + col);
+        if (mine[i]) e[i] = *(const V *)(t.emb + (size_t)off[i] * W + col);
       }
     }
 #pragma unroll
@@ -211,7 +208,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
       for (int k = 0; k < kHead; k++) {
         v[i][k] = Vec<VEC>::zero();
-        if (mine[i] && (uint32_t)k < len[i] && !(HCTR_ABL & 8)) v[i][k] = *(const V *)(grad + (size_t)si[i][k] * W + col);
+        if (mine[i] && (uint32_t)k < len[i]) v[i][k] = *(const V *)(grad + (size_t)si[i][k] * W + col);
       }
     V acc[G];
 #pragma unroll
@@ -241,7 +238,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
       if (kSingle) {
         V r = e[i];
         Vec<VEC>::add(r, scaled);
-        if (!(HCTR_ABL & 4)) *(V *)(t.emb + (size_t)off[i] * W + col) = r; // versions: bump_versions
+        *(V *)(t.emb + (size_t)off[i] * W + col) = r; // the version counters move in the last blocks of the launch
       } else {
         apply_row<VEC, K>(t, id_bits, p, a, u0 + i, scaled, col, c0 == 0 && gl == 0);
       }

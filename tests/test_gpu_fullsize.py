@@ -1,4 +1,4 @@
-"""The BASELINE.json configurations at their full sizes on the GPU.
+"""The benchmark configurations (hetuctr_amd.workloads.CONFIGS) at their full sizes on the GPU.
 
 cfg2 (headline) runs next to the CPU oracle and must agree bit for bit.  The larger ones are checked through
 properties that do not need an oracle of that size: the integer outputs against numpy's own unique / lexsort on
