@@ -97,6 +97,49 @@ def test_skewed_keys_long_runs(alpha, width):
     p.close()
 
 
+@pytest.mark.parametrize("width", [48, 192, 256, 512, 1024])
+def test_long_runs_slice_layouts(width):
+    # long runs with row widths that are cut into 1..32 column slices, or (48) take the path without slices
+    say("long runs, width", width)
+    rng = np.random.default_rng(width)
+    length, n = 50_000, 40_000
+    draw = zipf_sampler(length, 1.2, rng)
+    p = single(length, width, lr=0.05)
+    prev_n = 0
+    for step in range(3):
+        keys = draw(n)
+        p.preprocess([keys], device_keys=True)
+        g = rng.normal(0, 1e-3, size=(prev_n, width)).astype(np.float32)
+        out, ref = p.push_pull([g])
+        assert_close(out[0], ref[0], 1e-5, "dst step %d" % step)
+        p.compare_ints(INT_ITEMS_POST, "step %d" % step)
+        p.compare_state(1e-5, "step %d" % step)
+        prev_n = n
+    p.close()
+
+
+@pytest.mark.parametrize("width", [64, 128])
+def test_one_chain_longer_than_every_length_class(width):
+    # 140,000 occurrences of one key (more than 2^17) among skewed others, random gradients: the sum must come out in
+    # the reference's serial order
+    say("giant chain, width", width)
+    rng = np.random.default_rng(5)
+    length = 30_000
+    draw = zipf_sampler(length, 1.1, rng)
+    p = single(length, width, lr=0.05)
+    prev_n = 0
+    for step in range(2):
+        keys = np.concatenate([np.full(140_000, 7, np.int64), draw(30_000)])
+        rng.shuffle(keys)
+        p.preprocess([keys], device_keys=True)
+        g = rng.normal(0, 1e-3, size=(prev_n, width)).astype(np.float32)
+        out, ref = p.push_pull([g])
+        assert_close(out[0], ref[0], 1e-5, "dst step %d" % step)
+        p.compare_state(1e-5, "step %d" % step)
+        prev_n = keys.shape[0]
+    p.close()
+
+
 def test_one_key_repeated_and_all_distinct():
     say("extremes")
     length, width = 70_000, 32
