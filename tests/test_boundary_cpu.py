@@ -93,3 +93,22 @@ def test_product_never_touches_the_oracle():
         if os.path.isfile(path) and path.endswith((".py", ".hip", ".h", ".cpp")):
             text = open(path).read().lower()
             assert "oracle" not in text and "liborc" not in text, path
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # the build runs on one GPU; asking for more must end with a message and a non-zero status, before any GPU work
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2", "--steps", "1"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_workload_byte_accounting():
+    # algorithmic bytes per step: 4W(2N + 3U) + 41N + 81U, split into the stages bench.py reports
+    from hetuctr_amd import workloads
+    n, u, w = 1_703_936, 314_800, 128
+    total = workloads.algorithmic_bytes(n, u, w)
+    assert total == 4 * w * (2 * n + 3 * u) + 41 * n + 81 * u
+    assert workloads.stage_bytes("segment_sum_apply", n, u, n, u, w) == 4 * w * n + 8 * w * u + 8 * n + 32 * u
+    assert workloads.stage_bytes("gather", n, u, n, u, w) == 4 * w * n + 4 * w * u + 8 * n + 8 * u
