@@ -480,25 +480,30 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       for (int k = 0; k < kDepth; k++) next_chunk(idx[k]);
       // invariant at step k of a round: val[k] holds chunk g0+k, idx[k] the row indices of chunk g0+k+kDepth
       uint32_t slot = 0;
-      for (uint32_t g0 = 0; g0 < G; g0 += kDepth) {
+      auto step = [&](int k) {
+        float *sp = lds + slot * slot_floats;
+        slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
 #pragma unroll
-        for (int k = 0; k < kDepth; k++) {
-          if (g0 + k < G) { // uniform over the block: the summing wave makes the same number of barriers
-            float *sp = lds + slot * slot_floats;
-            slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
-#pragma unroll
-            for (int q = 0; q < kRPT; q++) {
-              if (in_slice) {
-                if (CSC) store_transposed(sp + my_lane * pitch + (q * RPL + my_row), (CSC / 4) * pitch, val[k][q]);
-                else *(V *)(sp + (q * RPL + my_row) * CS + lcol) = val[k][q];
-              }
-              val[k][q] = row_load(idx[k][q]); // chunk g0 + k + kDepth
-            }
-            next_chunk(idx[k]); // chunk g0 + k + 2 * kDepth
-            __syncthreads();    // barrier g0 + k
+        for (int q = 0; q < kRPT; q++) {
+          if (in_slice) {
+            if (CSC) store_transposed(sp + my_lane * pitch + (q * RPL + my_row), (CSC / 4) * pitch, val[k][q]);
+            else *(V *)(sp + (q * RPL + my_row) * CS + lcol) = val[k][q];
           }
+          val[k][q] = row_load(idx[k][q]); // chunk + kDepth
         }
+        next_chunk(idx[k]); // chunk + 2 * kDepth
+        __syncthreads();    // barrier of this chunk
+      };
+      // Whole rounds run without a condition inside: with one, the compiler must assume that loads may have been
+      // skipped and waits for nearly everything in flight before each use.
+      uint32_t g0 = 0;
+      for (; g0 + kDepth <= G; g0 += kDepth) {
+#pragma unroll
+        for (int k = 0; k < kDepth; k++) step(k);
       }
+#pragma unroll
+      for (int k = 0; k < kDepth; k++)
+        if (g0 + k < G) step(k); // uniform over the block: the summing wave makes the same number of barriers
     } else {
       // ---------------- summing wave: one column per lane, rows strictly in order ----------------
 #if HCTR_SUM_PRIO
