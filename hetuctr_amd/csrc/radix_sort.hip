@@ -177,7 +177,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
 template <typename K>
 void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
                           uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
-                          const K **keys_sorted) {
+                          const K **keys_sorted, bool first_hist_done) {
   *keys_sorted = keys_in;
   if (n == 0) return;
   if (bits < 1) bits = 1;
@@ -196,8 +196,9 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
     K *kout = ktmp[p & 1];
     uint32_t *vout = (p == passes - 1) ? vals_out : vtmp[p & 1];
     const uint32_t nb = 1u << dbits;
-    hipLaunchKernelGGL(digit_histogram<K>, dim3(nblocks), dim3(kSortBlock), 0, stream, kin, n, shift, dbits,
-                       scratch.ghist, nblocks);
+    if (p > 0 || !first_hist_done)
+      hipLaunchKernelGGL(digit_histogram<K>, dim3(nblocks), dim3(kSortBlock), 0, stream, kin, n, shift, dbits,
+                         scratch.ghist, nblocks);
     hipLaunchKernelGGL(scan_bins, dim3(nb), dim3(kSortBlock), 0, stream, scratch.ghist, nblocks, scratch.bintot);
     if (p == 0)
       hipLaunchKernelGGL((scatter<K, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
@@ -215,9 +216,9 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
 
 template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *, uint32_t *,
                                              uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
-                                             const uint32_t **);
+                                             const uint32_t **, bool);
 template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *, uint64_t *,
                                              uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
-                                             const uint64_t **);
+                                             const uint64_t **, bool);
 
 } // namespace hctr

@@ -217,7 +217,7 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
         HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
       }
       launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, comp.p, err_ptr(),
-                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>());
+                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), ghist.as<uint32_t>());
     }
     SortScratch sc;
     sc.ghist = ghist.as<uint32_t>();
@@ -229,13 +229,13 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
       const uint64_t *sk;
       radix_sort_positions<uint64_t>(s, comp.as<uint64_t>(), cur.n, kl.total_bits, ktmp0.as<uint64_t>(),
                                      ktmp1.as<uint64_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
-                                     cur.sorted_arg.as<uint32_t>(), sc, &sk);
+                                     cur.sorted_arg.as<uint32_t>(), sc, &sk, true);
       sorted_keys = sk;
     } else {
       const uint32_t *sk;
       radix_sort_positions<uint32_t>(s, comp.as<uint32_t>(), cur.n, kl.total_bits, ktmp0.as<uint32_t>(),
                                      ktmp1.as<uint32_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
-                                     cur.sorted_arg.as<uint32_t>(), sc, &sk);
+                                     cur.sorted_arg.as<uint32_t>(), sc, &sk, true);
       sorted_keys = sk;
     }
     delete sort_scope;
