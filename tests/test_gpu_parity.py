@@ -36,6 +36,22 @@ def test_init_values(kind, a, b, tol):
         p.close()
 
 
+def test_uniform_init_golden_vectors():
+    # the HIP initialiser against the committed known answers (tests/golden/minstd_uniform.json)
+    import json
+    import os
+    say("init golden")
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "minstd_uniform.json")
+    length, width = 4400, 16                      # 70,400 values: every offset below 70,000 is covered
+    for c in json.load(open(path))["cases"]:
+        p = single(length, width, init=("Uniform", c["a"], c["b"]), seed=c["seed"])
+        got = p.tables[0].fetch(capi.EMBEDDING).reshape(-1).view(np.uint32)
+        for n, bits in zip(c["offsets"], c["f32_bits"]):
+            if n < got.shape[0]:
+                assert int(got[n]) == bits, (c["seed"], c["a"], c["b"], n)
+        p.close()
+
+
 @pytest.mark.parametrize("width", [1, 3, 4, 16, 20, 64, 128, 200, 256, 300, 512])
 def test_single_shard_steps_all_widths(width):
     say("single shard width", width)

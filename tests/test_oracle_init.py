@@ -101,3 +101,21 @@ def test_normal_moments_and_determinism():
     n = orc.init_values(200000, "Normal", 0.0, 1.0, 9)
     inside = np.abs(n) <= 2.0
     assert np.array_equal(t[inside], n[inside])
+
+
+def test_uniform_golden_vectors():
+    # known answers committed under tests/golden (made by tests/golden/make_vectors.py from the engine's definition)
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "minstd_uniform.json")
+    cases = json.load(open(path))["cases"]
+    for c in cases:
+        small = [(n, b) for n, b in zip(c["offsets"], c["f32_bits"]) if n < 70000]
+        got = orc.init_values(70000, "Uniform", c["a"], c["b"], c["seed"]).view(np.uint32)
+        for n, bits in small:
+            assert int(got[n]) == bits, (c["seed"], c["a"], c["b"], n)
+    c = cases[0]
+    n_far = c["offsets"][-1]
+    far = orc.init_values(n_far + 1, "Uniform", c["a"], c["b"], c["seed"]).view(np.uint32)
+    for n, bits in zip(c["offsets"], c["f32_bits"]):
+        assert int(far[n]) == bits
