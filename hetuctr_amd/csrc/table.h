@@ -37,12 +37,13 @@ struct DeviceBuf {
     p = nullptr;
     bytes = 0;
   }
-  void reserve(size_t want) {
-    if (want <= bytes) return;
+  bool reserve(size_t want) { // true: a new allocation was made
+    if (want <= bytes) return false;
     release();
     size_t grow = want + want / 8; // headroom so that slowly growing batches do not reallocate every step
     HCTR_HIP(hipMalloc(&p, grow));
     bytes = grow;
+    return true;
   }
   template <typename T> T *as() const { return (T *)p; }
 };
@@ -52,10 +53,12 @@ struct Batch {
   uint32_t n = 0;   // keys
   uint32_t U = 0;   // unique keys (host copy, valid after the preprocess call returned)
   bool idx_map_valid = false;
+  bool cleared = false; // the device side reads as an empty batch (U = 0, no buckets, no runs) since clear()
   DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong, med_list;
   std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
   std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
   void reserve(uint32_t n_keys, int nrank, bool wide);
+  void clear(hipStream_t s, int nrank); // make the device side an empty batch; does nothing if it already is
   BatchView view() const;
 };
 
@@ -130,6 +133,8 @@ class Shard {
   HostMirror *mirror = nullptr;
   long long last_stats[6] = {0, 0, 0, 0, 0, 0};
   float last_pre_ms = 0.f, last_pp_ms = 0.f;
+  bool plan_cleared = false; // the device-side push counts read as zero
+  bool u_cleared = false;    // the device-side copy of the number of unique keys reads as zero
 
  private:
   void reserve_batch_scratch(uint32_t n);

@@ -34,13 +34,23 @@ void Batch::reserve(uint32_t n_keys, int nrank, bool wide) {
   rank_sorted.reserve(n * 4);
   idx_map.reserve(n * 4);
   ukey.reserve(n * (wide ? 8 : 4));
-  run_start.reserve((n + 1) * 4);
+  bool fresh = run_start.reserve((n + 1) * 4);
   uoff.reserve(n * sizeof(slot_t));
-  bucket_lo.reserve((size_t)(nrank + 1) * 4);
-  dU.reserve(4);
+  fresh |= bucket_lo.reserve((size_t)(nrank + 1) * 4);
+  fresh |= dU.reserve(4);
   long_list.reserve(long_list_capacity((uint32_t)n) * sizeof(uint4) * kLongBuckets);
-  dnlong.reserve(4 * kRunCounters);
+  fresh |= dnlong.reserve(4 * kRunCounters);
   med_list.reserve(med_list_capacity((uint32_t)n) * 4);
+  if (fresh) cleared = false;
+}
+
+void Batch::clear(hipStream_t s, int nrank) {
+  if (cleared) return;
+  HCTR_HIP(hipMemsetAsync(dU.p, 0, 4, s));
+  HCTR_HIP(hipMemsetAsync(bucket_lo.p, 0, (size_t)(nrank + 1) * 4, s));
+  HCTR_HIP(hipMemsetAsync(run_start.p, 0, 4, s));
+  HCTR_HIP(hipMemsetAsync(dnlong.p, 0, 4 * kRunCounters, s));
+  cleared = true;
 }
 
 BatchView Batch::view() const {
@@ -138,10 +148,7 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
   for (Batch *b : {&cur, &prev}) {
     b->reserve(1, c.nrank, kl.wide);
-    HCTR_HIP(hipMemsetAsync(b->dU.p, 0, 4, s));
-    HCTR_HIP(hipMemsetAsync(b->dnlong.p, 0, 4 * kRunCounters, s));
-    HCTR_HIP(hipMemsetAsync(b->bucket_lo.p, 0, b->bucket_lo.bytes, s));
-    HCTR_HIP(hipMemsetAsync(b->run_start.p, 0, 4, s));
+    b->clear(s, c.nrank);
     b->send_cnt.assign(c.nrank + 1, 0);
     b->recv_cnt.assign(c.nrank + 1, 0);
     b->push_cnt.assign(c.nrank + 1, 0);
@@ -199,11 +206,10 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
   cur.idx_map_valid = false;
   cur.reserve(cur.n, cfg.nrank, kl.wide);
   if (n == 0) { // :93-95
-    HCTR_HIP(hipMemsetAsync(cur.dU.p, 0, 4, s));
-    HCTR_HIP(hipMemsetAsync(cur.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
-    HCTR_HIP(hipMemsetAsync(cur.run_start.p, 0, 4, s));
-    HCTR_HIP(hipMemsetAsync(cur.dnlong.p, 0, 4 * kRunCounters, s));
+    cur.clear(s, cfg.nrank);
   } else {
+    cur.cleared = false;
+    u_cleared = false;
     reserve_batch_scratch(cur.n);
     {
       // ids -> device copy (:98-99) and sort keys.  When the caller's pointer is device-visible the copy is
@@ -252,10 +258,14 @@ void Shard::preprocess_gradient() {
   uint64_t *cnt = dst_->push_cnt;
   if (cfg.nrank == 1) return; // single shard: every key is owned, nothing is ever pushed
   if (prev.n == 0) {
-    HCTR_HIP(hipMemsetAsync(cnt, 0, (size_t)(cfg.nrank + 1) * sizeof(uint64_t), s));
-    HCTR_HIP(hipMemsetAsync(&dst_->push_total, 0, 4, s));
+    if (!plan_cleared) {
+      HCTR_HIP(hipMemsetAsync(cnt, 0, (size_t)(cfg.nrank + 1) * sizeof(uint64_t), s));
+      HCTR_HIP(hipMemsetAsync(&dst_->push_total, 0, 4, s));
+      plan_cleared = true;
+    }
     return;
   }
+  plan_cleared = false;
   need.reserve((size_t)prev.n * 4);
   prefix.reserve((size_t)prev.n * 4);
   reserve_batch_scratch(prev.n);
@@ -268,7 +278,10 @@ void Shard::preprocess_gradient() {
 
 void Shard::enqueue_readback_preprocess() {
   hipStream_t s = group->stream;
-  if (cur.n == 0) HCTR_HIP(hipMemsetAsync(&dst_->U, 0, 4, s));
+  if (cur.n == 0 && !u_cleared) {
+    HCTR_HIP(hipMemsetAsync(&dst_->U, 0, 4, s));
+    u_cleared = true;
+  }
   const size_t bytes = cfg.nrank == 1 ? 16 : sizeof(DevStat);
   HCTR_HIP(hipMemcpyAsync(&mirror->st, dstat.p, bytes, hipMemcpyDeviceToHost, s));
 }
@@ -298,9 +311,7 @@ void Shard::generate_gradient(const float *grad) {
   if (grad == nullptr) {
     prev.n = 0;
     prev.U = 0;
-    HCTR_HIP(hipMemsetAsync(prev.dU.p, 0, 4, s));
-    HCTR_HIP(hipMemsetAsync(prev.dnlong.p, 0, 4 * kRunCounters, s));
-    HCTR_HIP(hipMemsetAsync(prev.bucket_lo.p, 0, (size_t)(cfg.nrank + 1) * 4, s));
+    prev.clear(s, cfg.nrank);
     std::fill(prev.push_cnt.begin(), prev.push_cnt.end(), 0);
     std::fill(prev.pushrecv_cnt.begin(), prev.pushrecv_cnt.end(), 0);
   }
@@ -353,11 +364,17 @@ void Shard::handle_gradient() {
                         (uint32_t)rg_seg[src], (uint32_t)rg_seg[src + 1], err_ptr());
 }
 
-__global__ void segment_bounds(const uint32_t *__restrict__ out_pos, const uint32_t *__restrict__ total,
-                               const uint32_t *__restrict__ seg, int nseg, uint32_t q, uint32_t *__restrict__ out) {
+// rows to return per requester: where the segments of the query start in the compacted order of the rows that are
+// sent back; the last word carries the shard's error flags so that one transfer brings both to the host
+struct SegmentStarts {
+  uint32_t v[258];
+};
+__global__ void segment_bounds(const uint32_t *__restrict__ out_pos, const uint32_t *__restrict__ total, SegmentStarts seg,
+                               int nseg, uint32_t q, const uint32_t *__restrict__ err, uint32_t *__restrict__ out) {
   const int i = threadIdx.x;
+  if (i == 0) out[257] = *err;
   if (i > nseg) return;
-  const uint32_t k = seg[i];
+  const uint32_t k = seg.v[i];
   out[i] = k >= q ? *total : out_pos[k];
 }
 
@@ -378,23 +395,20 @@ void Shard::handle_query() {
                         ret_total.as<uint32_t>());
   launch_pack_rows(s, tv, rq_idx.as<index_t>(), outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q,
                    ret_ver.as<version_t>(), ret_val.as<embed_t>());
-  // rows to return per requester: positions of the segment starts in the compacted order
-  uint32_t *seg_h = mirror->ret_seg; // staged through the pinned mirror, overwritten by the result below
-  for (int i = 0; i <= R; i++) seg_h[i] = (uint32_t)rq_seg[i];
-  uint32_t *seg_d = ret_seg_dev.as<uint32_t>();
-  HCTR_HIP(hipMemcpyAsync(seg_d, seg_h, (size_t)(R + 1) * 4, hipMemcpyHostToDevice, s));
-  hipLaunchKernelGGL(segment_bounds, dim3(1), dim3(R + 1), 0, s, out_pos.as<uint32_t>(), ret_total.as<uint32_t>(),
-                     seg_d, R, Q, seg_d + 258);
+  SegmentStarts seg;
+  for (int i = 0; i <= R; i++) seg.v[i] = (uint32_t)rq_seg[i];
+  uint32_t *out = ret_seg_dev.as<uint32_t>();
+  hipLaunchKernelGGL(segment_bounds, dim3(1), dim3(R + 1), 0, s, out_pos.as<uint32_t>(), ret_total.as<uint32_t>(), seg, R, Q,
+                     err_ptr(), out);
   HCTR_HIP(hipGetLastError());
-  HCTR_HIP(hipMemcpyAsync(seg_h, seg_d + 258, (size_t)(R + 1) * 4, hipMemcpyDeviceToHost, s));
-  HCTR_HIP(hipMemcpyAsync(&mirror->st.err, err_ptr(), 4, hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipMemcpyAsync(mirror->ret_seg, out, 258 * 4, hipMemcpyDeviceToHost, s));
 }
 
 void Shard::finish_handle_query() {
   for (int i = 0; i <= cfg.nrank; i++) ret_seg[i] = mirror->ret_seg[i];
   last_stats[4] = (long long)ret_seg[cfg.nrank];
-  if (mirror->st.err) {
-    const uint32_t e = mirror->st.err;
+  if (mirror->ret_seg[257]) {
+    const uint32_t e = mirror->ret_seg[257];
     HCTR_HIP(hipMemsetAsync(err_ptr(), 0, 4, group->stream));
     HCTR_CHECK(!(e & 2u), "a pushed row reached a shard that does not own it");
     HCTR_CHECK(!(e & 4u), "a queried row reached a shard that does not own it");
