@@ -29,7 +29,8 @@ def parse():
     ap.add_argument("--batches", type=int, default=4, help="distinct key batches cycled through")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and samples (debugging only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-steps", type=int, default=3)
+    ap.add_argument("--cpu-steps", type=int, default=10,
+                    help="full-size steps of the CPU baseline leg (about 12 core-seconds at the default)")
     ap.add_argument("--no-stage-timing", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the library's plain 1 GiB copy kernel (scale factor of the HBM byte counters)")
