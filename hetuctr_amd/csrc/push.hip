@@ -157,6 +157,7 @@ __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const
 #endif
 constexpr int kRunsPerGroup = HCTR_RUNS_PER_GROUP;
 constexpr int kHead = 2; // occurrences per run fetched up front
+constexpr int kTail = 6; // occurrences per step after those
 
 template <int VEC, int LPR, typename K, bool kSingle>
 __device__ __forceinline__ void short_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
@@ -221,11 +222,10 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
     for (int i = 0; i < G; i++) {
       if (!mine[i]) continue;
-      if (len[i] > kHead) { // the rest of the run (at most kTinyRun - kHead rows), in order
-        constexpr int kTail = kTinyRun - kHead;
+      // the rest of the run (at most kTinyRun - kHead rows), in order, kTail rows at a time
+      for (uint32_t j = rs[i] + kHead; j < rs[i + 1]; j += kTail) {
         uint32_t sj[kTail];
         V x[kTail];
-        const uint32_t j = rs[i] + kHead;
 #pragma unroll
         for (int k = 0; k < kTail; k++) sj[k] = sorted_arg[min(j + k, rs[i + 1] - 1)];
 #pragma unroll
