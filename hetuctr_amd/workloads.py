@@ -15,6 +15,9 @@ CONFIGS = {
     # headline: ~33M rows in 26 log-uniform fields (10 .. 10M), dim 128
     "cfg2": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=1.05, lr=0.05,
                  init=("Normal", 0.0, 0.1), single_field=False),
+    # the same table and batch with uniform ids: nearly every key of a batch is distinct (no duplicates to sum)
+    "cfg2_uniform": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=None, lr=0.05,
+                         init=("Normal", 0.0, 0.1), single_field=True),
     # one GPU's shard of an 8-way partition of the cfg2 table: rank 0 owns 1/8 of the rows and caches the hottest
     # 10 % of the others; the peers live on the same GPU behind the loopback and only serve rank 0
     "cfg3": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=1.05, lr=0.05,

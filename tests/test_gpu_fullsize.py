@@ -74,7 +74,7 @@ def test_cfg2_headline_bit_exact_against_oracle():
     t.close(); o.close()
 
 
-@pytest.mark.parametrize("name", ["cfg4", "cfg5_zipf", "cfg5_uniform"])
+@pytest.mark.parametrize("name", ["cfg2_uniform", "cfg4", "cfg5_zipf", "cfg5_uniform"])
 def test_large_configs_by_properties(name):
     cfg = workloads.CONFIGS[name]
     ks = workloads.KeyStream(cfg, seed=0)
