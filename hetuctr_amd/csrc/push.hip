@@ -526,37 +526,52 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
           // Full chunks, kSumBatch rows at a time, one batch ahead: the LDS reads of a batch are in flight while the
           // previous batch is added.  Reading the first batch of a chunk passes that chunk's barrier, i.e. the wave
           // is at most one barrier ahead of its adds, which the three ring slots allow.
-          constexpr int kBatches = kChunkRows / kSumBatch; // per chunk
-          const uint32_t total = nfull * kBatches;
+          constexpr int kBatches = kChunkRows / kSumBatch; // per chunk, even
+          static_assert(!CSC || kBatches % 2 == 0, "the two batch buffers alternate, a chunk starts on the first");
           const uint32_t lane_off = (threadIdx.x < CS ? threadIdx.x : 0) * pitch;
           const float *sp = lds;
-          auto read_batch = [&](uint32_t b, float(&dst)[kSumBatch]) {
-            if (b % kBatches == 0) {
-              __syncthreads(); // barrier of this chunk
-              sp = lds + slot * slot_floats + lane_off;
-              slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
-            }
-            const float4 *bp = (const float4 *)(sp + (b % kBatches) * kSumBatch);
+          auto open_chunk = [&]() { // passes the chunk's barrier
+            __syncthreads();
+            sp = lds + slot * slot_floats + lane_off;
+            slot = slot + 1 == (uint32_t)kSlots ? 0 : slot + 1;
+          };
+          auto read_batch = [&](int k, float(&dst)[kSumBatch]) { // batch k of the open chunk
+            const float4 *bp = (const float4 *)(sp + k * kSumBatch);
 #pragma unroll
             for (int q = 0; q < kSumBatch / 4; q++) {
               const float4 v = bp[q];
               dst[4 * q] = v.x, dst[4 * q + 1] = v.y, dst[4 * q + 2] = v.z, dst[4 * q + 3] = v.w;
             }
           };
-          if (total) {
+          auto add_batch = [&](const float(&x)[kSumBatch]) {
+#pragma unroll
+            for (int q = 0; q < kSumBatch; q++) acc += x[q];
+          };
+          if (nfull) {
             float x0[kSumBatch], x1[kSumBatch];
+            open_chunk();
             read_batch(0, x0);
-            for (uint32_t b = 0;; b += 2) {
-              const bool more1 = b + 1 < total;
-              if (more1) read_batch(b + 1, x1);
+            // all chunks but the last: straight-line code, so that the waits for LDS data stay exact
+            for (uint32_t cc2 = 0; cc2 + 1 < nfull; cc2++) {
 #pragma unroll
-              for (int q = 0; q < kSumBatch; q++) acc += x0[q];
-              if (!more1) break;
-              const bool more2 = b + 2 < total;
-              if (more2) read_batch(b + 2, x0);
+              for (int k = 0; k < kBatches; k += 2) {
+                read_batch(k + 1, x1);
+                add_batch(x0);
+                if (k + 2 < kBatches) {
+                  read_batch(k + 2, x0);
+                } else {
+                  open_chunk();
+                  read_batch(0, x0);
+                }
+                add_batch(x1);
+              }
+            }
 #pragma unroll
-              for (int q = 0; q < kSumBatch; q++) acc += x1[q];
-              if (!more2) break;
+            for (int k = 0; k < kBatches; k += 2) { // the last full chunk
+              read_batch(k + 1, x1);
+              add_batch(x0);
+              if (k + 2 < kBatches) read_batch(k + 2, x0);
+              add_batch(x1);
             }
           }
           c = nfull;
