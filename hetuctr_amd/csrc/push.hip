@@ -11,11 +11,11 @@
 //
 // One launch, three ranges of blocks, one per class of run length (the long chains are dispatched first and the
 // other blocks fill the machine behind them):
-//  * long (> kLongRun duplicates): a run is streamed by a whole block.  Seven loader waves keep several
-//    16-byte loads of gradient rows in flight each and stage them through a ring of LDS slots; the first wave
-//    adds the staged rows in order, one column per lane.  The serial chain costs one LDS read and one add per
-//    duplicate while the memory latency is covered by the whole block.  A run is split by column slices of
-//    kSlice floats over several blocks; the longest runs are started first.
+//  * long (> kLongRun duplicates): bundles of runs are streamed by whole blocks, one column slice at a time.  Seven
+//    loader waves keep several 16-byte loads of gradient rows in flight each and stage them through a ring of
+//    LDS slots; the first wave adds the staged rows in order, one column per lane.  The serial chain costs a
+//    quarter of an LDS read and one add per duplicate while the memory latency is covered by the whole block.
+//    The longest runs are started first and cut into narrower slices, i.e. fed by more blocks.
 //  * medium (kTinyRun < duplicates <= kLongRun): one group of LPR lanes per run, kBatch rows in flight.
 //  * short (<= kTinyRun): a group of LPR lanes (LPR*VEC floats = one row) owns a few consecutive unique keys
 //    and sums their runs, all first loads of the group issued together.
@@ -70,8 +70,6 @@ constexpr int kGiantSlice = HCTR_GIANT_SLICE;     // long role: the longest runs
 constexpr int kGiantClasses = HCTR_GIANT_CLASSES; // they are the runs of the first length classes (>= 4096)
 static_assert(kSlice % kGiantSlice == 0, "tiers of the long role");
 constexpr int kMedBlocks = HCTR_MED_BLOCKS;
-
-
 
 namespace {
 
