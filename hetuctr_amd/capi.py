@@ -12,7 +12,9 @@ INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
 SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_push_pull", "hctr_group_preprocess",
            "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch",
            "hctr_stream", "hctr_last_times", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
-           "hctr_stage_times", "hctr_copy_probe", "hctr_version"]
+           "hctr_stage_times", "hctr_copy_probe", "hctr_version", "hctr_part_create", "hctr_part_destroy",
+           "hctr_part_sizes", "hctr_part_refine_data", "hctr_part_refine_embed", "hctr_part_get_communication",
+           "hctr_part_get_priority", "hctr_part_get_result", "hctr_part_get_counts", "hctr_part_cache_lists"]
 
 # items of hctr_debug_fetch (HCTR_F_*)
 UNIQUE, SORTED_ARG, RUN_START, IDX_MAP, ROOT, OFFSET, SEND_CNT, RECV_CNT = range(8)
@@ -57,6 +59,16 @@ def lib():
         l.hctr_stage_name.restype = C.c_char_p
         l.hctr_stage_times.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
         l.hctr_copy_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+        l.hctr_part_create.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_uint,
+                                       C.POINTER(C.c_void_p)]
+        l.hctr_part_sizes.argtypes = [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_int)]
+        for name in ("destroy", "refine_data", "refine_embed"):
+            getattr(l, "hctr_part_" + name).argtypes = [C.c_void_p]
+        l.hctr_part_get_communication.argtypes = [C.c_void_p, C.c_void_p]
+        l.hctr_part_get_priority.argtypes = [C.c_void_p, C.c_void_p]
+        l.hctr_part_get_result.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        l.hctr_part_get_counts.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        l.hctr_part_cache_lists.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
         _lib = l
     return _lib
 

@@ -4,12 +4,17 @@
 #include <cstdio>
 #include <cstring>
 
+#include "partition.h"
 #include "table.h"
 
 using namespace hctr;
 
 struct hctr_table {
   Shard *shard;
+};
+
+struct hctr_partition {
+  Partitioner *p;
 };
 
 namespace {
@@ -199,6 +204,83 @@ int hctr_copy_probe(void *dst, const void *src, size_t bytes, int repeats, float
     if (ms_avg) *ms_avg = ms / repeats;
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
+  });
+}
+
+int hctr_part_create(const int32_t *data, size_t n_data, size_t n_slot, const float *comm_mat, int n_part,
+                     int batch_size, unsigned seed, hctr_partition **out) {
+  return guarded([&] {
+    HCTR_CHECK(out, "null argument");
+    *out = nullptr;
+    *out = new hctr_partition{new Partitioner(data, n_data, n_slot, comm_mat, n_part, batch_size, seed)};
+  });
+}
+
+int hctr_part_destroy(hctr_partition *h) {
+  return guarded([&] {
+    if (!h) return;
+    delete h->p;
+    delete h;
+  });
+}
+
+int hctr_part_sizes(hctr_partition *h, size_t *n_data, size_t *n_embed, int *n_part) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p, "null partition");
+    if (n_data) *n_data = h->p->n_data;
+    if (n_embed) *n_embed = h->p->n_embed;
+    if (n_part) *n_part = h->p->n_part;
+  });
+}
+
+int hctr_part_refine_data(hctr_partition *h) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p, "null partition");
+    h->p->refine_data();
+  });
+}
+
+int hctr_part_refine_embed(hctr_partition *h) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p, "null partition");
+    h->p->refine_embed();
+  });
+}
+
+int hctr_part_get_communication(hctr_partition *h, float *cost) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p && cost, "null argument");
+    h->p->communication(cost);
+  });
+}
+
+int hctr_part_get_priority(hctr_partition *h, float *priority) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p && priority, "null argument");
+    h->p->priority(priority);
+  });
+}
+
+int hctr_part_get_result(hctr_partition *h, int32_t *data_part, int32_t *embed_part) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p, "null partition");
+    if (data_part) memcpy(data_part, h->p->res_data.data(), h->p->n_data * sizeof(int32_t));
+    if (embed_part) memcpy(embed_part, h->p->res_embed.data(), h->p->n_embed * sizeof(int32_t));
+  });
+}
+
+int hctr_part_get_counts(hctr_partition *h, int32_t *data_cnt, int32_t *embed_cnt) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p, "null partition");
+    if (data_cnt) memcpy(data_cnt, h->p->cnt_data.data(), h->p->n_part * sizeof(int32_t));
+    if (embed_cnt) memcpy(embed_cnt, h->p->cnt_embed.data(), h->p->n_part * sizeof(int32_t));
+  });
+}
+
+int hctr_part_cache_lists(hctr_partition *h, size_t max_len, int32_t *lists, size_t *lens, float *kernel_ms) {
+  return guarded([&] {
+    HCTR_CHECK(h && h->p, "null partition");
+    h->p->cache_lists(max_len, lists, lens, kernel_ms);
   });
 }
 

@@ -1,0 +1,373 @@
+// Offline partitioner (see partition.h).  The two sweeps are recurrences: every decision reads the part sizes and
+// counters that all earlier moves of the same sweep changed, and every score is a chain of float operations that
+// starts from those sizes, so the order of visits and of operations is the result.  They run on the host, one
+// sample / embedding after the other, over a layout that makes a visit cheap.  What has no such order (the priority
+// of every (part, embedding) pair and the sorted cache candidates per part) runs on the GPU.
+#include "partition.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <thread>
+
+#include "radix_sort.h"
+
+namespace hctr {
+namespace {
+
+// The C library's rand() (glibc, default 128-byte state): 31 words, x[f] += x[r] with the two cursors 3 apart,
+// result = the new word >> 1; seeded by x[i] = 16807 * x[i-1] mod (2^31 - 1) and 310 discarded results.  The
+// reference draws the initial assignment from rand() without seeding it (partition.cc:70,77), which is srand(1).
+class LibcRand {
+public:
+  explicit LibcRand(unsigned seed) {
+    int64_t w = (int32_t)(seed ? seed : 1u);
+    st_[0] = (uint32_t)w;
+    for (int i = 1; i < 31; i++) {
+      w = (16807 * w) % 2147483647;
+      if (w < 0) w += 2147483647;
+      st_[i] = (uint32_t)w;
+    }
+    f_ = 3;
+    r_ = 0;
+    for (int i = 0; i < 310; i++) next();
+  }
+  int next() {
+    const uint32_t v = (st_[f_] += st_[r_]);
+    f_ = f_ == 30 ? 0 : f_ + 1;
+    r_ = r_ == 30 ? 0 : r_ + 1;
+    return (int)(v >> 1);
+  }
+
+private:
+  uint32_t st_[31];
+  int f_, r_;
+};
+
+// runs fn(t, nthreads) on up to `want` host threads
+template <typename F> void on_threads(size_t want, F &&fn) {
+  size_t hw = std::thread::hardware_concurrency();
+  const size_t nt = std::max<size_t>(1, std::min<size_t>({want, hw ? hw : 1, 16}));
+  std::vector<std::thread> pool;
+  for (size_t t = 1; t < nt; t++) pool.emplace_back([&fn, t, nt] { fn(t, nt); });
+  fn(0, nt);
+  for (auto &th : pool) th.join();
+}
+
+int first_largest(const float *v, int n) { // partition.cc:17-24
+  int r = 0;
+  for (int i = 1; i < n; i++)
+    if (v[i] > v[r]) r = i;
+  return r;
+}
+
+} // namespace
+
+Partitioner::Partitioner(const int32_t *d, size_t nd, size_t ns, const float *comm_mat, int np, int bs, unsigned seed)
+    : n_part(np), batch(bs), n_data(nd), n_slot(ns) {
+  HCTR_CHECK(d && comm_mat, "partition: null argument");
+  HCTR_CHECK(np >= 1 && np <= 256, "partition: n_part must be in 1..256");
+  HCTR_CHECK(bs >= 1, "partition: batch_size must be positive");
+  HCTR_CHECK(ns >= 1 && nd >= (size_t)np, "partition: needs at least n_part samples and one slot");
+  HCTR_CHECK(nd * ns < (1ull << 31), "partition: samples x slots must stay below 2^31");
+  const size_t n_edge = nd * ns;
+  int32_t top = 0, low = 0;
+  for (size_t i = 0; i < n_edge; i++) {
+    top = std::max(top, d[i]);
+    low = std::min(low, d[i]);
+  }
+  HCTR_CHECK(low >= 0, "partition: negative embedding id");
+  n_embed = (size_t)top + 1; // partition.cc:33-37
+  HCTR_CHECK(n_embed >= (size_t)np, "partition: fewer embeddings than parts");
+  for (int i = 0; i < np * np; i++) HCTR_CHECK(std::isfinite(comm_mat[i]), "partition: comm_mat must be finite");
+  data.assign(d, d + n_edge);
+  comm.assign(comm_mat, comm_mat + (size_t)np * np);
+  comm_t.resize(comm.size());
+  for (int i = 0; i < np; i++)
+    for (int j = 0; j < np; j++) comm_t[(size_t)j * np + i] = comm[(size_t)i * np + j];
+
+  // partition.cc:59-65: soft[i] = (1 - (1 - i/m)^batch) * m / batch below m = n_data / n_part, 1 from there on;
+  // the power by repeated squaring in float (partition.cc:7-15)
+  const size_t m = nd / np;
+  soft.assign(nd, 1.0f);
+  for (size_t i = 0; i < m; i++) {
+    float sq = (float)(1.0 - (double)((float)i / (float)m)), pw = 1.0f;
+    for (int e = bs; e; e >>= 1) {
+      if (e & 1) pw *= sq;
+      sq *= sq;
+    }
+    float v = 1 - pw;
+    v *= (float)m / (float)bs;
+    soft[i] = v;
+  }
+  dsoft.assign(nd + 1, 0.0f);
+  for (size_t i = 0; i < nd; i++) dsoft[i] = soft_at((int64_t)i + 1) - soft[i];
+
+  // partition.cc:66-80: samples first, then embeddings, one rand() each
+  LibcRand rnd(seed);
+  res_data.resize(nd);
+  res_embed.resize(n_embed);
+  cnt_data.assign(np, 0);
+  cnt_embed.assign(np, 0);
+  cnt.assign(n_embed * (size_t)np, 0);
+  for (size_t i = 0; i < nd; i++) {
+    const int p = rnd.next() % np;
+    res_data[i] = p;
+    cnt_data[p]++;
+    for (size_t s = 0; s < ns; s++) cnt[(size_t)d[i * ns + s] * np + p]++;
+  }
+  for (size_t i = 0; i < n_embed; i++) {
+    const int p = rnd.next() % np;
+    res_embed[i] = p;
+    cnt_embed[p]++;
+  }
+  // partition.cc:82-83: integer quotient, double division, kept as float
+  alpha = (float)(-100.0 / (double)(nd / np));
+  beta = (float)(-100.0 / (double)(n_embed / np));
+}
+
+void Partitioner::refine_data() {
+  const int P = n_part;
+  const size_t S = n_slot;
+  std::vector<float> score_v(P);
+  float *score = score_v.data();
+  constexpr size_t kAhead = 6; // samples whose counter rows are requested before they are needed
+  for (size_t i = 0; i < n_data; i++) {
+    if (i + kAhead < n_data) {
+      const int32_t *nx = &data[(i + kAhead) * S];
+      for (size_t s = 0; s < S; s++) {
+        __builtin_prefetch(&cnt[(size_t)nx[s] * P], 1);
+        __builtin_prefetch(&res_embed[nx[s]], 0);
+      }
+    }
+    const int32_t *row = &data[i * S];
+    const int old = res_data[i];
+    for (int k = 0; k < P; k++) score[k] = alpha * (float)(cnt_data[k] - (k == old));
+    for (size_t s = 0; s < S; s++) {
+      const int32_t *c = &cnt[(size_t)row[s] * P];
+      const float *cm = &comm_t[(size_t)res_embed[row[s]] * P]; // cm[k] = comm[k][owner of the embedding]
+      for (int k = 0; k < P; k++) {
+        // what one more sample of part k using this embedding adds to the part's soft count, not counting this sample
+        const int64_t use = (int64_t)c[k] - (k == old);
+        const float step = use < (int64_t)n_data ? dsoft[use] : 0.0f;
+        score[k] -= step * cm[k];
+      }
+    }
+    const int to = first_largest(score, P);
+    if (to != old) {
+      cnt_data[old]--;
+      cnt_data[to]++;
+      for (size_t s = 0; s < S; s++) {
+        int32_t *c = &cnt[(size_t)row[s] * P];
+        c[to]++;
+        c[old]--;
+      }
+      res_data[i] = to;
+    }
+  }
+}
+
+// partition.cc:123-131.  The sum for owner part p runs over (viewing part i != p, embedding j owned by p) in that
+// nesting order; each owner's chain is independent of the others, so they run on separate threads.
+std::vector<float> Partitioner::embed_weight_now() const {
+  const int P = n_part;
+  std::vector<float> w(P, 0.0f);
+  on_threads(P, [&](size_t t, size_t nt) {
+    for (int p = (int)t; p < P; p += (int)nt) {
+      float acc = 0.0f;
+      for (int i = 0; i < P; i++) {
+        if (i == p) continue;
+        for (size_t j = 0; j < n_embed; j++)
+          if (res_embed[j] == p) acc += soft_at(cnt[j * P + i]);
+      }
+      w[p] = acc;
+    }
+  });
+  const float scale = (float)(batch * P) / (float)n_data;
+  for (int p = 0; p < P; p++) w[p] *= scale;
+  return w;
+}
+
+void Partitioner::refine_embed() {
+  const int P = n_part;
+  std::vector<float> w = embed_weight_now();
+  std::vector<float> score_v(P), seen_v(P);
+  float *score = score_v.data(), *seen = seen_v.data();
+  for (size_t i = 0; i < n_embed; i++) {
+    const int32_t *c = &cnt[i * P];
+    const int old = res_embed[i];
+    int64_t degree = 0;
+    for (int j = 0; j < P; j++) {
+      degree += c[j];
+      // the reference counts these in float (partition.cc:138-140): above 2^24 such a counter stops growing
+      seen[j] = soft_at(std::min<int64_t>(c[j], 1 << 24));
+    }
+    const double own = (double)soft_at(degree);
+    for (int k = 0; k < P; k++) score[k] = beta * (float)(cnt_embed[k] - (k == old));
+    for (int j = 0; j < P; j++) {
+      const float *cj = &comm[(size_t)j * P];
+      for (int k = 0; k < P; k++) score[k] -= cj[k] * seen[j];
+      // partition.cc:149: the literal 0.01 makes this one subtraction a double operation
+      score[j] = (float)((double)score[j] - 0.01 * (double)w[j] * own);
+    }
+    const int to = first_largest(score, P);
+    if (to != old) {
+      cnt_embed[old]--;
+      cnt_embed[to]++;
+      res_embed[i] = to;
+      for (int j = 0; j < P; j++) {
+        const float t = soft_at(c[j]) * (float)(batch * P) / (float)n_data;
+        if (j != to) w[to] += t;
+        if (j != old) w[old] -= t;
+      }
+    }
+  }
+}
+
+// cost[i][p]: soft counts, as seen from part i, of the embeddings part p owns, added in ascending embedding id.
+// One viewing part per thread.
+void Partitioner::communication(float *cost) const {
+  const int P = n_part;
+  on_threads(P, [&](size_t t, size_t nt) {
+    std::vector<float> acc(P);
+    for (int i = (int)t; i < P; i += (int)nt) {
+      std::fill(acc.begin(), acc.end(), 0.0f);
+      for (size_t j = 0; j < n_embed; j++) acc[res_embed[j]] += soft_at(cnt[j * P + i]);
+      for (int p = 0; p < P; p++) cost[(size_t)i * P + p] = acc[p];
+    }
+  });
+  const float scale = (float)(batch * P) / (float)n_data;
+  for (int i = 0; i < P * P; i++) cost[i] *= scale;
+}
+
+namespace {
+// partition.cc:188-191: comm * soft^2 * (1/degree + 1/count), every operand widened to double by the double literals
+// and std::pow(float, long), rounded to float once.  A float squared is exact in double.
+__host__ __device__ inline float priority_value(float comm_ij, float soft_c, int64_t degree, int32_t count) {
+  const double sq = (double)soft_c * (double)soft_c;
+  return (float)(((double)comm_ij * sq) * ((1.0 / (double)degree) + (1.0 / (double)count)));
+}
+} // namespace
+
+void Partitioner::priority(float *out) const {
+  const int P = n_part;
+  on_threads(16, [&](size_t t, size_t nt) {
+    const size_t lo = n_embed * t / nt, hi = n_embed * (t + 1) / nt;
+    for (size_t j = lo; j < hi; j++) {
+      const int32_t *c = &cnt[j * P];
+      int64_t degree = 0;
+      for (int i = 0; i < P; i++) degree += c[i];
+      for (int i = 0; i < P; i++)
+        out[(size_t)i * n_embed + j] =
+            c[i] == 0 ? 0.0f : priority_value(comm[(size_t)i * P + res_embed[j]], soft_at(c[i]), degree, c[i]);
+    }
+  });
+}
+
+// ---- cache candidates on the GPU ----------------------------------------------------------------------------
+
+namespace {
+
+constexpr int kKeyBlock = 256;
+
+// A float as an unsigned key of the same order, -0 counted as +0; 0 is kept free for "owned by the part".
+__device__ inline uint32_t order_key(float v) {
+  v += 0.0f;
+  const uint32_t b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : b | 0x80000000u;
+}
+
+// One thread per embedding: reads its counter row once and writes the sort key of every part.
+__global__ __launch_bounds__(kKeyBlock) void priority_keys(const int32_t *__restrict__ cnt,
+                                                           const int32_t *__restrict__ owner,
+                                                           const float *__restrict__ soft,
+                                                           const float *__restrict__ comm, int P, uint32_t n_embed,
+                                                           uint32_t n_data, uint32_t *__restrict__ keys) {
+  const uint32_t j = blockIdx.x * kKeyBlock + threadIdx.x;
+  if (j >= n_embed) return;
+  const int32_t *c = cnt + (size_t)j * P;
+  int64_t degree = 0;
+  for (int i = 0; i < P; i++) degree += c[i];
+  const int own = owner[j];
+  for (int i = 0; i < P; i++) {
+    uint32_t key = 0;
+    if (i != own) {
+      const int32_t ci = c[i];
+      float pr = 0.0f;
+      if (ci != 0) pr = priority_value(comm[i * P + own], (uint32_t)ci < n_data ? soft[ci] : 1.0f, degree, ci);
+      key = order_key(pr);
+    }
+    keys[(size_t)i * n_embed + j] = key;
+  }
+}
+
+// list[q] = the q-th from the end of the ascending order
+__global__ __launch_bounds__(kKeyBlock) void emit_reversed(const uint32_t *__restrict__ sorted_pos, uint32_t n,
+                                                           uint32_t len, int32_t *__restrict__ list) {
+  const uint32_t q = blockIdx.x * kKeyBlock + threadIdx.x;
+  if (q < len) list[q] = (int32_t)sorted_pos[n - 1 - q];
+}
+
+struct DevMem {
+  void *p = nullptr;
+  explicit DevMem(size_t bytes) { HCTR_HIP(hipMalloc(&p, std::max<size_t>(bytes, 16))); }
+  ~DevMem() { (void)hipFree(p); }
+  DevMem(const DevMem &) = delete;
+  template <typename T> T *as() const { return (T *)p; }
+};
+
+} // namespace
+
+void Partitioner::cache_lists(size_t max_len, int32_t *lists, size_t *lens, float *ms) const {
+  const int P = n_part;
+  HCTR_CHECK(lists && lens, "partition: null argument");
+  HCTR_CHECK(n_embed < (1ull << 31), "partition: too many embeddings");
+  const uint32_t n = (uint32_t)n_embed;
+  const size_t keep = std::min<size_t>(max_len, n_embed);
+  DevMem d_cnt(cnt.size() * 4), d_owner(n_embed * 4), d_soft(soft.size() * 4), d_comm(comm.size() * 4);
+  DevMem d_keys((size_t)P * n * 4), k0((size_t)n * 4), k1((size_t)n * 4), v0((size_t)n * 4), v1((size_t)n * 4),
+      pos((size_t)n * 4), d_lists((size_t)P * keep * 4);
+  SortScratch sc;
+  sc.blocks_cap = sort_blocks(n);
+  DevMem d_hist(((size_t)1 << kSortMaxDigitBits) * sc.blocks_cap * 4), d_tot(((size_t)1 << kSortMaxDigitBits) * 4);
+  sc.ghist = d_hist.as<uint32_t>();
+  sc.bintot = d_tot.as<uint32_t>();
+  hipStream_t s = nullptr;
+  HCTR_HIP(hipMemcpyAsync(d_cnt.p, cnt.data(), cnt.size() * 4, hipMemcpyHostToDevice, s));
+  HCTR_HIP(hipMemcpyAsync(d_owner.p, res_embed.data(), n_embed * 4, hipMemcpyHostToDevice, s));
+  HCTR_HIP(hipMemcpyAsync(d_soft.p, soft.data(), soft.size() * 4, hipMemcpyHostToDevice, s));
+  HCTR_HIP(hipMemcpyAsync(d_comm.p, comm.data(), comm.size() * 4, hipMemcpyHostToDevice, s));
+  hipEvent_t e0, e1;
+  HCTR_HIP(hipEventCreate(&e0));
+  HCTR_HIP(hipEventCreate(&e1));
+  HCTR_HIP(hipEventRecord(e0, s));
+  hipLaunchKernelGGL(priority_keys, dim3(div_up(n, kKeyBlock)), dim3(kKeyBlock), 0, s, d_cnt.as<int32_t>(),
+                     d_owner.as<int32_t>(), d_soft.as<float>(), d_comm.as<float>(), P, n, (uint32_t)n_data,
+                     d_keys.as<uint32_t>());
+  HCTR_HIP(hipGetLastError());
+  for (int i = 0; i < P; i++) {
+    const uint32_t *sorted_keys;
+    radix_sort_positions<uint32_t>(s, d_keys.as<uint32_t>() + (size_t)i * n, n, 32, k0.as<uint32_t>(),
+                                   k1.as<uint32_t>(), v0.as<uint32_t>(), v1.as<uint32_t>(), pos.as<uint32_t>(), sc,
+                                   &sorted_keys);
+    lens[i] = std::min<size_t>(keep, n_embed - (size_t)cnt_embed[i]);
+    if (lens[i]) {
+      hipLaunchKernelGGL(emit_reversed, dim3(div_up(lens[i], kKeyBlock)), dim3(kKeyBlock), 0, s, pos.as<uint32_t>(), n,
+                         (uint32_t)lens[i], d_lists.as<int32_t>() + (size_t)i * keep);
+      HCTR_HIP(hipGetLastError());
+    }
+  }
+  HCTR_HIP(hipEventRecord(e1, s));
+  for (int i = 0; i < P; i++)
+    if (lens[i])
+      HCTR_HIP(hipMemcpyAsync(lists + (size_t)i * max_len, d_lists.as<int32_t>() + (size_t)i * keep, lens[i] * 4,
+                              hipMemcpyDeviceToHost, s));
+  HCTR_HIP(hipStreamSynchronize(s));
+  float t = 0.f;
+  HCTR_HIP(hipEventElapsedTime(&t, e0, e1));
+  if (ms) *ms = t;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+}
+
+} // namespace hctr

@@ -117,6 +117,39 @@ int hctr_stage_times(hctr_table *t, double *ms_total, long long *launches, int c
  * reads and writes exactly `bytes`, which is what hardware byte counters are scaled against. */
 int hctr_copy_probe(void *dst, const void *src, size_t bytes, int repeats, float *ms_avg);
 
+/* ---- offline partitioner ---------------------------------------------------------------------------------------
+ * The C surface under the python module hetuCTR_partition (csrc/partition/pybind.cc:6-25).  Results are those of the
+ * reference's PartitionStruct run without OpenMP threads: samples and embeddings visited in index order, every move
+ * applied before the next decision (with threads the reference's sweeps race on their shared counters and its result
+ * is not a function of its input).  All pointers are HOST pointers. */
+typedef struct hctr_partition hctr_partition;
+
+/* Replaces partition() / PartitionStruct::PartitionStruct (csrc/partition/partition.cc:26-87,196-206).
+ * data: n_data x n_slot embedding ids, row-major; comm_mat: n_part x n_part, comm_mat[i][j] = cost for part i of
+ * fetching a row owned by part j.  The initial assignment is the one the reference draws from the C library's
+ * rand(); seed is what srand() would have been given (the reference never seeds: 1). */
+int hctr_part_create(const int32_t *data, size_t n_data, size_t n_slot, const float *comm_mat, int n_part,
+                     int batch_size, unsigned seed, hctr_partition **out);
+int hctr_part_destroy(hctr_partition *h);
+/* n_embed = largest id + 1 (partition.cc:33-37) */
+int hctr_part_sizes(hctr_partition *h, size_t *n_data, size_t *n_embed, int *n_part);
+/* PartitionStruct::refineData / refineEmbed (partition.cc:89-120 / 122-166): one sweep over the samples / embeddings */
+int hctr_part_refine_data(hctr_partition *h);
+int hctr_part_refine_embed(hctr_partition *h);
+/* PartitionStruct::getCommunication (partition.cc:168-181): cost[n_part * n_part] */
+int hctr_part_get_communication(hctr_partition *h, float *cost);
+/* PartitionStruct::getPriority (partition.cc:183-194): priority[n_part * n_embed] */
+int hctr_part_get_priority(hctr_partition *h, float *priority);
+/* get_result / get_data_cnt / get_embed_cnt (pybind.cc:13-21); any pointer may be NULL */
+int hctr_part_get_result(hctr_partition *h, int32_t *data_part, int32_t *embed_part);
+int hctr_part_get_counts(hctr_partition *h, int32_t *data_cnt, int32_t *embed_cnt);
+/* The cache candidates the reference's driver script derives from the priorities with one numpy argsort per part
+ * (experimental/partition.py:51-57): per part, the embeddings it does not own by descending priority; equal
+ * priorities, whose order numpy leaves open, by descending id.  Runs on the current HIP device (priorities, one radix
+ * sort per part).  lists[part * max_len + q], lens[part] <= max_len entries each; kernel_ms (may be NULL) receives
+ * the device time between the first and the last kernel. */
+int hctr_part_cache_lists(hctr_partition *h, size_t max_len, int32_t *lists, size_t *lens, float *kernel_ms);
+
 /* Version string of the library. */
 const char *hctr_version(void);
 
