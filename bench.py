@@ -40,6 +40,12 @@ def parse():
                     help="sharded configs: every rank caches hot rows and feeds batches (default: rank 0 only)")
     ap.add_argument("--pull-bound", type=int, default=0, help="sharded configs: staleness bound of pulls")
     ap.add_argument("--push-bound", type=int, default=0, help="sharded configs: staleness bound of pushes")
+    ap.add_argument("--partition", action="store_true",
+                    help="time the offline partitioner on a click log over the cfg2 table instead of the training step")
+    ap.add_argument("--part-samples", type=int, default=1_000_000, help="--partition: samples of the click log")
+    ap.add_argument("--part-rounds", type=int, default=2, help="--partition: rounds of both sweeps")
+    ap.add_argument("--part-cache-frac", type=float, default=0.10,
+                    help="--partition: cache candidates kept per part, as a fraction of the table")
     return ap.parse_args()
 
 
@@ -71,6 +77,108 @@ def cpu_baseline(cfg, ks, batches, width, lr, steps):
                 ms_per_step=1e3 * dt / steps,
                 sample="%d full-size steps (%d keys each, %d-row x %d table, zero-initialised) of the same batches, "
                        "OpenMP oracle, warm" % (steps, n, rows, width))
+
+
+def reference_partitioner():
+    """The reference's partitioner built from its own sources WITH OpenMP (as shipped), or None."""
+    import importlib.util
+    d = os.path.join(ROOT, "oracle", "_ref", "partition_omp")
+    so = [f for f in os.listdir(d) if f.startswith("hetuCTR_partition")] if os.path.isdir(d) else []
+    if not so:
+        return None
+    spec = importlib.util.spec_from_file_location("hetuCTR_partition", os.path.join(d, so[0]))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def click_log(workloads, samples, scale=1.0):
+    """samples x 26 ids over the cfg2 table (per-field Zipf), as int32."""
+    cfg = dict(workloads.CONFIGS["cfg2"])
+    cfg["samples"] = samples
+    ks = workloads.KeyStream(cfg, seed=0, scale=scale)
+    data = ks.batch().reshape(-1, ks.fields * ks.hot).astype(np.int32)
+    ks.release_tables()
+    return data, ks.rows
+
+
+def main_partition(a):
+    """Offline partitioner: construction, `rounds` x (sample sweep, embedding sweep, communication cost) on the host,
+    then the cache candidates of every part on the GPU.  The CPU leg runs the reference's own sources (OpenMP build)
+    through the same steps of its driver script on a quarter-size sample of the same log."""
+    import torch
+    from hetuctr_amd import workloads
+    import hetuctr_amd.partition as hp
+    P, B = 8, 8192
+    data, rows = click_log(workloads, a.part_samples, a.scale)
+    nd = data.shape[0]
+    mat = hp.get_comm_mat(P, P)
+    t0 = time.perf_counter()
+    p = hp.partition(data, mat, P, B)
+    create_s = time.perf_counter() - t0
+    cost0 = float((p.get_communication() * mat).sum())
+    rounds, costs = [], []
+    for r in range(a.part_rounds):
+        t0 = time.perf_counter()
+        p.refine_data()
+        t1 = time.perf_counter()
+        p.refine_embed()
+        t2 = time.perf_counter()
+        c = p.get_communication()
+        t3 = time.perf_counter()
+        rounds.append({"sample_sweep_s": t1 - t0, "embedding_sweep_s": t2 - t1, "communication_s": t3 - t2})
+        costs.append(float((c * mat).sum()))
+    refine_s = sum(sum(r.values()) for r in rounds)
+    keep = int(a.part_cache_frac * p.n_embed)
+    torch.cuda.synchronize()
+    p.cache_lists(1024)                                           # warm-up: kernels loaded
+    t0 = time.perf_counter()
+    lists, kernel_ms = p.cache_lists(keep)
+    lists_s = time.perf_counter() - t0
+    list_bytes = workloads.cache_list_bytes(p.n_embed, P, keep)
+    gbs = list_bytes / (kernel_ms * 1e-3) / 1e9
+    out = {
+        "metric": "partitioner: samples refined per second (one round = sample sweep + embedding sweep + cost)",
+        "value": nd * a.part_rounds / refine_s, "unit": "samples/s", "n_gpus": 1, "steps": a.part_rounds, "warmup": 0,
+        "ms_per_step": 1e3 * refine_s / a.part_rounds, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "click log of %d samples x %d slots over the %d-id cfg2 table (per-field Zipf 1.05), "
+                               "%d parts, batch %d, cost 0.1 between all parts" % (nd, data.shape[1], rows, P, B),
+                   "n_embed": p.n_embed},
+        "construction_s": create_s, "rounds": rounds, "cost_initial": cost0, "cost_after_round": costs,
+        "cache_lists": {"kept_per_part": keep, "wall_s_with_upload_and_download": lists_s, "kernel_ms": kernel_ms},
+        "roofline": {"bound": "hbm", "kernel": "priority keys + %d radix sorts + list emit" % P, "achieved": gbs,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": int(list_bytes)},
+    }
+    p.close()
+    del lists
+    if not a.no_cpu:
+        ref = reference_partitioner()
+        if ref is None:
+            out["cpu_baseline"] = {"value": None, "error": "oracle/_ref/partition_omp is not built"}
+        else:
+            sdata, srows = click_log(workloads, a.part_samples, a.scale * 0.25)
+            t0 = time.perf_counter()
+            rp = ref.partition(sdata, mat, P, B)
+            t1 = time.perf_counter()
+            rp.refine_data()
+            rp.refine_embed()
+            rp.get_communication()
+            t2 = time.perf_counter()
+            pr = rp.get_priority()
+            owner = rp.get_result()[1]
+            for i in range(P):                                    # experimental/partition.py:53-57
+                idxs = np.where(owner == i)[0]
+                pr[i][idxs] = -1
+                np.argsort(pr[i])[len(idxs):][::-1]
+            t3 = time.perf_counter()
+            out["cpu_baseline"] = dict(
+                value=sdata.shape[0] / (t2 - t1), unit="samples/s", cores=min(16, os.cpu_count() or 1),
+                kind="reference", construction_s=t1 - t0, round_s=t2 - t1, priority_and_sort_s=t3 - t2,
+                sample="the reference's partition.cc + pybind.cc compiled with -O3 -fopenmp, one round and the "
+                       "script's priority sort on a quarter-size log (%d samples, %d ids)" % (sdata.shape[0], srows))
+    print(json.dumps(out), flush=True)
 
 
 def main_sharded(a, cfg):
@@ -194,6 +302,8 @@ def main():
         print(json.dumps({"probe": "plain_copy", "bytes_read": nbytes, "bytes_written": nbytes, "avg_ms": ms,
                           "GBps": 2 * nbytes / (ms * 1e-3) / 1e9}), flush=True)
         return
+    if a.partition:
+        return main_partition(a)
     cfg = workloads.CONFIGS[a.config]
     if cfg.get("nrank", 1) > 1:
         return main_sharded(a, cfg)

@@ -21,6 +21,8 @@ HEADERS = ["common.h", "kernels.h", "radix_sort.h", "table.h", "partition.h", os
 # operations are written explicitly where they are meant)
 HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# host code of the partitioner's sweeps: AVX2 (no fused multiply-add is formed: contraction is off above)
+EXTRA_FLAGS = {"partition.hip": ["-Xarch_host", "-march=x86-64-v3"]}
 LIB = os.path.join(LIBDIR, "libhetuctr_hip.so")
 PYMOD = os.path.join(LIBDIR, "hetuCTR" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
@@ -51,7 +53,7 @@ def build_hip(force=False, verbose=True):
         o = os.path.join(OBJ, src + ".o")
         objs.append(o)
         if force or not _newer(o, [s] + hdrs):
-            jobs.append(["hipcc"] + HIPFLAGS + ["-c", s, "-o", o])
+            jobs.append(["hipcc"] + HIPFLAGS + EXTRA_FLAGS.get(src, []) + ["-c", s, "-o", o])
     if jobs:
         if verbose:
             print("hipcc: compiling %d file(s) for gfx950" % len(jobs), flush=True)

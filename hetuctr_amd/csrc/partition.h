@@ -6,11 +6,26 @@
 // 4*n_part-byte row, one cache line for 8 parts) replaces the per-part arrays, and the transposed sample list per
 // embedding is not built at all, because what the embedding sweep counts with it is that same row.
 #pragma once
+#include <memory>
+#include <utility>
 #include <vector>
 
 #include "common.h"
 
 namespace hctr {
+
+// std::allocator whose value-less construct leaves the memory as it is (resize() without the zero fill)
+template <typename T> struct LeaveUninit : std::allocator<T> {
+  template <typename U> struct rebind {
+    using other = LeaveUninit<U>;
+  };
+  template <typename U, typename... A> void construct(U *p, A &&...a) {
+    if constexpr (sizeof...(A) == 0)
+      ::new ((void *)p) U;
+    else
+      ::new ((void *)p) U(std::forward<A>(a)...);
+  }
+};
 
 class Partitioner {
 public:
@@ -33,10 +48,12 @@ public:
 private:
   float soft_at(int64_t i) const { return i < (int64_t)n_data ? soft[i] : 1.0f; }
   std::vector<float> embed_weight_now() const;
+  template <int PC> void refine_data_sweep();
+  template <int PC> void refine_embed_sweep(std::vector<float> &w);
 
   float alpha, beta;
   std::vector<int32_t> data; // [n_data][n_slot]
-  std::vector<int32_t> cnt;  // [n_embed][n_part]: samples of the part using the embedding, once per slot
+  std::vector<int32_t, LeaveUninit<int32_t>> cnt; // [n_embed][n_part]: samples of the part using the embedding, once per slot
   std::vector<float> soft;   // [n_data]
   std::vector<float> dsoft;  // [n_data + 1]: soft_at(i + 1) - soft_at(i); the last entry (and all beyond) 0
   std::vector<float> comm;   // [n_part][n_part], comm[i][j] = cost for part i of a row owned by part j

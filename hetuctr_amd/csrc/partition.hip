@@ -109,10 +109,18 @@ Partitioner::Partitioner(const int32_t *d, size_t nd, size_t ns, const float *co
   res_embed.resize(n_embed);
   cnt_data.assign(np, 0);
   cnt_embed.assign(np, 0);
-  cnt.assign(n_embed * (size_t)np, 0);
+  // the table is zeroed by several threads: first touch of a gigabyte from one thread is the slowest step otherwise
+  cnt.resize(n_embed * (size_t)np);
+  on_threads(16, [&](size_t t, size_t nt) {
+    const size_t lo = cnt.size() * t / nt, hi = cnt.size() * (t + 1) / nt;
+    memset(cnt.data() + lo, 0, (hi - lo) * sizeof(int32_t));
+  });
+  for (size_t i = 0; i < nd; i++) res_data[i] = rnd.next() % np;
+  constexpr size_t kAhead = 8; // samples whose counter rows are requested before they are counted
   for (size_t i = 0; i < nd; i++) {
-    const int p = rnd.next() % np;
-    res_data[i] = p;
+    if (i + kAhead < nd)
+      for (size_t s = 0; s < ns; s++) __builtin_prefetch(&cnt[(size_t)d[(i + kAhead) * ns + s] * np], 1);
+    const int p = res_data[i];
     cnt_data[p]++;
     for (size_t s = 0; s < ns; s++) cnt[(size_t)d[i * ns + s] * np + p]++;
   }
@@ -126,8 +134,8 @@ Partitioner::Partitioner(const int32_t *d, size_t nd, size_t ns, const float *co
   beta = (float)(-100.0 / (double)(n_embed / np));
 }
 
-void Partitioner::refine_data() {
-  const int P = n_part;
+template <int PC> void Partitioner::refine_data_sweep() {
+  const int P = PC ? PC : n_part;
   const size_t S = n_slot;
   std::vector<float> score_v(P);
   float *score = score_v.data();
@@ -167,19 +175,46 @@ void Partitioner::refine_data() {
   }
 }
 
+void Partitioner::refine_data() {
+  switch (n_part) {
+  case 2: refine_data_sweep<2>(); break;
+  case 4: refine_data_sweep<4>(); break;
+  case 8: refine_data_sweep<8>(); break;
+  case 16: refine_data_sweep<16>(); break;
+  default: refine_data_sweep<0>();
+  }
+}
+
 // partition.cc:123-131.  The sum for owner part p runs over (viewing part i != p, embedding j owned by p) in that
-// nesting order; each owner's chain is independent of the others, so they run on separate threads.
+// nesting order.  Unused (part, embedding) pairs add soft[0] = 0 and are left out.  The counter table is read once,
+// by threads over ranges of j that keep the nonzero terms per (p, i); a chain then adds its terms range after range.
 std::vector<float> Partitioner::embed_weight_now() const {
   const int P = n_part;
+  size_t nt_used = 1;
+  std::vector<std::vector<std::vector<float>>> terms; // [thread][p * P + i]
+  on_threads(16, [&](size_t t, size_t nt) {
+    if (t == 0) {
+      nt_used = nt;
+      terms.assign(nt, std::vector<std::vector<float>>((size_t)P * P));
+    }
+  });
+  on_threads(nt_used, [&](size_t t, size_t nt) {
+    auto &mine = terms[t];
+    const size_t lo = n_embed * t / nt, hi = n_embed * (t + 1) / nt;
+    for (size_t j = lo; j < hi; j++) {
+      const int32_t *c = &cnt[j * P];
+      const int p = res_embed[j];
+      for (int i = 0; i < P; i++)
+        if (c[i] != 0 && i != p) mine[(size_t)p * P + i].push_back(soft_at(c[i]));
+    }
+  });
   std::vector<float> w(P, 0.0f);
   on_threads(P, [&](size_t t, size_t nt) {
     for (int p = (int)t; p < P; p += (int)nt) {
       float acc = 0.0f;
-      for (int i = 0; i < P; i++) {
-        if (i == p) continue;
-        for (size_t j = 0; j < n_embed; j++)
-          if (res_embed[j] == p) acc += soft_at(cnt[j * P + i]);
-      }
+      for (int i = 0; i < P; i++)
+        for (size_t r = 0; r < nt_used; r++)
+          for (float v : terms[r][(size_t)p * P + i]) acc += v;
       w[p] = acc;
     }
   });
@@ -188,39 +223,68 @@ std::vector<float> Partitioner::embed_weight_now() const {
   return w;
 }
 
-void Partitioner::refine_embed() {
-  const int P = n_part;
-  std::vector<float> w = embed_weight_now();
-  std::vector<float> score_v(P), seen_v(P);
+// PC: the number of parts when known at compile time (loops over parts unroll), 0 for any
+template <int PC> void Partitioner::refine_embed_sweep(std::vector<float> &w) {
+  const int P = PC ? PC : n_part;
+  std::vector<float> score_v(P), seen_v(P), base_v(P), below_v(P);
   float *score = score_v.data(), *seen = seen_v.data();
+  // beta * size of part k, with and without the embedding under decision; refreshed for the two parts of a move
+  float *base = base_v.data(), *below = below_v.data();
+  for (int k = 0; k < P; k++) {
+    base[k] = beta * (float)cnt_embed[k];
+    below[k] = beta * (float)(cnt_embed[k] - 1);
+  }
+  const float per_batch = (float)(batch * P), samples = (float)n_data;
   for (size_t i = 0; i < n_embed; i++) {
     const int32_t *c = &cnt[i * P];
     const int old = res_embed[i];
     int64_t degree = 0;
-    for (int j = 0; j < P; j++) {
-      degree += c[j];
+    for (int j = 0; j < P; j++) degree += c[j];
+    for (int k = 0; k < P; k++) score[k] = base[k];
+    score[old] = below[old];
+    // A part that never uses the embedding sees soft count 0 (soft[0] is exactly 0): subtracting comm * 0 leaves
+    // every score as it is, so that part's row of products is skipped; an embedding nobody uses skips all of it.
+    if (degree != 0) {
+      const double own = (double)soft_at(degree);
       // the reference counts these in float (partition.cc:138-140): above 2^24 such a counter stops growing
-      seen[j] = soft_at(std::min<int64_t>(c[j], 1 << 24));
-    }
-    const double own = (double)soft_at(degree);
-    for (int k = 0; k < P; k++) score[k] = beta * (float)(cnt_embed[k] - (k == old));
-    for (int j = 0; j < P; j++) {
-      const float *cj = &comm[(size_t)j * P];
-      for (int k = 0; k < P; k++) score[k] -= cj[k] * seen[j];
-      // partition.cc:149: the literal 0.01 makes this one subtraction a double operation
-      score[j] = (float)((double)score[j] - 0.01 * (double)w[j] * own);
+      for (int j = 0; j < P; j++) seen[j] = soft_at(std::min<int64_t>(c[j], 1 << 24));
+      for (int j = 0; j < P; j++) {
+        if (seen[j] != 0.0f) {
+          const float *cj = &comm[(size_t)j * P];
+          for (int k = 0; k < P; k++) score[k] -= cj[k] * seen[j];
+        }
+        // partition.cc:149: the literal 0.01 makes this one subtraction a double operation
+        score[j] = (float)((double)score[j] - 0.01 * (double)w[j] * own);
+      }
     }
     const int to = first_largest(score, P);
     if (to != old) {
       cnt_embed[old]--;
       cnt_embed[to]++;
       res_embed[i] = to;
-      for (int j = 0; j < P; j++) {
-        const float t = soft_at(c[j]) * (float)(batch * P) / (float)n_data;
-        if (j != to) w[to] += t;
-        if (j != old) w[old] -= t;
+      for (int k : {old, to}) {
+        base[k] = beta * (float)cnt_embed[k];
+        below[k] = beta * (float)(cnt_embed[k] - 1);
       }
+      if (degree != 0)
+        for (int j = 0; j < P; j++) {
+          if (c[j] == 0) continue; // soft[0] is 0: the weights would change by 0
+          const float t = soft_at(c[j]) * per_batch / samples;
+          if (j != to) w[to] += t;
+          if (j != old) w[old] -= t;
+        }
     }
+  }
+}
+
+void Partitioner::refine_embed() {
+  std::vector<float> w = embed_weight_now();
+  switch (n_part) {
+  case 2: refine_embed_sweep<2>(w); break;
+  case 4: refine_embed_sweep<4>(w); break;
+  case 8: refine_embed_sweep<8>(w); break;
+  case 16: refine_embed_sweep<16>(w); break;
+  default: refine_embed_sweep<0>(w);
   }
 }
 
@@ -277,22 +341,32 @@ __device__ inline uint32_t order_key(float v) {
   return (b & 0x80000000u) ? ~b : b | 0x80000000u;
 }
 
-// One thread per embedding: reads its counter row once and writes the sort key of every part.
+// One thread per embedding: reads its counter row once and writes the sort key of every part.  PC: the number of
+// parts when known at compile time (the row is then read with 16-byte loads), 0 for any.
+template <int PC>
 __global__ __launch_bounds__(kKeyBlock) void priority_keys(const int32_t *__restrict__ cnt,
                                                            const int32_t *__restrict__ owner,
                                                            const float *__restrict__ soft,
-                                                           const float *__restrict__ comm, int P, uint32_t n_embed,
+                                                           const float *__restrict__ comm, int n_part, uint32_t n_embed,
                                                            uint32_t n_data, uint32_t *__restrict__ keys) {
+  const int P = PC ? PC : n_part;
   const uint32_t j = blockIdx.x * kKeyBlock + threadIdx.x;
   if (j >= n_embed) return;
   const int32_t *c = cnt + (size_t)j * P;
+  int32_t row[PC ? PC : 1];
+  if (PC) {
+    for (int q = 0; q < PC / 4; q++) {
+      const int4 v = reinterpret_cast<const int4 *>(c)[q];
+      row[4 * q] = v.x, row[4 * q + 1] = v.y, row[4 * q + 2] = v.z, row[4 * q + 3] = v.w;
+    }
+  }
   int64_t degree = 0;
-  for (int i = 0; i < P; i++) degree += c[i];
+  for (int i = 0; i < P; i++) degree += PC ? row[i] : c[i];
   const int own = owner[j];
   for (int i = 0; i < P; i++) {
     uint32_t key = 0;
     if (i != own) {
-      const int32_t ci = c[i];
+      const int32_t ci = PC ? row[i] : c[i];
       float pr = 0.0f;
       if (ci != 0) pr = priority_value(comm[i * P + own], (uint32_t)ci < n_data ? soft[ci] : 1.0f, degree, ci);
       key = order_key(pr);
@@ -341,7 +415,11 @@ void Partitioner::cache_lists(size_t max_len, int32_t *lists, size_t *lens, floa
   HCTR_HIP(hipEventCreate(&e0));
   HCTR_HIP(hipEventCreate(&e1));
   HCTR_HIP(hipEventRecord(e0, s));
-  hipLaunchKernelGGL(priority_keys, dim3(div_up(n, kKeyBlock)), dim3(kKeyBlock), 0, s, d_cnt.as<int32_t>(),
+  auto keys_kernel = priority_keys<0>;
+  if (P == 4) keys_kernel = priority_keys<4>;
+  if (P == 8) keys_kernel = priority_keys<8>;
+  if (P == 16) keys_kernel = priority_keys<16>;
+  hipLaunchKernelGGL(keys_kernel, dim3(div_up(n, kKeyBlock)), dim3(kKeyBlock), 0, s, d_cnt.as<int32_t>(),
                      d_owner.as<int32_t>(), d_soft.as<float>(), d_comm.as<float>(), P, n, (uint32_t)n_data,
                      d_keys.as<uint32_t>());
   HCTR_HIP(hipGetLastError());
@@ -349,7 +427,7 @@ void Partitioner::cache_lists(size_t max_len, int32_t *lists, size_t *lens, floa
     const uint32_t *sorted_keys;
     radix_sort_positions<uint32_t>(s, d_keys.as<uint32_t>() + (size_t)i * n, n, 32, k0.as<uint32_t>(),
                                    k1.as<uint32_t>(), v0.as<uint32_t>(), v1.as<uint32_t>(), pos.as<uint32_t>(), sc,
-                                   &sorted_keys);
+                                   &sorted_keys, false, true);
     lens[i] = std::min<size_t>(keep, n_embed - (size_t)cnt_embed[i]);
     if (lens[i]) {
       hipLaunchKernelGGL(emit_reversed, dim3(div_up(lens[i], kKeyBlock)), dim3(kKeyBlock), 0, s, pos.as<uint32_t>(), n,

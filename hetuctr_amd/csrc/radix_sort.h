@@ -35,17 +35,18 @@ inline int sort_first_digit_bits(int bits) {
 // buffers of n elements; the sorted keys end in *keys_sorted (one of tmp_k0/tmp_k1) and the sorted
 // positions in vals_out.  n == 0 is a no-op.  first_hist_done: scratch.ghist already holds the per-block counts of
 // the first pass' digit (sort_first_digit_bits(bits) low bits, tiles of kSortTile keys), written by the kernel
-// that made the keys.
+// that made the keys.  long_runs: most keys are expected to repeat over long stretches of the input (the digit counts
+// then add once per wave where a wave's keys agree).
 template <typename K>
 void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
                           uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
-                          const K **keys_sorted, bool first_hist_done = false);
+                          const K **keys_sorted, bool first_hist_done = false, bool long_runs = false);
 
 extern template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *,
                                                     uint32_t *, uint32_t *, uint32_t *, uint32_t *,
-                                                    const SortScratch &, const uint32_t **, bool);
+                                                    const SortScratch &, const uint32_t **, bool, bool);
 extern template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *,
                                                     uint64_t *, uint32_t *, uint32_t *, uint32_t *,
-                                                    const SortScratch &, const uint64_t **, bool);
+                                                    const SortScratch &, const uint64_t **, bool, bool);
 
 } // namespace hctr

@@ -18,7 +18,9 @@ constexpr int kWaves = kSortBlock / kWave;
 constexpr int kSub = kSortTile / kWaves; // keys per wave
 constexpr int kRounds = kSub / kWave;    // 64-key groups per wave
 
-template <typename K>
+// kRuns: the keys are expected to come in long runs of equal digits (a sort key that is constant over most of the
+// input).  A wave whose 64 keys share one digit then adds once instead of 64 times to the same LDS word.
+template <typename K, bool kRuns>
 __global__ __launch_bounds__(kSortBlock) void digit_histogram(const K *__restrict__ keys, uint32_t n, int shift,
                                                               int dbits, uint32_t *__restrict__ ghist,
                                                               uint32_t nblocks) {
@@ -27,10 +29,27 @@ __global__ __launch_bounds__(kSortBlock) void digit_histogram(const K *__restric
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
   __syncthreads();
   const uint32_t base = blockIdx.x * kSortTile;
+  K held[kSortItems]; // all loads of the thread first: they are in flight together
 #pragma unroll
   for (int k = 0; k < kSortItems; k++) {
     uint32_t idx = base + k * kSortBlock + threadIdx.x;
-    if (idx < n) atomicAdd(&h[(uint32_t)(keys[idx] >> shift) & mask], 1u);
+    held[k] = idx < n ? keys[idx] : (K)0;
+  }
+#pragma unroll
+  for (int k = 0; k < kSortItems; k++) {
+    uint32_t idx = base + k * kSortBlock + threadIdx.x;
+    const bool in = idx < n;
+    const uint32_t d = in ? (uint32_t)(held[k] >> shift) & mask : 0;
+    if (kRuns) {
+      // lanes inside the input are a prefix of the wave, so lane 0 is inside whenever any lane is
+      const unsigned long long act = __ballot(in);
+      const uint32_t d0 = __builtin_amdgcn_readfirstlane(d);
+      if (act != 0 && __ballot(in && d == d0) == act) {
+        if (lane_id() == 0) atomicAdd(&h[d0], (uint32_t)__popcll(act));
+        continue;
+      }
+    }
+    if (in) atomicAdd(&h[d], 1u);
   }
   __syncthreads();
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) ghist[(size_t)i * nblocks + blockIdx.x] = h[i];
@@ -177,7 +196,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
 template <typename K>
 void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
                           uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
-                          const K **keys_sorted, bool first_hist_done) {
+                          const K **keys_sorted, bool first_hist_done, bool long_runs) {
   *keys_sorted = keys_in;
   if (n == 0) return;
   if (bits < 1) bits = 1;
@@ -196,9 +215,14 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
     K *kout = ktmp[p & 1];
     uint32_t *vout = (p == passes - 1) ? vals_out : vtmp[p & 1];
     const uint32_t nb = 1u << dbits;
-    if (p > 0 || !first_hist_done)
-      hipLaunchKernelGGL(digit_histogram<K>, dim3(nblocks), dim3(kSortBlock), 0, stream, kin, n, shift, dbits,
-                         scratch.ghist, nblocks);
+    if (p > 0 || !first_hist_done) {
+      if (long_runs)
+        hipLaunchKernelGGL((digit_histogram<K, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, n, shift,
+                           dbits, scratch.ghist, nblocks);
+      else
+        hipLaunchKernelGGL((digit_histogram<K, false>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, n, shift,
+                           dbits, scratch.ghist, nblocks);
+    }
     hipLaunchKernelGGL(scan_bins, dim3(nb), dim3(kSortBlock), 0, stream, scratch.ghist, nblocks, scratch.bintot);
     if (p == 0)
       hipLaunchKernelGGL((scatter<K, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
@@ -216,9 +240,9 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
 
 template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *, uint32_t *,
                                              uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
-                                             const uint32_t **, bool);
+                                             const uint32_t **, bool, bool);
 template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *, uint64_t *,
                                              uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
-                                             const uint64_t **, bool);
+                                             const uint64_t **, bool, bool);
 
 } // namespace hctr

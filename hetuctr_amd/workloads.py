@@ -129,3 +129,13 @@ def stage_bytes(stage, n_keys, n_unique, n_prev, u_prev, width):
     if stage == "gather":              # output write + unique-row read; idx_map read per key; offset read per unique
         return row * n_keys + row * n_unique + 8 * n_keys + 8 * n_unique
     raise KeyError(stage)
+
+
+def cache_list_bytes(n_embed, n_part, kept):
+    """Algorithmic bytes of the partitioner's cache-candidate kernels: per embedding one counter row (4 B per part) and
+    the owner read, one 4-byte key per part written; per part a 32-bit radix sort in four 8-bit passes (key read for
+    the counts, key + position read and written for the move; the first pass reads no positions) and the kept list
+    (position read, id written)."""
+    keys = n_embed * (4 * n_part + 4 + 4 * n_part)
+    sort = n_part * n_embed * (4 * (4 + 8 + 8) - 4)
+    return keys + sort + n_part * min(kept, n_embed) * 8
