@@ -40,6 +40,9 @@ def parse():
                     help="sharded configs: every rank caches hot rows and feeds batches (default: rank 0 only)")
     ap.add_argument("--pull-bound", type=int, default=0, help="sharded configs: staleness bound of pulls")
     ap.add_argument("--push-bound", type=int, default=0, help="sharded configs: staleness bound of pushes")
+    ap.add_argument("--layout", choices=("random", "partitioned"), default="random",
+                    help="sharded configs: owners drawn uniformly and the hottest rows cached (random), or owners, "
+                         "cache contents and per-rank batches from the offline partitioner run on a click log")
     ap.add_argument("--partition", action="store_true",
                     help="time the offline partitioner on a click log over the cfg2 table instead of the training step")
     ap.add_argument("--part-samples", type=int, default=1_000_000, help="--partition: samples of the click log")
@@ -193,10 +196,20 @@ def main_sharded(a, cfg):
     active = list(range(R)) if a.active_peers else [0]
     ks = workloads.KeyStream(cfg, seed=0, scale=a.scale)
     nb = max(2, a.batches)
-    batches = {r: [ks.batch() for _ in range(nb)] for r in active}
+    layout_info = None
+    if a.layout == "partitioned":
+        say = lambda m: print("[bench] " + m, file=sys.stderr, flush=True)
+        root, storage, per_rank, layout_info = workloads.partitioned_layout(
+            ks, R, cfg["cache_frac"], R * ks.samples * (nb + 1), ks.samples, rounds=3, cached_ranks=active, log=say)
+        nb = min(nb, min(len(per_rank[r]) for r in active))
+        assert nb >= 2, "the click log leaves a rank fewer than two full batches"
+        batches = {r: per_rank[r][:nb] for r in active}
+        del per_rank
+    else:
+        batches = {r: [ks.batch() for _ in range(nb)] for r in active}
+        root, storage = workloads.shard_layout(ks, R, cfg["cache_frac"], cached_ranks=active)
     ks.release_tables()
     n = batches[0][0].shape[0]
-    root, storage = workloads.shard_layout(ks, R, cfg["cache_frac"], cached_ranks=active)
     print("[bench] %s: %d rows x %d over %d shards, rank 0 owns %d and caches %d rows, %d keys/batch, ranks with "
           "batches: %s" % (a.config, ks.rows, width, R, int((root == 0).sum()),
                            storage[0].shape[0] - int((root == 0).sum()), n, active), file=sys.stderr, flush=True)
@@ -258,11 +271,15 @@ def main_sharded(a, cfg):
         "metric": "sparse IDs/sec per train step (pull+push)", "value": keys_step * a.steps / dt, "unit": "IDs/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "%s: %d shards of a %d-row x %d fp32 table (uniform owners) on one GPU behind the "
-                               "loopback, ranks %s feed batches of %d keys (per-field Zipf %.2f) and cache the hottest "
-                               "%.0f%% of their remote rows, bounds pull/push %d/%d; the other ranks only serve" %
-                               (a.config, R, ks.rows, width, active, n, cfg["alpha"], 100 * cfg["cache_frac"],
-                                bounds[0], bounds[1]),
+        "config": {"workload": "%s: %d shards of a %d-row x %d fp32 table (%s) on one GPU behind the "
+                               "loopback, ranks %s feed batches of %d keys (per-field Zipf %.2f) and cache %.0f%% of "
+                               "their remote rows (%s), bounds pull/push %d/%d; the other ranks only serve" %
+                               (a.config, R, ks.rows, width,
+                                "uniform owners" if a.layout == "random" else "owners from the offline partitioner",
+                                active, n, cfg["alpha"], 100 * cfg["cache_frac"],
+                                "the hottest" if a.layout == "random" else "the partitioner's first candidates; "
+                                "each rank's batches are the samples assigned to it", bounds[0], bounds[1]),
+                   "layout": a.layout, "partitioner": layout_info,
                    "keys_per_step": keys_step, "unique_keys_per_step": us, "width": width, "rows": ks.rows},
         "cache_per_step_all_ranks": {"remote_unique_keys_hit": hit, "missed_not_cached": miss, "refreshed": refresh,
                                      "rows_pushed_to_owners": pushed, "rows_returned_by_owners": served},

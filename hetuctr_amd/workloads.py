@@ -103,6 +103,47 @@ def shard_layout(ks, nrank, cache_frac, seed=0, cached_ranks=(0,)):
     return root, storage
 
 
+def partitioned_layout(ks, nrank, cache_frac, log_samples, batch_samples, rounds=3, cached_ranks=(0,), log=None):
+    """Owners, resident ids and per-rank batches as the reference's offline flow produces them
+    (experimental/partition.py): a click log of `log_samples` samples is drawn from the stream, the partitioner
+    assigns its samples and the ids to `nrank` parts, a rank in `cached_ranks` stores what it owns plus the first
+    `cache_frac` of its cache candidates (counted like shard_layout: a fraction of the ids it does not own), and a
+    rank's batches are its own samples in log order, `batch_samples` at a time.  Ids beyond the largest id of the log
+    are owned round-robin.  Returns (root, storage, batches per rank, info)."""
+    from . import partition as hp
+    saved = ks.samples
+    ks.samples = log_samples
+    data = ks.batch().reshape(log_samples, ks.fields * ks.hot).astype(np.int32)
+    ks.samples = saved
+    mat = hp.get_comm_mat(nrank, nrank)
+    p = hp.partition(data, mat, nrank, batch_samples)
+    cost = [float((p.get_communication() * mat).sum())]
+    for _ in range(rounds):
+        p.refine_data()
+        p.refine_embed()
+        cost.append(float((p.get_communication() * mat).sum()))
+    part_of_sample, part_of_id = p.get_result()
+    root = (np.arange(ks.rows) % nrank).astype(np.uint8)
+    root[:p.n_embed] = part_of_id
+    keep = {r: int(np.ceil(cache_frac * (ks.rows - int((root == r).sum())))) for r in cached_ranks}
+    lists, kernel_ms = p.cache_lists(max(keep.values()) if keep else 0)
+    p.close()
+    storage = [np.flatnonzero(root == r).astype(np.int64) for r in range(nrank)]
+    for r in cached_ranks:
+        storage[r] = np.concatenate([storage[r], lists[r][:keep[r]].astype(np.int64)])
+    batches = {}
+    for r in range(nrank):
+        mine = data[part_of_sample == r].astype(np.int64)
+        full = mine.shape[0] // batch_samples
+        batches[r] = [mine[b * batch_samples:(b + 1) * batch_samples].reshape(-1) for b in range(full)]
+    info = {"log_samples": log_samples, "rounds": rounds, "cost_per_round": cost, "cache_list_kernel_ms": kernel_ms,
+            "samples_per_rank": np.bincount(part_of_sample, minlength=nrank).tolist(),
+            "ids_per_rank": np.bincount(root, minlength=nrank).tolist()}
+    if log:
+        log("partitioned layout: cost %s, samples per rank %s" % (["%.0f" % c for c in cost], info["samples_per_rank"]))
+    return root, storage, batches, info
+
+
 def sharded_extra_bytes(width, touched_cached, pushed, received, queried, returned, refreshed):
     """Bytes a step moves on top of algorithmic_bytes when rows are sharded and cached (same accounting): the
     pending-gradient store and update counter of touched cached rows, the push buffer and its loopback copy,

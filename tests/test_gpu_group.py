@@ -139,6 +139,59 @@ def test_partitioned_table_with_hot_row_cache(bounds, cached):
     p.close()
 
 
+def test_layout_from_the_offline_partitioner():
+    # the whole offline flow at 1/100 scale: click log -> partitioner (owners, cache candidates, samples per rank)
+    # -> eight tables that train on their own samples; parity with the oracle, and fewer rows cross ranks than
+    # with uniform owners and the hottest rows cached
+    from hetuctr_amd import workloads
+    say("layout from the partitioner")
+    cfg = workloads.CONFIGS["cfg3"]
+    R, width = cfg["nrank"], cfg["width"]
+    ranks = tuple(range(R))
+    ks = workloads.KeyStream(cfg, seed=0, scale=0.01)
+    steps = 4
+    root, storage, batches, info = workloads.partitioned_layout(ks, R, cfg["cache_frac"], R * ks.samples * (steps + 1),
+                                                                ks.samples, rounds=3, cached_ranks=ranks)
+    assert info["cost_per_round"][-1] < 0.8 * info["cost_per_round"][0]
+    assert min(len(b) for b in batches.values()) >= steps
+    for r in ranks:                                   # a rank stores what it owns and nothing twice
+        assert np.array_equal(np.sort(storage[r][:int((root == r).sum())]), np.flatnonzero(root == r))
+        assert np.unique(storage[r]).shape[0] == storage[r].shape[0]
+
+    def run(root, storage, batches, check):
+        p = Pair(R, ks.rows, width, root, storage, init=("Uniform", -0.1, 0.1), lr=cfg["lr"], bounds=(2, 3), seed=0)
+        rng = np.random.default_rng(4)
+        prev_n = [0] * R
+        totals = np.zeros(6)
+        for step in range(steps):
+            keys = [batches[r][step] for r in range(R)]
+            p.preprocess(keys, device_keys=True)
+            if check:
+                p.compare_ints(INT_ITEMS_PRE, "step %d" % step)
+            out, ref = p.push_pull([rng.normal(0, 1e-2, size=(prev_n[r], width)).astype(np.float32) for r in range(R)])
+            if check:
+                p.compare_ints(INT_ITEMS_POST, "step %d" % step)
+                for r in range(R):
+                    assert_close(out[r], ref[r], 1e-5, "dst step %d rank %d" % (step, r))
+            for r in range(R):
+                totals += p.tables[r].fetch(capi.STATS)[:6]
+            prev_n = [k.shape[0] for k in keys]
+        if check:
+            p.compare_state(1e-5, "end")
+        p.close()
+        return totals
+
+    hit, miss, refreshed, pushed, returned, received = run(root, storage, batches, True)
+    assert pushed == received and returned == miss + refreshed
+    ks2 = workloads.KeyStream(cfg, seed=0, scale=0.01)
+    root2, storage2 = workloads.shard_layout(ks2, R, cfg["cache_frac"], cached_ranks=ranks)
+    plain = {r: [ks2.batch() for _ in range(steps)] for r in range(R)}
+    _, miss2, refreshed2, pushed2, returned2, _ = run(root2, storage2, plain, False)
+    say("  rows returned by owners: %d partitioned, %d uniform owners; pushed %d vs %d" %
+        (returned, returned2, pushed, pushed2))
+    assert returned < returned2 and pushed < pushed2
+
+
 def test_hand_computed_staleness_scenario():
     # same scenario as tests/test_oracle_update.py::test_staleness_scenario_both_update, on the GPU
     root = np.array([0, 1], np.uint8)
