@@ -75,9 +75,17 @@ def cpu_baseline(cfg, ks, batches, width, lr, steps):
         o.push_pull_into([grad], [dst])
     dt = time.perf_counter() - t0
     cores = o.num_threads()
+    o.set_parallel(False)                                 # the same steps on one host thread
+    one = max(1, steps // 5)
+    t0 = time.perf_counter()
+    for s in range(one):
+        o.preprocess_raw([batches[(s + 2) % len(batches)]])
+        o.push_pull_into([grad], [dst])
+    dt1 = time.perf_counter() - t0
     o.close()
     return dict(value=n * steps / dt, unit="IDs/s", cores=cores, kind="port",
                 ms_per_step=1e3 * dt / steps,
+                single_thread={"value": n * one / dt1, "ms_per_step": 1e3 * dt1 / one, "steps": one},
                 sample="%d full-size steps (%d keys each, %d-row x %d table, zero-initialised) of the same batches, "
                        "OpenMP oracle, warm" % (steps, n, rows, width))
 
