@@ -100,10 +100,16 @@ class Shard {
 
   // ---- stages, each only enqueues on the group's stream (names follow hetu_gpu_table.h:82-97) ----
   void swap_batches() { std::swap(cur, prev); }
-  void preprocess_index(const int64_t *keys, size_t n);
+  void preprocess_index(const int64_t *keys, size_t n) {
+    ingest_keys(keys, n);
+    index_batch();
+  }
+  void ingest_keys(const int64_t *keys, size_t n); // the caller's ids -> device copy and sort keys
+  void index_batch();                              // sort, unique, run lists of the ingested batch
   void preprocess_gradient();
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
+  void check_key_error();                   // raises if the ingested batch held a key outside [0, length)
   void generate_gradient(const float *grad);
   void generate_query();
   void handle_gradient();
@@ -150,8 +156,16 @@ class Group {
   const int nrank;
   const int device_id;
   const std::string key;
-  hipStream_t stream = nullptr;
+  hipStream_t stream = nullptr;          // the stream the stages enqueue on (see StreamSwitch)
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  // Single shard: preprocess enqueues its work on a second stream and returns once the caller's ids are consumed;
+  // sorting and deduplicating them has no dependence on the pending gradient push, so the next push_pull starts the
+  // push on the main stream right away and only the gather waits for both.
+  hipStream_t index_stream = nullptr;
+  hipEvent_t ev_index = nullptr, ev_keys = nullptr;
+  bool defer_index = false;              // the mode is on (one shard, HETUCTR_DEFER_INDEX != 0)
+  bool index_pending = false;            // a batch's index is enqueued and nobody has waited for it yet
+  void flush_index();                    // waits for a pending index and takes its results over
   std::vector<Shard *> members;
   DeviceBuf desc_dev;
   CopyDesc *desc_host = nullptr;
@@ -181,6 +195,7 @@ class Group {
   void push_pull_one(int rank, const float *grad, float *dst);
 
  private:
+  void exchange_shapes();
   void exchange_query();
   void exchange_return();
   void run_copies(std::vector<CopyDesc> &descs);
@@ -210,6 +225,14 @@ struct StageScope {
   ~StageScope() {
     if (idx >= 0) (void)hipEventRecord(g.marks[idx].b, g.stream);
   }
+};
+
+// makes the stages enqueue on another stream for the lifetime of the object
+struct StreamSwitch {
+  Group &g;
+  hipStream_t saved;
+  StreamSwitch(Group &grp, hipStream_t s) : g(grp), saved(grp.stream) { g.stream = s; }
+  ~StreamSwitch() { g.stream = saved; }
 };
 
 std::shared_ptr<Group> find_or_create_group(int nrank, int device_id, const std::string &ip, int port);

@@ -197,7 +197,7 @@ void Shard::reserve_batch_scratch(uint32_t n) {
 }
 
 // csrc/core/preprocess.cu:92-141
-void Shard::preprocess_index(const int64_t *keys, size_t n) {
+void Shard::ingest_keys(const int64_t *keys, size_t n) {
   HCTR_CHECK(n < 0xfffffff0ull, "a batch holds fewer than 2^32 keys");
   HCTR_CHECK(keys != nullptr || n == 0, "null key pointer");
   hipStream_t s = group->stream;
@@ -225,6 +225,12 @@ void Shard::preprocess_index(const int64_t *keys, size_t n) {
       launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, comp.p, err_ptr(),
                        visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), ghist.as<uint32_t>());
     }
+  }
+}
+
+void Shard::index_batch() {
+  hipStream_t s = group->stream;
+  if (cur.n != 0) {
     SortScratch sc;
     sc.ghist = ghist.as<uint32_t>();
     sc.bintot = bintot.as<uint32_t>();
@@ -298,8 +304,13 @@ void Shard::finish_preprocess() {
       prev.push_cnt[i] = mirror->st.push_cnt[i];
     }
   }
+  check_key_error();
+}
+
+void Shard::check_key_error() {
   if (mirror->st.err) {
     const uint32_t e = mirror->st.err;
+    mirror->st.err = 0;
     HCTR_HIP(hipMemsetAsync(err_ptr(), 0, 4, group->stream));
     HCTR_CHECK(!(e & 1u), "preprocess: a key lies outside [0, length) (it was treated as id 0)");
   }
@@ -469,6 +480,7 @@ template <typename V> size_t put64(const V &v, size_t n, void *out, size_t cap) 
 
 size_t Shard::fetch(int which, void *out, size_t cap) {
   HCTR_HIP(hipSetDevice(cfg.device_id));
+  group->flush_index();
   HCTR_HIP(hipStreamSynchronize(group->stream));
   const int R = cfg.nrank;
   const uint64_t id_mask = kl.id_bits >= 64 ? ~0ull : (((uint64_t)1 << kl.id_bits) - 1);
@@ -546,6 +558,11 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   // a blocking stream, like the reference's cudaStreamCreate (table_initialize.cu:16): work the caller queued on the
   // legacy default stream (torch's default) is ordered before ours without an explicit synchronisation
   HCTR_HIP(hipStreamCreate(&stream));
+  HCTR_HIP(hipStreamCreate(&index_stream));
+  HCTR_HIP(hipEventCreateWithFlags(&ev_index, hipEventDisableTiming));
+  HCTR_HIP(hipEventCreateWithFlags(&ev_keys, hipEventDisableTiming));
+  const char *defer = getenv("HETUCTR_DEFER_INDEX");
+  defer_index = nr == 1 && !(defer && atoi(defer) == 0);
   HCTR_HIP(hipEventCreate(&ev0));
   HCTR_HIP(hipEventCreate(&ev1));
   a_keys_.resize(nr);
@@ -562,6 +579,9 @@ Group::~Group() {
   for (auto &m : marks) { (void)hipEventDestroy(m.a); (void)hipEventDestroy(m.b); }
   for (auto e : event_pool) (void)hipEventDestroy(e);
   if (stream) (void)hipStreamDestroy(stream);
+  if (index_stream) (void)hipStreamDestroy(index_stream);
+  if (ev_index) (void)hipEventDestroy(ev_index);
+  if (ev_keys) (void)hipEventDestroy(ev_keys);
 }
 
 void Group::join(Shard *s) {
@@ -573,6 +593,7 @@ void Group::join(Shard *s) {
 void Group::leave(Shard *s) {
   std::lock_guard<std::mutex> lk(mu_);
   if (members[s->cfg.rank] == s) members[s->cfg.rank] = nullptr;
+  index_pending = false;
 }
 
 bool Group::complete() const {
@@ -711,9 +732,63 @@ void Group::sync_stream() {
   HCTR_HIP(e);
 }
 
+namespace {
+void wait_for(hipStream_t s) {
+  hipError_t e;
+  while ((e = hipStreamQuery(s)) == hipErrorNotReady) {
+  }
+  HCTR_HIP(e);
+}
+} // namespace
+
+// Enqueues the index stages of the ingested batch (single shard) on the stream the stages currently use.
+static void enqueue_index(Shard *m) {
+  m->index_batch();
+  m->preprocess_gradient();
+  m->enqueue_readback_preprocess();
+}
+
+void Group::flush_index() {
+  if (!index_pending) return;
+  index_pending = false;
+  HCTR_HIP(hipSetDevice(device_id));
+  wait_for(index_stream);
+  members[0]->finish_preprocess();
+  exchange_shapes();
+}
+
 void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
+  flush_index(); // preprocess twice in a row: the earlier batch is indexed before it becomes the previous one
+  if (defer_index && !stage_timing) {
+    // One shard: everything is enqueued on the second stream, and the call returns as soon as the caller's ids have
+    // been read.  Sorting and deduplicating them does not depend on the pending gradient push, which the next
+    // push_pull puts on the main stream while this is still running; the gather waits for both.
+    Shard *m = members[0];
+    StreamSwitch on(*this, index_stream);
+    HCTR_HIP(hipEventRecord(ev0, stream));
+    m->swap_batches();
+    m->ingest_keys(keys[0], n[0]);
+    HCTR_HIP(hipMemcpyAsync(&m->mirror->st.err, m->err_ptr(), 4, hipMemcpyDeviceToHost, stream));
+    HCTR_HIP(hipEventRecord(ev1, stream));
+    HCTR_HIP(hipEventRecord(ev_keys, stream));
+    enqueue_index(m);
+    HCTR_HIP(hipEventRecord(ev_index, stream));
+    index_pending = true;
+    hipError_t e;
+    while ((e = hipEventQuery(ev_keys)) == hipErrorNotReady) {
+    }
+    HCTR_HIP(e);
+    float ms = 0.f;
+    HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+    m->last_pre_ms = ms;
+    if (m->mirror->st.err) {
+      wait_for(index_stream); // the later read-back of the same flag must land before the flag is cleared
+      m->check_key_error();
+    }
+    return;
+  }
   HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) {
     m->swap_batches();
@@ -735,13 +810,17 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
       if (first_error.empty()) first_error = e.what();
     }
   }
-  // all2allExchangeShape, csrc/core/all2all.cu:6-16
+  exchange_shapes();
+  if (!first_error.empty()) throw Error(first_error);
+}
+
+// all2allExchangeShape, csrc/core/all2all.cu:6-16
+void Group::exchange_shapes() {
   for (Shard *m : members)
     for (int s = 0; s < nrank; s++) {
       m->cur.recv_cnt[s] = members[s]->cur.send_cnt[m->cfg.rank];
       m->prev.pushrecv_cnt[s] = members[s]->prev.push_cnt[m->cfg.rank];
     }
-  if (!first_error.empty()) throw Error(first_error);
 }
 
 // csrc/core/hetu_gpu_table.cu:9-41 for every shard of the group
@@ -752,6 +831,13 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
   for (Shard *m : members) {
     m->generate_gradient(grads[m->cfg.rank]);
     m->generate_query();
+  }
+  const bool join_index = index_pending;
+  if (join_index) {
+    // the push kernel is in the main stream's queue; the gather below also needs the index of the current batch,
+    // still running or done on the second stream
+    index_pending = false;
+    HCTR_HIP(hipStreamWaitEvent(stream, ev_index, 0));
   }
   if (nrank > 1) {
     exchange_query();
@@ -768,6 +854,10 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
   float ms = 0.f;
   HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
   collect_marks();
+  if (join_index) {
+    members[0]->finish_preprocess();
+    exchange_shapes();
+  }
   for (Shard *m : members) {
     m->last_pp_ms = ms;
     m->finish_push_pull();
