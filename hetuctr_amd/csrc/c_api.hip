@@ -162,6 +162,13 @@ int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms) {
   });
 }
 
+int hctr_last_push_ms(hctr_table *t, float *push_ms) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard && push_ms, "null argument");
+    *push_ms = t->shard->last_push_ms;
+  });
+}
+
 int hctr_stage_timing(hctr_table *t, int on) {
   return guarded([&] {
     HCTR_CHECK(t && t->shard, "null table");

@@ -138,7 +138,7 @@ class Shard {
   uint64_t in_rows = 0;
   HostMirror *mirror = nullptr;
   long long last_stats[6] = {0, 0, 0, 0, 0, 0};
-  float last_pre_ms = 0.f, last_pp_ms = 0.f;
+  float last_pre_ms = 0.f, last_pp_ms = 0.f, last_push_ms = 0.f;
   bool plan_cleared = false; // the device-side push counts read as zero
   bool u_cleared = false;    // the device-side copy of the number of unique keys reads as zero
 
@@ -162,7 +162,7 @@ class Group {
   // sorting and deduplicating them has no dependence on the pending gradient push, so the next push_pull starts the
   // push on the main stream right away and only the gather waits for both.
   hipStream_t index_stream = nullptr;
-  hipEvent_t ev_index = nullptr, ev_keys = nullptr;
+  hipEvent_t ev_index = nullptr, ev_keys = nullptr, ev_push = nullptr;
   bool defer_index = false;              // the mode is on (one shard, HETUCTR_DEFER_INDEX != 0)
   bool index_pending = false;            // a batch's index is enqueued and nobody has waited for it yet
   void flush_index();                    // waits for a pending index and takes its results over

@@ -561,6 +561,7 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   HCTR_HIP(hipStreamCreate(&index_stream));
   HCTR_HIP(hipEventCreateWithFlags(&ev_index, hipEventDisableTiming));
   HCTR_HIP(hipEventCreateWithFlags(&ev_keys, hipEventDisableTiming));
+  HCTR_HIP(hipEventCreate(&ev_push));
   const char *defer = getenv("HETUCTR_DEFER_INDEX");
   defer_index = nr == 1 && !(defer && atoi(defer) == 0);
   HCTR_HIP(hipEventCreate(&ev0));
@@ -582,6 +583,7 @@ Group::~Group() {
   if (index_stream) (void)hipStreamDestroy(index_stream);
   if (ev_index) (void)hipEventDestroy(ev_index);
   if (ev_keys) (void)hipEventDestroy(ev_keys);
+  if (ev_push) (void)hipEventDestroy(ev_push);
 }
 
 void Group::join(Shard *s) {
@@ -832,6 +834,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
     m->generate_gradient(grads[m->cfg.rank]);
     m->generate_query();
   }
+  HCTR_HIP(hipEventRecord(ev_push, stream));
   const bool join_index = index_pending;
   if (join_index) {
     // the push kernel is in the main stream's queue; the gather below also needs the index of the current batch,
@@ -858,8 +861,11 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
     members[0]->finish_preprocess();
     exchange_shapes();
   }
+  float push_ms = 0.f;
+  HCTR_HIP(hipEventElapsedTime(&push_ms, ev0, ev_push));
   for (Shard *m : members) {
     m->last_pp_ms = ms;
+    m->last_push_ms = push_ms;
     m->finish_push_pull();
   }
 }

@@ -102,6 +102,16 @@ int hctr_stream(hctr_table *t, void **stream_out);
  * that stream around the launched work (host-side waits excluded). */
 int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
 
+/* With one shard, hctr_preprocess returns as soon as the caller's ids have been read (the buffer may be reused): the
+ * sort / unique stages of that batch keep running on a second stream, next to the gradient push that the following
+ * hctr_push_pull starts, and are waited for before the rows are gathered.  preprocess_ms above is then the time up to
+ * that return, push_pull_ms covers the rest.  Anything that needs the batch's index earlier (a second hctr_preprocess,
+ * hctr_debug_fetch, hctr_stage_timing) waits for it.  HETUCTR_DEFER_INDEX=0 in the environment restores a
+ * preprocess that returns only when all its work is done (hetu_gpu_table.cu:64); with stage timing on it always is.
+ * hctr_last_push_ms: device time from the start of the last hctr_push_pull to the end of its push stage, i.e. the
+ * push kernel while the index of the next batch runs beside it.  No counterpart in the reference. */
+int hctr_last_push_ms(hctr_table *t, float *push_ms);
+
 /* Per-stage device time.  hctr_stage_timing(t, 1) resets the accumulators and makes every later call bracket
  * each stage's launches with HIP events on the table's stream; hctr_stage_times returns, per stage, the
  * accumulated milliseconds and the number of bracketed intervals.  Stage i is named hctr_stage_name(i),

@@ -216,3 +216,110 @@ def test_constructor_errors_and_strings():
     assert repr(t) == "<HetuTable root/store/all=8/8/8>"       # csrc/core/debug.cu:5-12
     assert t.debug() == "<HetuTable root/store/all=8/8/8 rank=0 nrank=1 device_id=0 width=4 push/pull=5/3>"
     t.close()
+
+
+def test_key_buffer_is_free_when_preprocess_returns():
+    # preprocess returns before the batch is sorted; the caller may overwrite its id buffer at once, whether it
+    # lives on the device or on the host, and every step still matches the oracle
+    import torch
+    say("ids overwritten right after preprocess")
+    rng = np.random.default_rng(31)
+    length, width, n = 40_000, 32, 30_000
+    p = single(length, width, lr=0.05)
+    t, o = p.tables[0], p.oracle
+    dev = torch.empty(n, dtype=torch.int64, device="cuda")
+    host = np.empty(n, np.int64)
+    dst = torch.empty((n, width), device="cuda")
+    prev = 0
+    for step in range(8):
+        keys = rng.integers(0, length, size=n).astype(np.int64)
+        if step % 2:
+            dev.copy_(torch.from_numpy(keys))
+            torch.cuda.synchronize()
+            t.preprocess(dev.data_ptr(), n)
+            dev.fill_(-1)                                 # next work on the default stream: ordered after ours
+        else:
+            host[:] = keys
+            t.preprocess(host.ctypes.data, n)
+            host[:] = -1
+        g = rng.normal(0, 1e-3, size=(prev, width)).astype(np.float32)
+        dg = torch.from_numpy(g).cuda()
+        torch.cuda.synchronize()
+        t.push_pull(dg.data_ptr() if prev else 0, dst.data_ptr())
+        o.preprocess([keys])
+        ref = o.push_pull([g if prev else None])[0]
+        assert np.array_equal(dst.cpu().numpy(), ref), "step %d" % step
+        for item in (capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.KEYS):
+            assert np.array_equal(t.fetch(item), o.fetch(0, item)), (step, item)
+        prev = n
+    p.close()
+
+
+def test_repeated_and_changing_batch_sizes():
+    # many steps of one batch size, then size changes, an empty batch, a doubled preprocess and state fetches between
+    # preprocess and push_pull (each of which has to wait for the index still running on the second stream)
+    say("repeated and changing batch sizes")
+    rng = np.random.default_rng(32)
+    length, width = 60_000, 16
+    p = single(length, width, lr=0.1)
+    sizes = [20_000] * 7 + [5_000, 20_000, 20_000, 0, 20_000, 20_000, 45_000, 45_000, 45_000, 45_000, 20_000, 20_000]
+    prev_n = 0
+    for step, n in enumerate(sizes):
+        keys = rng.integers(0, length, size=n).astype(np.int64)
+        if step == 12:                                     # preprocess twice in a row: the first batch becomes "previous"
+            extra = rng.integers(0, length, size=20_000).astype(np.int64)
+            p.preprocess([extra], device_keys=True)
+            prev_n = 20_000
+        p.preprocess([keys], device_keys=(step % 3 != 0))
+        if step % 4 == 1:
+            p.compare_ints(INT_ITEMS_PRE, "step %d before push_pull" % step)
+        g = rng.normal(0, 1e-3, size=(prev_n, width)).astype(np.float32)
+        out, ref = p.push_pull([g])
+        assert_close(out[0], ref[0], 1e-5, "dst step %d" % step)
+        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.SIZES, capi.VERSION], "step %d" % step)
+        prev_n = n
+    p.compare_state(1e-5, "end")
+    p.close()
+
+
+def test_key_error_is_raised_by_preprocess_and_the_table_goes_on():
+    say("bad key, early return")
+    length, width, n = 1000, 8, 500
+    p = single(length, width)
+    t = p.tables[0]
+    rng = np.random.default_rng(33)
+    good = rng.integers(0, length, size=n).astype(np.int64)
+    bad = good.copy()
+    bad[17] = length + 5
+    p.preprocess([good])
+    p.push_pull([np.zeros((0, width), np.float32)])
+    with pytest.raises(RuntimeError, match="outside"):
+        t.preprocess(bad.ctypes.data, n)
+    import torch
+    dst = torch.empty((n, width), device="cuda")
+    t.push_pull(0, dst.data_ptr())                         # the batch is usable (the key counted as id 0)
+    for _ in range(3):                                     # and the flag does not come back
+        t.preprocess(good.ctypes.data, n)
+        t.push_pull(0, dst.data_ptr())
+    ref = p.oracle.fetch(0, capi.EMBEDDING).reshape(length, width)[good]
+    assert np.array_equal(dst.cpu().numpy(), ref)
+    p.close()
+
+
+def test_preprocess_that_waits_for_all_its_work(monkeypatch):
+    # HETUCTR_DEFER_INDEX=0: the reference's call protocol literally (preprocess returns when the batch is indexed)
+    say("synchronous preprocess")
+    monkeypatch.setenv("HETUCTR_DEFER_INDEX", "0")
+    rng = np.random.default_rng(34)
+    length, width, n = 30_000, 64, 25_000
+    p = single(length, width, lr=0.05)
+    prev_n = 0
+    for step in range(5):
+        keys = rng.integers(0, length, size=n).astype(np.int64)
+        p.preprocess([keys], device_keys=True)
+        g = rng.normal(0, 1e-3, size=(prev_n, width)).astype(np.float32)
+        out, ref = p.push_pull([g])
+        assert_close(out[0], ref[0], 1e-5, "dst step %d" % step)
+        prev_n = n
+    p.compare_ints([capi.VERSION])
+    p.close()
