@@ -41,7 +41,7 @@ namespace hctr {
 #define HCTR_SLICE 64
 #endif
 #ifndef HCTR_LONG_BLOCKS
-#define HCTR_LONG_BLOCKS 192
+#define HCTR_LONG_BLOCKS 128
 #endif
 #ifndef HCTR_MED_BLOCKS
 #define HCTR_MED_BLOCKS 512
