@@ -269,3 +269,16 @@ def test_cache_list_rule_of_the_oracle():
         idx = np.where(owner == i)[0]
         q[idx] = -1
         assert np.array_equal(lists[i], np.argsort(q)[len(idx):][::-1])
+
+
+def test_importable_under_the_reference_module_name():
+    import hetuctr_amd
+    mod = hetuctr_amd.install_as_hetuCTR_partition()
+    import hetuCTR_partition
+    assert hetuCTR_partition is mod
+    rng = np.random.default_rng(2)
+    p = hetuCTR_partition.partition(slot_data(rng, 200, 3, 20, 1.3), np.ones((2, 2), np.float32), 2, 8)
+    for name in ("refine_data", "refine_embed", "get_communication", "get_priority", "get_result", "get_data_cnt",
+                 "get_embed_cnt"):                      # csrc/partition/pybind.cc:9-21
+        assert callable(getattr(p, name))
+    assert type(p).__name__ == "_PartitionStruct"
