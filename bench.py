@@ -148,6 +148,11 @@ def main_partition(a):
     lists_s = time.perf_counter() - t0
     list_bytes = workloads.cache_list_bytes(p.n_embed, P, keep)
     gbs = list_bytes / (kernel_ms * 1e-3) / 1e9
+    # measured HBM bytes of the same kernels at the default size (rocprofv3 --pmc runs summarised under profiles/)
+    measured = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath) and a.scale == 1.0 and a.part_samples == 1_000_000 and a.part_cache_frac == 0.10:
+        measured = json.load(open(tpath)).get("partition", {}).get("cache_lists")
     out = {
         "metric": "partitioner: samples refined per second (one round = sample sweep + embedding sweep + cost)",
         "value": nd * a.part_rounds / refine_s, "unit": "samples/s", "n_gpus": 1, "steps": a.part_rounds, "warmup": 0,
@@ -159,7 +164,7 @@ def main_partition(a):
         "construction_s": create_s, "rounds": rounds, "cost_initial": cost0, "cost_after_round": costs,
         "cache_lists": {"kept_per_part": keep, "wall_s_with_upload_and_download": lists_s, "kernel_ms": kernel_ms},
         "roofline": {"bound": "hbm", "kernel": "priority keys + %d radix sorts + list emit" % P, "achieved": gbs,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": measured,
                      "algorithmic_bytes": int(list_bytes)},
     }
     p.close()
