@@ -34,9 +34,6 @@ namespace hctr {
 #ifndef HCTR_RPT
 #define HCTR_RPT 2
 #endif
-#ifndef HCTR_SUM_PRIO
-#define HCTR_SUM_PRIO 0
-#endif
 #ifndef HCTR_SLICE
 #define HCTR_SLICE 64
 #endif
@@ -45,9 +42,6 @@ namespace hctr {
 #endif
 #ifndef HCTR_MED_BLOCKS
 #define HCTR_MED_BLOCKS 512
-#endif
-#ifndef HCTR_ONLY_ROLE
-#define HCTR_ONLY_ROLE 0 // 1: long, 2: short, 3: medium role only (timing experiments; results are incomplete)
 #endif
 constexpr int kPushBlock = 512;
 
@@ -504,9 +498,6 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
         if (g0 + k < G) step(k); // uniform over the block: the summing wave makes the same number of barriers
     } else {
       // ---------------- summing wave: one column per lane, rows strictly in order ----------------
-#if HCTR_SUM_PRIO
-      __builtin_amdgcn_s_setprio(HCTR_SUM_PRIO); // the chain of this wave is the critical path of the whole push
-#endif
       // the column this lane sums: lane = place in the fast path's layout
       const uint32_t mycol = slice * CS + (CSC ? (threadIdx.x % (CSC ? CSC / 4 : 1)) * 4 + threadIdx.x / (CSC ? CSC / 4 : 1) : threadIdx.x);
       const bool col_ok = threadIdx.x < CS && mycol < W;
@@ -618,7 +609,6 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
   __shared__ uint4 run_table[kTable];
   __shared__ uint32_t run_totals[3];
   if (blockIdx.x < kLongBlocks) {
-    if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 1) return;
     // Every block first takes tickets of the longest runs, which are cut into narrower column slices so that more
     // blocks feed each of them (the blocks of a saturated memory system get equal shares of it, and a chain
     // advances with the share of the block that feeds it), then tickets of the other long runs.
@@ -632,14 +622,12 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
       long_role<VEC, K, 0>(t, id_bits, p, a, lds, run_table, run_totals, 0, kLongBuckets, blockIdx.x, kLongBlocks, tk);
     }
   } else if (blockIdx.x < kLongBlocks + kMedBlocks) { // medium runs take long per block: they start early
-    if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 3) return;
     medium_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, (uint32_t *)lds, blockIdx.x - kLongBlocks, kMedBlocks);
   } else {
     constexpr int kGroups = kPushBlock / LPR;
     const uint32_t short_blocks = div_up_dev(U, kGroups * kRunsPerGroup);
     const uint32_t b = blockIdx.x - kLongBlocks - kMedBlocks;
     if (b < short_blocks) {
-      if (HCTR_ONLY_ROLE != 0 && HCTR_ONLY_ROLE != 2) return;
       short_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, b, U);
     } else if (kSingle) {
       // Single shard: every key is owned, so the only counter is the row version, which grows by the number of

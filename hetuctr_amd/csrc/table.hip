@@ -595,7 +595,10 @@ void Group::join(Shard *s) {
 void Group::leave(Shard *s) {
   std::lock_guard<std::mutex> lk(mu_);
   if (members[s->cfg.rank] == s) members[s->cfg.rank] = nullptr;
-  index_pending = false;
+  if (index_pending) { // the shard's buffers are about to be freed: nothing of it may still be running
+    index_pending = false;
+    (void)hipStreamSynchronize(index_stream);
+  }
 }
 
 bool Group::complete() const {

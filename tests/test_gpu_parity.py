@@ -323,3 +323,23 @@ def test_preprocess_that_waits_for_all_its_work(monkeypatch):
         prev_n = n
     p.compare_ints([capi.VERSION])
     p.close()
+
+
+def test_table_closed_while_the_index_is_still_running():
+    # preprocess returns early; destroying the table right away must wait for what it left on the GPU
+    say("close right after preprocess")
+    import torch
+    rng = np.random.default_rng(35)
+    length, width, n = 200_000, 32, 150_000
+    for _ in range(3):
+        p = single(length, width)
+        keys = torch.from_numpy(rng.integers(0, length, size=n).astype(np.int64)).cuda()
+        torch.cuda.synchronize()
+        p.tables[0].preprocess(keys.data_ptr(), n)
+        p.close()
+    p = single(length, width)                      # and a fresh table works afterwards
+    k = rng.integers(0, length, size=n).astype(np.int64)
+    p.preprocess([k])
+    out, ref = p.push_pull([np.zeros((0, width), np.float32)])
+    assert np.array_equal(out[0], ref[0])
+    p.close()
