@@ -20,6 +20,9 @@ struct SortScratch {
 };
 
 inline size_t sort_blocks(size_t n) { return (n + kSortTile - 1) / kSortTile; }
+// a sort of at most this many tiles launches no scan kernel: every block of the scatter sums the raw per-block counts
+// of its bins itself (the sum over so few blocks costs less than a launch)
+constexpr uint32_t kSmallSortBlocks = 16;
 // tiles of the scan / unique kernels of the preprocess (256 threads x 8 items), whatever the sort tile is
 inline size_t scan_blocks(size_t n) { return (n + 2047) / 2048; }
 

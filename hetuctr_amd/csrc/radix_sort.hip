@@ -74,7 +74,9 @@ __global__ __launch_bounds__(kSortBlock) void scan_bins(uint32_t *__restrict__ g
   if (threadIdx.x == 0) bintot[blockIdx.x] = total;
 }
 
-template <typename K, bool kFirst>
+// kSmall: ghist holds the raw counts of a sort of few tiles (no scan kernel ran, bintot is unused): the block sums
+// its bins over the blocks itself, which is cheaper than a launch when the blocks are few.
+template <typename K, bool kFirst, bool kSmall = false>
 __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
                                                       K *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
                                                       uint32_t n, int shift, int dbits,
@@ -93,7 +95,27 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
   const uint32_t blo = min(threadIdx.x * per, nb), bhi = min(blo + per, nb);
 
   // global base of each bin for this block: sum of the totals of lower bins + this bin's lower blocks
-  {
+  if (kSmall) {
+    uint32_t s = 0;
+    for (uint32_t i = blo; i < bhi; i++) {
+      const uint32_t *row = ghist + (size_t)i * nblocks;
+      uint32_t lower = 0, all = 0;
+      for (uint32_t j = 0; j < nblocks; j++) {
+        const uint32_t v = row[j];
+        lower += j < blockIdx.x ? v : 0u;
+        all += v;
+      }
+      base[i] = lower;      // completed below
+      bin_start[i] = all;   // the bin's total, parked here until the scan is through
+      s += all;
+    }
+    uint32_t total;
+    uint32_t off = block_exclusive_scan<kSortBlock>(s, sm, total);
+    for (uint32_t i = blo; i < bhi; i++) {
+      base[i] += off;
+      off += bin_start[i];
+    }
+  } else {
     uint32_t s = 0;
     for (uint32_t i = blo; i < bhi; i++) s += bintot[i];
     uint32_t total;
@@ -209,6 +231,7 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
   const uint32_t *vin = nullptr;
   K *ktmp[2] = {tmp_k0, tmp_k1};
   uint32_t *vtmp[2] = {tmp_v0, tmp_v1};
+  const bool small = nblocks <= kSmallSortBlocks;
   for (int p = 0; p < passes; p++) {
     const int left = bits - shift;
     const int dbits = (left + (passes - p) - 1) / (passes - p);
@@ -223,13 +246,22 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
         hipLaunchKernelGGL((digit_histogram<K, false>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, n, shift,
                            dbits, scratch.ghist, nblocks);
     }
-    hipLaunchKernelGGL(scan_bins, dim3(nb), dim3(kSortBlock), 0, stream, scratch.ghist, nblocks, scratch.bintot);
-    if (p == 0)
-      hipLaunchKernelGGL((scatter<K, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
-                         shift, dbits, scratch.ghist, nblocks, scratch.bintot);
-    else
-      hipLaunchKernelGGL((scatter<K, false>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
-                         shift, dbits, scratch.ghist, nblocks, scratch.bintot);
+    if (small) { // few tiles: the blocks of the scatter scan the raw counts themselves
+      if (p == 0)
+        hipLaunchKernelGGL((scatter<K, true, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
+                           shift, dbits, scratch.ghist, nblocks, scratch.bintot);
+      else
+        hipLaunchKernelGGL((scatter<K, false, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout,
+                           n, shift, dbits, scratch.ghist, nblocks, scratch.bintot);
+    } else {
+      hipLaunchKernelGGL(scan_bins, dim3(nb), dim3(kSortBlock), 0, stream, scratch.ghist, nblocks, scratch.bintot);
+      if (p == 0)
+        hipLaunchKernelGGL((scatter<K, true>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
+                           shift, dbits, scratch.ghist, nblocks, scratch.bintot);
+      else
+        hipLaunchKernelGGL((scatter<K, false>), dim3(nblocks), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
+                           shift, dbits, scratch.ghist, nblocks, scratch.bintot);
+    }
     HCTR_HIP(hipGetLastError());
     kin = kout;
     vin = vout;
