@@ -16,28 +16,33 @@ constexpr int kTile = kBlock * kItems; // 2048: scan_blocks(n) sizes the scratch
 // ids -> sort keys (owner << id_bits | id), the copy of the ids, the range check, the reset of the batch's run
 // counters, and the per-block counts of the first sort pass' digit: a block works on one sort tile, so the sort
 // needs no histogram launch of its own for that pass.
+// one sort tile per block, with more threads than the sort's own blocks: twice the loads in flight per tile
+#ifndef HCTR_KEY_BLOCK
+#define HCTR_KEY_BLOCK 512
+#endif
+constexpr int kKeyBlock = HCTR_KEY_BLOCK, kKeyItems = kSortTile / kKeyBlock;
 template <typename K>
-__global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
+__global__ __launch_bounds__(kKeyBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
                                                         int id_bits, int nrank, const worker_t *__restrict__ root,
                                                         K *__restrict__ comp, uint32_t *__restrict__ err,
                                                         index_t *__restrict__ keys_copy, uint32_t *__restrict__ nlong,
                                                         int dbits, uint32_t *__restrict__ ghist, uint32_t nblocks) {
   __shared__ uint32_t h[1 << kSortMaxDigitBits];
   const uint32_t nb = 1u << dbits, mask = nb - 1;
-  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
+  for (uint32_t i = threadIdx.x; i < nb; i += kKeyBlock) h[i] = 0;
   if (blockIdx.x == 0 && threadIdx.x < kRunCounters && nlong) nlong[threadIdx.x] = 0; // counters of this batch
   __syncthreads();
   const uint32_t base = blockIdx.x * kSortTile;
-  uint64_t id[kSortItems];
+  uint64_t id[kKeyItems];
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
-    const uint32_t i = base + k * kSortBlock + threadIdx.x;
+  for (int k = 0; k < kKeyItems; k++) {
+    const uint32_t i = base + k * kKeyBlock + threadIdx.x;
     id[k] = i < n ? (uint64_t)keys[i] : 0;
   }
   bool bad = false;
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
-    const uint32_t i = base + k * kSortBlock + threadIdx.x;
+  for (int k = 0; k < kKeyItems; k++) {
+    const uint32_t i = base + k * kKeyBlock + threadIdx.x;
     if (i >= n) continue;
     if (keys_copy) keys_copy[i] = (index_t)id[k];
     if (id[k] >= id_max) { // also catches negative ids
@@ -46,19 +51,19 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
     }
   }
   if (bad) atomicOr(err, 1u);
-  uint64_t owner[kSortItems];
+  uint64_t owner[kKeyItems];
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) owner[k] = nrank > 1 ? root[id[k]] : 0;
+  for (int k = 0; k < kKeyItems; k++) owner[k] = nrank > 1 ? root[id[k]] : 0;
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
-    const uint32_t i = base + k * kSortBlock + threadIdx.x;
+  for (int k = 0; k < kKeyItems; k++) {
+    const uint32_t i = base + k * kKeyBlock + threadIdx.x;
     if (i >= n) continue;
     const K c = (K)((owner[k] << id_bits) | id[k]);
     comp[i] = c;
     atomicAdd(&h[(uint32_t)c & mask], 1u);
   }
   __syncthreads();
-  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) ghist[(size_t)i * nblocks + blockIdx.x] = h[i];
+  for (uint32_t i = threadIdx.x; i < nb; i += kKeyBlock) ghist[(size_t)i * nblocks + blockIdx.x] = h[i];
 }
 
 // Sorted position j of a block's tile is handled by thread (j % kBlock) in round (j / kBlock): every load
@@ -272,10 +277,10 @@ void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, co
   const unsigned nblocks = (unsigned)sort_blocks(n);
   const int dbits = sort_first_digit_bits(kl.total_bits);
   if (kl.wide)
-    hipLaunchKernelGGL(make_keys<uint64_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
+    hipLaunchKernelGGL(make_keys<uint64_t>, dim3(nblocks), dim3(kKeyBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
                        t.root, (uint64_t *)comp_keys, err, keys_copy, nlong, dbits, ghist, nblocks);
   else
-    hipLaunchKernelGGL(make_keys<uint32_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
+    hipLaunchKernelGGL(make_keys<uint32_t>, dim3(nblocks), dim3(kKeyBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
                        t.root, (uint32_t *)comp_keys, err, keys_copy, nlong, dbits, ghist, nblocks);
   HCTR_HIP(hipGetLastError());
 }
