@@ -44,10 +44,15 @@ private:
   int f_, r_;
 };
 
-// runs fn(t, nthreads) on up to `want` host threads
+// host threads a parallel step gets when it asks for `want`: at most 16 and at most what the machine has
+size_t thread_count(size_t want) {
+  const size_t hw = std::thread::hardware_concurrency();
+  return std::max<size_t>(1, std::min<size_t>({want, hw ? hw : 1, 16}));
+}
+
+// runs fn(t, nthreads) on thread_count(want) host threads
 template <typename F> void on_threads(size_t want, F &&fn) {
-  size_t hw = std::thread::hardware_concurrency();
-  const size_t nt = std::max<size_t>(1, std::min<size_t>({want, hw ? hw : 1, 16}));
+  const size_t nt = thread_count(want);
   std::vector<std::thread> pool;
   for (size_t t = 1; t < nt; t++) pool.emplace_back([&fn, t, nt] { fn(t, nt); });
   fn(0, nt);
@@ -190,14 +195,8 @@ void Partitioner::refine_data() {
 // by threads over ranges of j that keep the nonzero terms per (p, i); a chain then adds its terms range after range.
 std::vector<float> Partitioner::embed_weight_now() const {
   const int P = n_part;
-  size_t nt_used = 1;
-  std::vector<std::vector<std::vector<float>>> terms; // [thread][p * P + i]
-  on_threads(16, [&](size_t t, size_t nt) {
-    if (t == 0) {
-      nt_used = nt;
-      terms.assign(nt, std::vector<std::vector<float>>((size_t)P * P));
-    }
-  });
+  const size_t nt_used = thread_count(16);
+  std::vector<std::vector<std::vector<float>>> terms(nt_used, std::vector<std::vector<float>>((size_t)P * P)); // [thread][p * P + i]
   on_threads(nt_used, [&](size_t t, size_t nt) {
     auto &mine = terms[t];
     const size_t lo = n_embed * t / nt, hi = n_embed * (t + 1) / nt;
