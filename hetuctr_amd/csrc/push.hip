@@ -633,7 +633,13 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
       // Single shard: every key is owned, so the only counter is the row version, which grows by the number of
       // duplicates (generate_query.cu:68-69).  One thread per unique key, in the last blocks of the grid.
       const uint32_t u = (b - short_blocks) * kPushBlock + threadIdx.x;
-      if (u < U) t.ver[p.uoff[u]] += (version_t)(p.run_start[u + 1] - p.run_start[u]);
+      // nontemporal: a counter line is touched once per step; left in the cache it is written back in the middle of
+      // the gather that follows
+      if (u < U) {
+        version_t *vp = &t.ver[p.uoff[u]];
+        const version_t v = __builtin_nontemporal_load(vp) + (version_t)(p.run_start[u + 1] - p.run_start[u]);
+        __builtin_nontemporal_store(v, vp);
+      }
     }
   }
 }
