@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, Pull
 #define HCTR_GATHER_ROWS 8
 #endif
 #ifndef HCTR_GATHER_NT
-#define HCTR_GATHER_NT 0
+#define HCTR_GATHER_NT 1
 #endif
 constexpr int kRows = HCTR_GATHER_ROWS;
 template <int VEC, int LPR, bool kLocalOnly>

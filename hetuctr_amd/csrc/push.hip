@@ -69,6 +69,26 @@ namespace {
 
 __device__ __forceinline__ uint32_t div_up_dev(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
+#ifndef HCTR_GRAD_NT
+#define HCTR_GRAD_NT 1
+#endif
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// a gradient row is read exactly once per step
+__device__ __forceinline__ float4 grad_load(const float4 *p) {
+#if HCTR_GRAD_NT
+  const f32x4 r = __builtin_nontemporal_load((const f32x4 *)p);
+  return make_float4(r.x, r.y, r.z, r.w);
+#else
+  return *p;
+#endif
+}
+__device__ __forceinline__ float grad_load(const float *p) {
+#if HCTR_GRAD_NT
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
 template <int VEC> struct Vec;
 template <> struct Vec<4> {
   typedef float4 T;
@@ -201,7 +221,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
       for (int k = 0; k < kHead; k++) {
         v[i][k] = Vec<VEC>::zero();
-        if (mine[i] && (uint32_t)k < len[i]) v[i][k] = *(const V *)(grad + (size_t)si[i][k] * W + col);
+        if (mine[i] && (uint32_t)k < len[i]) v[i][k] = grad_load((const V *)(grad + (size_t)si[i][k] * W + col));
       }
     V acc[G];
 #pragma unroll
@@ -221,7 +241,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
         for (int k = 0; k < kTail; k++) sj[k] = sorted_arg[min(j + k, rs[i + 1] - 1)];
 #pragma unroll
-        for (int k = 0; k < kTail; k++) x[k] = *(const V *)(grad + (size_t)sj[k] * W + col);
+        for (int k = 0; k < kTail; k++) x[k] = grad_load((const V *)(grad + (size_t)sj[k] * W + col));
 #pragma unroll
         for (int k = 0; k < kTail; k++)
           if (j + k < rs[i + 1]) Vec<VEC>::add(acc[i], x[k]);
@@ -276,7 +296,7 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
       V xa[kBatch], xb[kBatch];
       auto fetch = [&](V(&x)[kBatch], uint32_t q0) { // rows q0 .. q0+kBatch-1 of the run (clamped to its end)
 #pragma unroll
-        for (int k = 0; k < kBatch; k++) x[k] = *(const V *)(gcol + (size_t)my_idx[min(q0 + k, len - 1)] * W);
+        for (int k = 0; k < kBatch; k++) x[k] = grad_load((const V *)(gcol + (size_t)my_idx[min(q0 + k, len - 1)] * W));
       };
       auto add = [&](const V(&x)[kBatch], uint32_t q0) {
 #pragma unroll
@@ -436,7 +456,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       // Loads are unconditional and branch-free so that kDepth chunks stay in flight per thread: positions
       // past the end of a run re-read its last row (never summed), lanes outside the slice read column 0.
       const embed_t *gbase = a.grad + ((in_slice && col < W) ? col : 0);
-      auto row_load = [&](uint32_t idx) -> V { return *(const V *)(gbase + (size_t)idx * W); };
+      auto row_load = [&](uint32_t idx) -> V { return grad_load((const V *)(gbase + (size_t)idx * W)); };
       // cursor of the index stage, 2 * kDepth chunks ahead of the LDS stage; past the end of the stream it
       // stays on the last run
       uint32_t cj = 0, cc = 0;
