@@ -44,6 +44,9 @@ inline unsigned div_up(size_t a, size_t b) { return (unsigned)((a + b - 1) / b);
 constexpr int kWave = 64;
 
 // ---- device helpers ---------------------------------------------------------------------------
+// a load of data that nothing reads again soon: it should not push other lines out of the caches
+template <typename T> __device__ __forceinline__ T load_once(const T *p) { return __builtin_nontemporal_load(p); }
+
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 
 // inclusive scan over the 64 lanes of a wave

@@ -37,14 +37,14 @@ __global__ __launch_bounds__(kKeyBlock) void make_keys(const index_t *__restrict
 #pragma unroll
   for (int k = 0; k < kKeyItems; k++) {
     const uint32_t i = base + k * kKeyBlock + threadIdx.x;
-    id[k] = i < n ? (uint64_t)keys[i] : 0;
+    id[k] = i < n ? (uint64_t)load_once(&keys[i]) : 0; // the caller's ids are read here and nowhere else
   }
   bool bad = false;
 #pragma unroll
   for (int k = 0; k < kKeyItems; k++) {
     const uint32_t i = base + k * kKeyBlock + threadIdx.x;
     if (i >= n) continue;
-    if (keys_copy) keys_copy[i] = (index_t)id[k];
+    if (keys_copy) __builtin_nontemporal_store((index_t)id[k], &keys_copy[i]); // only read back on request
     if (id[k] >= id_max) { // also catches negative ids
       bad = true;
       id[k] = 0;

@@ -138,8 +138,9 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
   for (int r = 0; r < kRounds; r++) {
     const uint32_t idx = wbase + r * kWave + lane;
     const bool valid = idx < n;
-    key[r] = valid ? keys_in[idx] : (K)0;
-    val[r] = kFirst ? idx : (valid ? vals_in[idx] : 0u);
+    // a pass reads its input once
+    key[r] = valid ? load_once(&keys_in[idx]) : (K)0;
+    val[r] = kFirst ? idx : (valid ? load_once(&vals_in[idx]) : 0u);
   }
 #pragma unroll
   for (int r = 0; r < kRounds; r++) {
