@@ -77,6 +77,7 @@ struct HostMirror {
   uint32_t ret_total;
   uint32_t stats[4];
   uint32_t ret_seg[258];
+  uint32_t key_err; // written by the kernel that reads the caller's ids when preprocess returns early (no copy)
 };
 
 class Group;
@@ -104,7 +105,8 @@ class Shard {
     ingest_keys(keys, n);
     index_batch();
   }
-  void ingest_keys(const int64_t *keys, size_t n); // the caller's ids -> device copy and sort keys
+  // the caller's ids -> device copy and sort keys; flag: where the range check reports (default: the device word)
+  void ingest_keys(const int64_t *keys, size_t n, uint32_t *flag = nullptr);
   void index_batch();                              // sort, unique, run lists of the ingested batch
   void preprocess_gradient();
   void enqueue_readback_preprocess();

@@ -197,7 +197,7 @@ void Shard::reserve_batch_scratch(uint32_t n) {
 }
 
 // csrc/core/preprocess.cu:92-141
-void Shard::ingest_keys(const int64_t *keys, size_t n) {
+void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag) {
   HCTR_CHECK(n < 0xfffffff0ull, "a batch holds fewer than 2^32 keys");
   HCTR_CHECK(keys != nullptr || n == 0, "null key pointer");
   hipStream_t s = group->stream;
@@ -222,7 +222,7 @@ void Shard::ingest_keys(const int64_t *keys, size_t n) {
         (void)hipGetLastError(); // an unregistered host pointer leaves a sticky "invalid value"
         HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
       }
-      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, comp.p, err_ptr(),
+      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, comp.p, flag ? flag : err_ptr(),
                        visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), ghist.as<uint32_t>());
     }
   }
@@ -774,8 +774,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     StreamSwitch on(*this, index_stream);
     HCTR_HIP(hipEventRecord(ev0, stream));
     m->swap_batches();
-    m->ingest_keys(keys[0], n[0]);
-    HCTR_HIP(hipMemcpyAsync(&m->mirror->st.err, m->err_ptr(), 4, hipMemcpyDeviceToHost, stream));
+    m->ingest_keys(keys[0], n[0], &m->mirror->key_err); // the flag lives in pinned host memory the kernel can write
     HCTR_HIP(hipEventRecord(ev1, stream));
     HCTR_HIP(hipEventRecord(ev_keys, stream));
     enqueue_index(m);
@@ -788,9 +787,9 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     float ms = 0.f;
     HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
     m->last_pre_ms = ms;
-    if (m->mirror->st.err) {
-      wait_for(index_stream); // the later read-back of the same flag must land before the flag is cleared
-      m->check_key_error();
+    if (m->mirror->key_err) {
+      m->mirror->key_err = 0;
+      throw Error("hetuCTR: preprocess: a key lies outside [0, length) (it was treated as id 0)");
     }
     return;
   }
