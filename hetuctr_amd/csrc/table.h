@@ -107,7 +107,9 @@ class Shard {
   }
   // the caller's ids -> device copy and sort keys; flag: where the range check reports (default: the device word)
   void ingest_keys(const int64_t *keys, size_t n, uint32_t *flag = nullptr);
-  void index_batch();                              // sort, unique, run lists of the ingested batch
+  // sort, unique, run lists of the ingested batch; u_out: where the number of unique keys goes besides the batch's
+  // own device word (default: the device block that is read back after the call)
+  void index_batch(uint32_t *u_out = nullptr);
   void preprocess_gradient();
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks

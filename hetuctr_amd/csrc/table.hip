@@ -228,7 +228,7 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag) {
   }
 }
 
-void Shard::index_batch() {
+void Shard::index_batch(uint32_t *u_out) {
   hipStream_t s = group->stream;
   if (cur.n != 0) {
     SortScratch sc;
@@ -252,7 +252,7 @@ void Shard::index_batch() {
     }
     delete sort_scope;
     StageScope st(*group, S_UNIQUE);
-    launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>(), &dst_->U);
+    launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>(), u_out ? u_out : &dst_->U);
     launch_list_long_runs(s, cur.view());
   }
   if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt);
@@ -747,10 +747,11 @@ void wait_for(hipStream_t s) {
 } // namespace
 
 // Enqueues the index stages of the ingested batch (single shard) on the stream the stages currently use.
+// The number of unique keys is written by its kernel straight into the pinned host block finish_preprocess() reads: no
+// copy stands between the last index kernel and the gather that waits for it.
 static void enqueue_index(Shard *m) {
-  m->index_batch();
-  m->preprocess_gradient();
-  m->enqueue_readback_preprocess();
+  if (m->cur.n == 0) m->mirror->st.U = 0; // nothing of this shard is in flight that writes the block
+  m->index_batch(&m->mirror->st.U);
 }
 
 void Group::flush_index() {
