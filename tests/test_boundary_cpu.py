@@ -112,3 +112,6 @@ def test_workload_byte_accounting():
     assert total == 4 * w * (2 * n + 3 * u) + 41 * n + 81 * u
     assert workloads.stage_bytes("segment_sum_apply", n, u, n, u, w) == 4 * w * n + 8 * w * u + 8 * n + 32 * u
     assert workloads.stage_bytes("gather", n, u, n, u, w) == 4 * w * n + 4 * w * u + 8 * n + 8 * u
+    # the partitioner's cache-candidate kernels: 68 B per embedding for the keys at 8 parts, 76 B per (embedding, part)
+    # for the four sort passes, 8 B per kept candidate
+    assert workloads.cache_list_bytes(1000, 8, 100) == 1000 * 68 + 8 * 1000 * 76 + 8 * 100 * 8

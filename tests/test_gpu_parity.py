@@ -249,6 +249,8 @@ def test_key_buffer_is_free_when_preprocess_returns():
         o.preprocess([keys])
         ref = o.push_pull([g if prev else None])[0]
         assert np.array_equal(dst.cpu().numpy(), ref), "step %d" % step
+        pre_ms, pp_ms = t.last_times()
+        assert pre_ms > 0 and pp_ms > 0 and 0 <= t.last_push_ms() <= pp_ms   # device times of the two calls
         for item in (capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.KEYS):
             assert np.array_equal(t.fetch(item), o.fetch(0, item)), (step, item)
         prev = n
