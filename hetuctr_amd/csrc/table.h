@@ -113,6 +113,11 @@ class Shard {
   void preprocess_gradient();
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
+  // the same in two halves, for a preprocess whose push plan and index run on different streams
+  void enqueue_readback_plan();
+  void enqueue_readback_index();
+  void finish_plan();
+  void finish_index();
   void check_key_error();                   // raises if the ingested batch held a key outside [0, length)
   void generate_gradient(const float *grad);
   void generate_query();
@@ -129,7 +134,7 @@ class Shard {
   DeviceBuf root, slot, emb, ver, pend, upd, store_ids;
   // scratch shared by the stages
   DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, ghist, bintot, block_sums, dstat, stats;
-  DeviceBuf need, prefix;
+  DeviceBuf need, prefix, plan_sums; // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
   DevStat *dst_ = nullptr; // == dstat.p
   uint32_t *err_ptr() const { return &dst_->err; }
   // send side
@@ -167,7 +172,7 @@ class Group {
   // push on the main stream right away and only the gather waits for both.
   hipStream_t index_stream = nullptr;
   hipEvent_t ev_index = nullptr, ev_keys = nullptr, ev_push = nullptr;
-  bool defer_index = false;              // the mode is on (one shard, HETUCTR_DEFER_INDEX != 0)
+  bool defer_index = false;              // the mode is on (HETUCTR_DEFER_INDEX != 0)
   bool index_pending = false;            // a batch's index is enqueued and nobody has waited for it yet
   void flush_index();                    // waits for a pending index and takes its results over
   std::vector<Shard *> members;

@@ -274,11 +274,11 @@ void Shard::preprocess_gradient() {
   plan_cleared = false;
   need.reserve((size_t)prev.n * 4);
   prefix.reserve((size_t)prev.n * 4);
-  reserve_batch_scratch(prev.n);
+  plan_sums.reserve((scan_blocks(prev.n) + 2) * 4); // its own: the index of the current batch may be running beside it
   StageScope st(*group, S_PLAN);
   launch_decide_update(s, tv, kl, prev.view(), need.as<uint32_t>());
   launch_exclusive_scan(s, need.as<uint32_t>(), prefix.as<uint32_t>(), prev.n, prev.dU.as<uint32_t>(),
-                        block_sums.as<uint32_t>(), &dst_->push_total);
+                        plan_sums.as<uint32_t>(), &dst_->push_total);
   launch_bucket_counts(s, prev.view(), prefix.as<uint32_t>(), &dst_->push_total, cfg.nrank, cnt);
 }
 
@@ -293,17 +293,40 @@ void Shard::enqueue_readback_preprocess() {
 }
 
 void Shard::finish_preprocess() {
-  cur.U = mirror->st.U;
-  prev_active = prev.n > 0;
-  if (cfg.nrank == 1) {
-    cur.send_cnt[0] = cur.U;
-    prev.push_cnt[0] = 0;
-  } else {
-    for (int i = 0; i <= cfg.nrank; i++) {
-      cur.send_cnt[i] = mirror->st.send_cnt[i];
-      prev.push_cnt[i] = mirror->st.push_cnt[i];
-    }
+  finish_plan();
+  finish_index();
+}
+
+// The two halves of the read-back: what the push plan of the previous batch produced (rows pushed per owner) and what
+// the index of the current batch produced (unique keys, queries per owner, the error word).
+void Shard::enqueue_readback_plan() {
+  if (cfg.nrank == 1) return;
+  HCTR_HIP(hipMemcpyAsync(mirror->st.push_cnt, dst_->push_cnt, (size_t)(cfg.nrank + 1) * sizeof(uint64_t),
+                          hipMemcpyDeviceToHost, group->stream));
+}
+
+void Shard::enqueue_readback_index() {
+  hipStream_t s = group->stream;
+  if (cur.n == 0 && !u_cleared) {
+    HCTR_HIP(hipMemsetAsync(&dst_->U, 0, 4, s));
+    u_cleared = true;
   }
+  const size_t bytes = offsetof(DevStat, send_cnt) + (size_t)(cfg.nrank + 1) * sizeof(uint64_t);
+  HCTR_HIP(hipMemcpyAsync(&mirror->st, dstat.p, bytes, hipMemcpyDeviceToHost, s));
+}
+
+void Shard::finish_plan() {
+  prev_active = prev.n > 0;
+  if (cfg.nrank == 1) prev.push_cnt[0] = 0;
+  else
+    for (int i = 0; i <= cfg.nrank; i++) prev.push_cnt[i] = mirror->st.push_cnt[i];
+}
+
+void Shard::finish_index() {
+  cur.U = mirror->st.U;
+  if (cfg.nrank == 1) cur.send_cnt[0] = cur.U;
+  else
+    for (int i = 0; i <= cfg.nrank; i++) cur.send_cnt[i] = mirror->st.send_cnt[i];
   check_key_error();
 }
 
@@ -563,7 +586,7 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   HCTR_HIP(hipEventCreateWithFlags(&ev_keys, hipEventDisableTiming));
   HCTR_HIP(hipEventCreate(&ev_push));
   const char *defer = getenv("HETUCTR_DEFER_INDEX");
-  defer_index = nr == 1 && !(defer && atoi(defer) == 0);
+  defer_index = !(defer && atoi(defer) == 0);
   HCTR_HIP(hipEventCreate(&ev0));
   HCTR_HIP(hipEventCreate(&ev1));
   a_keys_.resize(nr);
@@ -759,7 +782,9 @@ void Group::flush_index() {
   index_pending = false;
   HCTR_HIP(hipSetDevice(device_id));
   wait_for(index_stream);
-  members[0]->finish_preprocess();
+  if (nrank == 1) members[0]->finish_preprocess();
+  else
+    for (Shard *m : members) m->finish_index(); // the plan half was taken over when preprocess returned
   exchange_shapes();
 }
 
@@ -767,7 +792,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
   flush_index(); // preprocess twice in a row: the earlier batch is indexed before it becomes the previous one
-  if (defer_index && !stage_timing) {
+  if (defer_index && !stage_timing && nrank == 1) {
     // One shard: everything is enqueued on the second stream, and the call returns as soon as the caller's ids have
     // been read.  Sorting and deduplicating them does not depend on the pending gradient push, which the next
     // push_pull puts on the main stream while this is still running; the gather waits for both.
@@ -792,6 +817,45 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
       m->mirror->key_err = 0;
       throw Error("hetuCTR: preprocess: a key lies outside [0, length) (it was treated as id 0)");
     }
+    return;
+  }
+  if (defer_index && !stage_timing) {
+    // Several shards: the ids are read and the push plan of the previous batches is made on the main stream, and the
+    // call returns when that is done (the plan sizes the push buffers).  The index of the current batches runs on the
+    // second stream; the next push_pull starts the pushes at once and waits for the index before it builds the
+    // queries, which are the first thing that needs it.
+    HCTR_HIP(hipEventRecord(ev0, stream));
+    for (Shard *m : members) {
+      m->swap_batches();
+      m->ingest_keys(keys[m->cfg.rank], n[m->cfg.rank], &m->mirror->key_err);
+    }
+    HCTR_HIP(hipEventRecord(ev_keys, stream));
+    for (Shard *m : members) {
+      m->preprocess_gradient();
+      m->enqueue_readback_plan();
+    }
+    HCTR_HIP(hipEventRecord(ev1, stream));
+    HCTR_HIP(hipStreamWaitEvent(index_stream, ev_keys, 0));
+    {
+      StreamSwitch on(*this, index_stream);
+      for (Shard *m : members) {
+        m->index_batch();
+        m->enqueue_readback_index();
+      }
+    }
+    index_pending = true;
+    sync_stream();
+    float ms = 0.f;
+    HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+    bool bad_key = false;
+    for (Shard *m : members) {
+      m->last_pre_ms = ms;
+      m->finish_plan();
+      bad_key |= m->mirror->key_err != 0;
+      m->mirror->key_err = 0;
+    }
+    exchange_shapes();
+    if (bad_key) throw Error("hetuCTR: preprocess: a key lies outside [0, length) (it was treated as id 0)");
     return;
   }
   HCTR_HIP(hipEventRecord(ev0, stream));
@@ -833,11 +897,17 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
   HCTR_HIP(hipEventRecord(ev0, stream));
-  for (Shard *m : members) {
-    m->generate_gradient(grads[m->cfg.rank]);
-    m->generate_query();
-  }
+  for (Shard *m : members) m->generate_gradient(grads[m->cfg.rank]);
   HCTR_HIP(hipEventRecord(ev_push, stream));
+  if (index_pending && nrank > 1) {
+    // the pushes are queued; the queries are built from the index of the current batches, which the host needs too
+    // (unique keys and queries per owner size the exchange)
+    index_pending = false;
+    wait_for(index_stream);
+    for (Shard *m : members) m->finish_index();
+    exchange_shapes();
+  }
+  for (Shard *m : members) m->generate_query();
   const bool join_index = index_pending;
   if (join_index) {
     // the push kernel is in the main stream's queue; the gather below also needs the index of the current batch,

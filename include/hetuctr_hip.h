@@ -102,9 +102,10 @@ int hctr_stream(hctr_table *t, void **stream_out);
  * that stream around the launched work (host-side waits excluded). */
 int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
 
-/* With one shard, hctr_preprocess returns as soon as the caller's ids have been read (the buffer may be reused): the
- * sort / unique stages of that batch keep running on a second stream, next to the gradient push that the following
- * hctr_push_pull starts, and are waited for before the rows are gathered.  preprocess_ms above is then the time up to
+/* hctr_preprocess returns as soon as the caller's ids have been read (the buffer may be reused) and, with several
+ * shards, the push plan of the previous batch is made.  The sort / unique stages of that batch keep running on a
+ * second stream, next to the gradient push that the following hctr_push_pull starts, and are waited for before the
+ * rows are gathered (several shards: before the queries are built).  preprocess_ms above is then the time up to
  * that return, push_pull_ms covers the rest.  Anything that needs the batch's index earlier (a second hctr_preprocess,
  * hctr_debug_fetch, hctr_stage_timing) waits for it.  HETUCTR_DEFER_INDEX=0 in the environment restores a
  * preprocess that returns only when all its work is done (hetu_gpu_table.cu:64); with stage timing on it always is.
