@@ -133,6 +133,7 @@ struct PullArgs {
   const version_t *in_ver;
   const embed_t *in_val;
   embed_t *dst;              // [n][width]
+  bool stream_stores;        // write dst with nontemporal stores (see Shard::write_back)
 };
 void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
                     uint32_t *stats);

@@ -152,11 +152,10 @@ __global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, Pull
 #ifndef HCTR_GATHER_ROWS
 #define HCTR_GATHER_ROWS 8
 #endif
-#ifndef HCTR_GATHER_NT
-#define HCTR_GATHER_NT 1
-#endif
 constexpr int kRows = HCTR_GATHER_ROWS;
-template <int VEC, int LPR, bool kLocalOnly>
+// kStream: dst is written with nontemporal stores (a compile-time choice: merged into one store by the compiler, a
+// run-time one loses the hint)
+template <int VEC, int LPR, bool kLocalOnly, bool kStream>
 __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullArgs a) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
@@ -183,7 +182,7 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
 #pragma unroll
     for (int k = 0; k < kRows; k++)
       if (j0 + k < n) {
-        if (HCTR_GATHER_NT) __builtin_nontemporal_store(v[k], (V *)(dst[k] + col));
+        if (kStream) __builtin_nontemporal_store(v[k], (V *)(dst[k] + col));
         else *(V *)(dst[k] + col) = v[k];
       }
   }
@@ -305,8 +304,10 @@ void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, cons
 #define CALL(V, L)                                                                                               \
   do {                                                                                                           \
     const unsigned blocks = div_up(div_up(cur.n, kRows), kBlock / L);                                            \
-    if (local_only) hipLaunchKernelGGL((gather<V, L, true>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a);       \
-    else hipLaunchKernelGGL((gather<V, L, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a);                 \
+    if (local_only && a.stream_stores) hipLaunchKernelGGL((gather<V, L, true, true>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a); \
+    else if (local_only) hipLaunchKernelGGL((gather<V, L, true, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a); \
+    else if (a.stream_stores) hipLaunchKernelGGL((gather<V, L, false, true>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a); \
+    else hipLaunchKernelGGL((gather<V, L, false, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a);          \
   } while (0)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL

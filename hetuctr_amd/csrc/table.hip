@@ -458,6 +458,10 @@ void Shard::write_back(float *dst) {
   a.in_ver = nullptr;
   a.in_val = nullptr;
   a.dst = dst;
+  // The gathered rows are not read again by this library: streamed past the caches they leave the table rows of the
+  // batch there for the push that updates them next.  The one case where that loses is a batch of (almost) all
+  // distinct keys, where the gather reads as many rows as it writes; the previous batch is the predictor.
+  a.stream_stores = !(prev.n != 0 && (double)prev.U >= 0.9 * (double)prev.n);
   if (cfg.nrank > 1) {
     ret_i.reserve(std::max<uint32_t>(cur.U, 1) * 4);
     reserve_batch_scratch(cur.U);
