@@ -75,9 +75,10 @@ struct TableView {
 
 // ---- preprocess ---------------------------------------------------------------------------------
 // ids -> sort keys; flags ids outside [0, id_max) in *err (and sorts them as id 0)
-// keys_copy (optional): the ids are also copied there (the reference's d_idx); nlong (optional) is zeroed
+// keys_copy (optional): the ids are also copied there (the reference's d_idx); nlong (optional) is zeroed;
+// sort_counts: the sort's scratch, which receives the per-tile counts of the first pass' digit
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong, uint32_t *ghist);
+                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong, uint32_t *sort_counts);
 // sorted keys -> everything per unique key + inverse index.  block_heads: scratch of scan_blocks(n) words.
 // u_copy (optional) receives the number of unique keys as well (b.d_U always does)
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,

@@ -401,10 +401,9 @@ void Partitioner::cache_lists(size_t max_len, int32_t *lists, size_t *lens, floa
   DevMem d_keys((size_t)P * n * 4), k0((size_t)n * 4), k1((size_t)n * 4), v0((size_t)n * 4), v1((size_t)n * 4),
       pos((size_t)n * 4), d_lists((size_t)P * keep * 4);
   SortScratch sc;
-  sc.blocks_cap = sort_blocks(n);
-  DevMem d_hist(((size_t)1 << kSortMaxDigitBits) * sc.blocks_cap * 4), d_tot(((size_t)1 << kSortMaxDigitBits) * 4);
-  sc.ghist = d_hist.as<uint32_t>();
-  sc.bintot = d_tot.as<uint32_t>();
+  DevMem d_ws(sort_scratch_words(n) * 4);
+  sc.words = d_ws.as<uint32_t>();
+  sc.n_cap = n;
   hipStream_t s = nullptr;
   HCTR_HIP(hipMemcpyAsync(d_cnt.p, cnt.data(), cnt.size() * 4, hipMemcpyHostToDevice, s));
   HCTR_HIP(hipMemcpyAsync(d_owner.p, res_embed.data(), n_embed * 4, hipMemcpyHostToDevice, s));
@@ -426,7 +425,7 @@ void Partitioner::cache_lists(size_t max_len, int32_t *lists, size_t *lens, floa
     const uint32_t *sorted_keys;
     radix_sort_positions<uint32_t>(s, d_keys.as<uint32_t>() + (size_t)i * n, n, 32, k0.as<uint32_t>(),
                                    k1.as<uint32_t>(), v0.as<uint32_t>(), v1.as<uint32_t>(), pos.as<uint32_t>(), sc,
-                                   &sorted_keys, false, true);
+                                   &sorted_keys);
     lens[i] = std::min<size_t>(keep, n_embed - (size_t)cnt_embed[i]);
     if (lens[i]) {
       hipLaunchKernelGGL(emit_reversed, dim3(div_up(lens[i], kKeyBlock)), dim3(kKeyBlock), 0, s, pos.as<uint32_t>(), n,

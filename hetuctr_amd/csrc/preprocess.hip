@@ -14,35 +14,31 @@ constexpr int kItems = 8;
 constexpr int kTile = kBlock * kItems; // 2048: scan_blocks(n) sizes the scratch
 
 // ids -> sort keys (owner << id_bits | id), the copy of the ids, the range check, the reset of the batch's run
-// counters, and the per-block counts of the first sort pass' digit: a block works on one sort tile, so the sort
-// needs no histogram launch of its own for that pass.
-// one sort tile per block, with more threads than the sort's own blocks: twice the loads in flight per tile
-#ifndef HCTR_KEY_BLOCK
-#define HCTR_KEY_BLOCK 512
-#endif
-constexpr int kKeyBlock = HCTR_KEY_BLOCK, kKeyItems = kSortTile / kKeyBlock;
+// counters, and the per-tile counts of the first sort pass' digit: a block works on one sort tile, so the sort
+// needs no counting launch of its own for that pass.  This is the one kernel that reads the caller's buffer: the
+// call may return when it is through.
 template <typename K>
-__global__ __launch_bounds__(kKeyBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
-                                                        int id_bits, int nrank, const worker_t *__restrict__ root,
-                                                        K *__restrict__ comp, uint32_t *__restrict__ err,
-                                                        index_t *__restrict__ keys_copy, uint32_t *__restrict__ nlong,
-                                                        int dbits, uint32_t *__restrict__ ghist, uint32_t nblocks) {
-  __shared__ uint32_t h[1 << kSortMaxDigitBits];
+__global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
+                                                         int id_bits, int nrank, const worker_t *__restrict__ root,
+                                                         K *__restrict__ comp, uint32_t *__restrict__ err,
+                                                         index_t *__restrict__ keys_copy, uint32_t *__restrict__ nlong,
+                                                         int dbits, uint32_t *__restrict__ counts) {
+  __shared__ uint32_t h[kSortMaxBins];
   const uint32_t nb = 1u << dbits, mask = nb - 1;
-  for (uint32_t i = threadIdx.x; i < nb; i += kKeyBlock) h[i] = 0;
+  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
   if (blockIdx.x == 0 && threadIdx.x < kRunCounters && nlong) nlong[threadIdx.x] = 0; // counters of this batch
-  __syncthreads();
   const uint32_t base = blockIdx.x * kSortTile;
-  uint64_t id[kKeyItems];
+  uint64_t id[kSortItems];
 #pragma unroll
-  for (int k = 0; k < kKeyItems; k++) {
-    const uint32_t i = base + k * kKeyBlock + threadIdx.x;
+  for (int k = 0; k < kSortItems; k++) {
+    const uint32_t i = base + k * kSortBlock + threadIdx.x;
     id[k] = i < n ? (uint64_t)load_once(&keys[i]) : 0; // the caller's ids are read here and nowhere else
   }
+  __syncthreads();
   bool bad = false;
 #pragma unroll
-  for (int k = 0; k < kKeyItems; k++) {
-    const uint32_t i = base + k * kKeyBlock + threadIdx.x;
+  for (int k = 0; k < kSortItems; k++) {
+    const uint32_t i = base + k * kSortBlock + threadIdx.x;
     if (i >= n) continue;
     if (keys_copy) __builtin_nontemporal_store((index_t)id[k], &keys_copy[i]); // only read back on request
     if (id[k] >= id_max) { // also catches negative ids
@@ -51,19 +47,18 @@ __global__ __launch_bounds__(kKeyBlock) void make_keys(const index_t *__restrict
     }
   }
   if (bad) atomicOr(err, 1u);
-  uint64_t owner[kKeyItems];
+  uint64_t owner[kSortItems];
 #pragma unroll
-  for (int k = 0; k < kKeyItems; k++) owner[k] = nrank > 1 ? root[id[k]] : 0;
+  for (int k = 0; k < kSortItems; k++) owner[k] = nrank > 1 ? root[id[k]] : 0;
 #pragma unroll
-  for (int k = 0; k < kKeyItems; k++) {
-    const uint32_t i = base + k * kKeyBlock + threadIdx.x;
-    if (i >= n) continue;
+  for (int k = 0; k < kSortItems; k++) {
+    const uint32_t i = base + k * kSortBlock + threadIdx.x;
     const K c = (K)((owner[k] << id_bits) | id[k]);
-    comp[i] = c;
-    atomicAdd(&h[(uint32_t)c & mask], 1u);
+    if (i < n) comp[i] = c;
+    count_digit(h, (uint32_t)c & mask, i < n);
   }
   __syncthreads();
-  for (uint32_t i = threadIdx.x; i < nb; i += kKeyBlock) ghist[(size_t)i * nblocks + blockIdx.x] = h[i];
+  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) counts[(size_t)blockIdx.x * nb + i] = h[i];
 }
 
 // Sorted position j of a block's tile is handled by thread (j % kBlock) in round (j / kBlock): every load
@@ -272,16 +267,16 @@ __global__ void bucket_sizes(BatchView b, int nrank, uint64_t *__restrict__ cnt_
 } // namespace
 
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong, uint32_t *ghist) {
+                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong, uint32_t *sort_counts) {
   if (!n) return;
-  const unsigned nblocks = (unsigned)sort_blocks(n);
+  const unsigned nblocks = (unsigned)sort_tiles(n);
   const int dbits = sort_first_digit_bits(kl.total_bits);
   if (kl.wide)
-    hipLaunchKernelGGL(make_keys<uint64_t>, dim3(nblocks), dim3(kKeyBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
-                       t.root, (uint64_t *)comp_keys, err, keys_copy, nlong, dbits, ghist, nblocks);
+    hipLaunchKernelGGL(make_keys<uint64_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
+                       t.root, (uint64_t *)comp_keys, err, keys_copy, nlong, dbits, sort_counts);
   else
-    hipLaunchKernelGGL(make_keys<uint32_t>, dim3(nblocks), dim3(kKeyBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
-                       t.root, (uint32_t *)comp_keys, err, keys_copy, nlong, dbits, ghist, nblocks);
+    hipLaunchKernelGGL(make_keys<uint32_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
+                       t.root, (uint32_t *)comp_keys, err, keys_copy, nlong, dbits, sort_counts);
   HCTR_HIP(hipGetLastError());
 }
 

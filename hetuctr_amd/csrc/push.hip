@@ -387,6 +387,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
   const uint32_t share = min(min(slices, nblk), (uint32_t)kTicketLanes);
   const uint32_t lane_id = bidx % share;
   const uint32_t n_sl = (slices - lane_id + share - 1) / share; // slices lane_id, lane_id + share, ...
+  const uint32_t group_blocks = (nblk - lane_id + share - 1) / share; // blocks drawing from this counter
   uint32_t cnt[kLongBuckets];
   uint32_t nbundles = 0;
 #pragma unroll
@@ -405,7 +406,14 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
     if (threadIdx.x == 0) tk = atomicAdd(counters + lane_id, 1u);
     tk = (uint32_t)__builtin_amdgcn_readfirstlane((int)tk);
     pend_runs = 0;
-    if (tk >= tickets) return;
+    if (tk >= tickets) {
+      // Every block of the group draws exactly one ticket past the end.  The block that draws the last of them
+      // knows that nobody will touch the counter again in this launch and puts it back to zero, so that the same
+      // batch can be pushed again (push_pull twice without a preprocess in between applies the gradient twice,
+      // csrc/core/hetu_gpu_table.cu:9-41).
+      if (threadIdx.x == 0 && tk == tickets + group_blocks - 1) atomicExch(counters + lane_id, 0u);
+      return;
+    }
     uint32_t bundle = tk / n_sl;
     pend_slice = lane_id + (tk % n_sl) * share;
     int cls = 0;

@@ -5,24 +5,26 @@
 
 namespace hctr {
 
-constexpr int kSortBlock = 256;                 // threads per block (4 waves)
+#ifndef HCTR_SORT_BLOCK
+#define HCTR_SORT_BLOCK 512
+#endif
+constexpr int kSortBlock = HCTR_SORT_BLOCK;     // threads per block
 #ifndef HCTR_SORT_ITEMS
-#define HCTR_SORT_ITEMS 16
+#define HCTR_SORT_ITEMS 8
 #endif
 constexpr int kSortItems = HCTR_SORT_ITEMS;     // keys per thread
 constexpr int kSortTile = kSortBlock * kSortItems;
-constexpr int kSortMaxDigitBits = 10;           // up to 1024 bins: 4 wave-private rows of 4 KiB in LDS
+constexpr int kSortMaxDigitBits = 10;           // up to 1024 bins
+constexpr int kSortMaxBins = 1 << kSortMaxDigitBits;
+inline size_t sort_tiles(size_t n) { return (n + kSortTile - 1) / kSortTile; }
+// words of scratch a sort of n keys needs: per tile and bin the count of the digit in the earlier tiles, then the
+// total of every bin
+inline size_t sort_scratch_words(size_t n) { return (sort_tiles(n) + 1) * (size_t)kSortMaxBins; }
 
 struct SortScratch {
-  uint32_t *ghist = nullptr;   // [bins][blocks] per-block digit counts, scanned in place per bin
-  uint32_t *bintot = nullptr;  // [bins] totals per digit value
-  size_t blocks_cap = 0;
+  uint32_t *words = nullptr;   // sort_scratch_words(n) of them
+  size_t n_cap = 0;            // the n they were sized for
 };
-
-inline size_t sort_blocks(size_t n) { return (n + kSortTile - 1) / kSortTile; }
-// a sort of at most this many tiles launches no scan kernel: every block of the scatter sums the raw per-block counts
-// of its bins itself (the sum over so few blocks costs less than a launch)
-constexpr uint32_t kSmallSortBlocks = 16;
 // tiles of the scan / unique kernels of the preprocess (256 threads x 8 items), whatever the sort tile is
 inline size_t scan_blocks(size_t n) { return (n + 2047) / 2048; }
 
@@ -33,23 +35,40 @@ inline int sort_first_digit_bits(int bits) {
   return (bits + passes - 1) / passes;
 }
 
+// One key's digit into the block's LDS counters h[].  Called by every lane of the wave with consecutive keys in
+// consecutive lanes; lanes inside the input (`in`) are a prefix of the wave.  A run of equal digits in consecutive
+// lanes (what a partly sorted input and a hot key make of most waves) adds once, from its first lane, so that the
+// LDS atomics of one instruction rarely meet on one word.
+__device__ __forceinline__ void count_digit(uint32_t *h, uint32_t d, bool in) {
+  const unsigned lane = lane_id();
+  const uint32_t dp = __shfl_up(d, 1, kWave);
+  const bool head = in && (lane == 0 || d != dp);
+  const uint64_t act = __ballot(in);
+  const uint64_t heads = __ballot(head);
+  if (head) {
+    const uint64_t above = lane == 63 ? 0ull : (heads >> (lane + 1));
+    const uint32_t end = above ? lane + 1 + (uint32_t)__builtin_ctzll(above) : (uint32_t)__popcll(act);
+    atomicAdd(&h[d], end - lane);
+  }
+}
+
 // Sorts n pairs by the low `bits` bits of the key.  The value of element i is its position i (never
 // materialised as an input).  keys_in is left untouched; tmp_k0/tmp_k1 and tmp_v0/tmp_v1 are ping-pong
 // buffers of n elements; the sorted keys end in *keys_sorted (one of tmp_k0/tmp_k1) and the sorted
-// positions in vals_out.  n == 0 is a no-op.  first_hist_done: scratch.ghist already holds the per-block counts of
-// the first pass' digit (sort_first_digit_bits(bits) low bits, tiles of kSortTile keys), written by the kernel
-// that made the keys.  long_runs: most keys are expected to repeat over long stretches of the input (the digit counts
-// then add once per wave where a wave's keys agree).
+// positions in vals_out.  n == 0 is a no-op.  Three launches per pass of up to kSortMaxDigitBits bits.
+// first_counts_done: scratch.words already holds the per-tile counts of the first pass' digit
+// (sort_first_digit_bits(bits) low bits, rows of 1 << that many words, tiles of kSortTile keys), written by the
+// kernel that made the keys (see count_digit).
 template <typename K>
 void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
                           uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
-                          const K **keys_sorted, bool first_hist_done = false, bool long_runs = false);
+                          const K **keys_sorted, bool first_counts_done = false);
 
 extern template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *,
                                                     uint32_t *, uint32_t *, uint32_t *, uint32_t *,
-                                                    const SortScratch &, const uint32_t **, bool, bool);
+                                                    const SortScratch &, const uint32_t **, bool);
 extern template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *,
                                                     uint64_t *, uint32_t *, uint32_t *, uint32_t *,
-                                                    const SortScratch &, const uint64_t **, bool, bool);
+                                                    const SortScratch &, const uint64_t **, bool);
 
 } // namespace hctr

@@ -133,7 +133,7 @@ class Shard {
   bool prev_active = false; // false: inference step or no previous batch, nothing is pushed
   DeviceBuf root, slot, emb, ver, pend, upd, store_ids;
   // scratch shared by the stages
-  DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, ghist, bintot, block_sums, dstat, stats;
+  DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, sortws, block_sums, dstat, stats;
   DeviceBuf need, prefix, plan_sums; // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
   DevStat *dst_ = nullptr; // == dstat.p
   uint32_t *err_ptr() const { return &dst_->err; }

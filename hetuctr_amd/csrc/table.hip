@@ -190,9 +190,7 @@ void Shard::reserve_batch_scratch(uint32_t n) {
   ktmp1.reserve(m * ks);
   vtmp0.reserve(m * 4);
   vtmp1.reserve(m * 4);
-  const size_t blocks = sort_blocks(m);
-  ghist.reserve(((size_t)1 << kSortMaxDigitBits) * blocks * 4);
-  bintot.reserve(((size_t)1 << kSortMaxDigitBits) * 4);
+  sortws.reserve(sort_scratch_words(m) * 4);
   block_sums.reserve((scan_blocks(m) + 2) * 4);
 }
 
@@ -223,7 +221,7 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag) {
         HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
       }
       launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, comp.p, flag ? flag : err_ptr(),
-                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), ghist.as<uint32_t>());
+                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), sortws.as<uint32_t>());
     }
   }
 }
@@ -232,9 +230,8 @@ void Shard::index_batch(uint32_t *u_out) {
   hipStream_t s = group->stream;
   if (cur.n != 0) {
     SortScratch sc;
-    sc.ghist = ghist.as<uint32_t>();
-    sc.bintot = bintot.as<uint32_t>();
-    sc.blocks_cap = sort_blocks(cur.n);
+    sc.words = sortws.as<uint32_t>();
+    sc.n_cap = cur.n;
     const void *sorted_keys = nullptr;
     StageScope *sort_scope = new StageScope(*group, S_SORT);
     if (kl.wide) {

@@ -345,3 +345,40 @@ def test_table_closed_while_the_index_is_still_running():
     out, ref = p.push_pull([np.zeros((0, width), np.float32)])
     assert np.array_equal(out[0], ref[0])
     p.close()
+
+
+@pytest.mark.parametrize("nrank", [1, 2])
+def test_push_pull_twice_without_preprocess(nrank):
+    # The same previous batch pushed twice: the reference applies the whole gradient again
+    # (csrc/core/hetu_gpu_table.cu:9-41 keeps no "already pushed" state), including the keys with more than 128
+    # duplicates, whose blocks draw their work from counters that have to be back at zero for the second launch.
+    say("push_pull twice, shards", nrank)
+    rng = np.random.default_rng(36 + nrank)
+    length, width, n = 20_000, 128, 30_000
+    root = (np.arange(length) % nrank).astype(np.uint8)
+    storage = [np.concatenate([np.where(root == r)[0], np.where(root != r)[0][:500]]).astype(np.int64)
+               for r in range(nrank)]
+    p = Pair(nrank, length, width, root, storage, init=("Uniform", -0.01, 0.01), lr=0.05, bounds=(2, 2))
+    draw = zipf_sampler(length, 1.2, rng)
+
+    def batch():
+        k = np.concatenate([np.full(3000, 5, np.int64), np.full(700, 6, np.int64), np.full(200, 9, np.int64),
+                            draw(n - 3900)])
+        rng.shuffle(k)
+        return k
+
+    p.preprocess([batch() for _ in range(nrank)], device_keys=True)
+    p.preprocess([batch() for _ in range(nrank)], device_keys=True)
+    for rep in range(3):
+        g = [rng.normal(0, 1e-3, size=(n, width)).astype(np.float32) for _ in range(nrank)]
+        out, ref = p.push_pull(g)
+        for r in range(nrank):
+            assert_close(out[r], ref[r], 1e-5, "dst rank %d, push %d" % (r, rep))
+        p.compare_ints([capi.VERSION, capi.UPDATES], "push %d" % rep)
+        p.compare_state(1e-5, "push %d" % rep)
+    p.preprocess([batch() for _ in range(nrank)])          # and the table goes on as usual
+    out, ref = p.push_pull([rng.normal(0, 1e-3, size=(n, width)).astype(np.float32) for _ in range(nrank)])
+    for r in range(nrank):
+        assert_close(out[r], ref[r], 1e-5, "dst rank %d after" % r)
+    p.compare_state(1e-5, "after")
+    p.close()
