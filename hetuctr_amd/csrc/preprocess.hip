@@ -61,76 +61,96 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) counts[(size_t)blockIdx.x * nb + i] = h[i];
 }
 
-// Sorted position j of a block's tile is handled by thread (j % kBlock) in round (j / kBlock): every load
-// and store below is coalesced across the wave.
+// The unique pass works on tiles of kUTile sorted positions; position j of a tile is handled by thread (j % kUBlock)
+// in round (j / kUBlock): every load and store below is coalesced across the wave.
+constexpr int kUBlock = 512, kUItems = 8, kUTile = kUBlock * kUItems;
+inline unsigned unique_tiles(uint32_t n) { return div_up(n, kUTile); }
+
+// the key before sorted position j of this lane: the neighbouring lane holds it, except for lane 0
 template <typename K>
-__global__ __launch_bounds__(kBlock) void head_count(const K *__restrict__ sk, uint32_t n,
-                                                     uint32_t *__restrict__ block_heads) {
-  __shared__ uint32_t sm[kBlock / kWave + 1];
-  const uint32_t base = blockIdx.x * kTile;
-  uint32_t c = 0;
-#pragma unroll
-  for (int k = 0; k < kItems; k++) {
-    const uint32_t j = base + k * kBlock + threadIdx.x;
-    if (j < n) c += (j == 0) || (sk[j] != sk[j - 1]);
-  }
-  uint32_t total;
-  block_exclusive_scan<kBlock>(c, sm, total);
-  if (threadIdx.x == 0) block_heads[blockIdx.x] = total;
+__device__ __forceinline__ K key_before(const K *__restrict__ sk, uint32_t j, bool valid, K mine) {
+  K edge = (K)0;
+  if (lane_id() == 0 && valid && j > 0) edge = sk[j - 1];
+  const K up = (K)__shfl_up(mine, 1, kWave);
+  return lane_id() == 0 ? edge : up;
 }
 
 template <typename K>
-__global__ __launch_bounds__(kBlock) void unique_emit(const K *__restrict__ sk, uint32_t n, int id_bits, int nrank,
-                                                      const slot_t *__restrict__ slot,
-                                                      const uint32_t *__restrict__ block_heads, BatchView b,
-                                                      uint32_t *__restrict__ u_copy) {
-  constexpr int NW = kBlock / kWave;
-  __shared__ uint32_t sm[NW + 1];
-  __shared__ uint32_t wsum[kItems * NW + 1];
-  // unique ranks before this block
-  uint32_t s = 0;
-  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlock) s += block_heads[i];
-  uint32_t prefix;
-  block_exclusive_scan<kBlock>(s, sm, prefix);
+__global__ __launch_bounds__(kUBlock) void head_count(const K *__restrict__ sk, uint32_t n,
+                                                      uint32_t *__restrict__ tile_heads) {
+  __shared__ uint32_t sm[kUBlock / kWave + 1];
+  const uint32_t base = blockIdx.x * kUTile;
+  K key[kUItems];
+#pragma unroll
+  for (int k = 0; k < kUItems; k++) {
+    const uint32_t j = base + k * kUBlock + threadIdx.x;
+    key[k] = j < n ? sk[j] : (K)0;
+  }
+  uint32_t c = 0;
+#pragma unroll
+  for (int k = 0; k < kUItems; k++) {
+    const uint32_t j = base + k * kUBlock + threadIdx.x;
+    const K pk = key_before(sk, j, j < n, key[k]);
+    c += (j < n) && (j == 0 || key[k] != pk);
+  }
+  uint32_t total;
+  block_exclusive_scan<kUBlock>(c, sm, total);
+  if (threadIdx.x == 0) tile_heads[blockIdx.x] = total;
+}
 
-  const uint32_t base = blockIdx.x * kTile;
+template <typename K>
+__global__ __launch_bounds__(kUBlock) void unique_emit(const K *__restrict__ sk, uint32_t n, int id_bits, int nrank,
+                                                       const slot_t *__restrict__ slot,
+                                                       const uint32_t *__restrict__ tile_heads, BatchView b,
+                                                       uint32_t *__restrict__ u_copy) {
+  constexpr int NW = kUBlock / kWave;
+  __shared__ uint32_t sm[NW + 1];
+  __shared__ uint32_t wsum[kUItems * NW + 1];
+  const uint32_t base = blockIdx.x * kUTile;
   const unsigned lane = lane_id();
   const int w = threadIdx.x / kWave;
-  K key[kItems], pk[kItems];
-  bool head[kItems];
-  uint32_t before[kItems];
+  // everything that comes from memory first: the keys of the tile and the head counts of the tiles before it
+  K key[kUItems], pk[kUItems];
 #pragma unroll
-  for (int k = 0; k < kItems; k++) {
-    const uint32_t j = base + k * kBlock + threadIdx.x;
+  for (int k = 0; k < kUItems; k++) {
+    const uint32_t j = base + k * kUBlock + threadIdx.x;
+    key[k] = j < n ? sk[j] : (K)0;
+  }
+  uint32_t s = 0;
+  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kUBlock) s += tile_heads[i];
+  bool head[kUItems];
+  uint32_t before[kUItems];
+#pragma unroll
+  for (int k = 0; k < kUItems; k++) {
+    const uint32_t j = base + k * kUBlock + threadIdx.x;
     const bool valid = j < n;
-    key[k] = valid ? sk[j] : (K)0;
-    pk[k] = (valid && j > 0) ? sk[j - 1] : (K)0;
+    pk[k] = key_before(sk, j, valid, key[k]);
     head[k] = valid && (j == 0 || key[k] != pk[k]);
     const uint64_t m = __ballot(head[k]);
     before[k] = __popcll(m & ((1ull << lane) - 1ull));
     if (lane == 0) wsum[k * NW + w] = __popcll(m);
   }
-  __syncthreads();
-  if (threadIdx.x == 0) { // 32 wave totals, in item order
-    uint32_t run = 0;
+  // the directory lookups of the heads travel while the ranks are worked out
+  const K id_mask = (K)(((uint64_t)1 << id_bits) - 1);
+  slot_t off[kUItems];
 #pragma unroll
-    for (int i = 0; i < kItems * NW; i++) {
-      const uint32_t v = wsum[i];
-      wsum[i] = run;
-      run += v;
+  for (int k = 0; k < kUItems; k++) off[k] = head[k] ? slot[(uint64_t)(key[k] & id_mask)] : kNoSlot;
+  uint32_t prefix;
+  block_exclusive_scan<kUBlock>(s, sm, prefix); // unique ranks before this tile
+  if (threadIdx.x < kWave) { // the wave totals, in item order, by one wave
+    uint32_t run = 0;
+    for (int i0 = 0; i0 < kUItems * NW; i0 += kWave) {
+      const uint32_t v = wsum[i0 + lane];
+      const uint32_t inc = wave_inclusive_scan(v);
+      wsum[i0 + lane] = run + inc - v;
+      run += __shfl(inc, kWave - 1, kWave);
     }
   }
   __syncthreads();
   K *ukey = (K *)b.ukey;
-  const K id_mask = (K)(((uint64_t)1 << id_bits) - 1);
-  slot_t off[kItems];
 #pragma unroll
-  // all lookups are issued before the first store (the compiler cannot prove that the output arrays do not
-  // alias the directory, so a store in between would serialise them)
-  for (int k = 0; k < kItems; k++) off[k] = head[k] ? slot[(uint64_t)(key[k] & id_mask)] : kNoSlot;
-#pragma unroll
-  for (int k = 0; k < kItems; k++) {
-    const uint32_t j = base + k * kBlock + threadIdx.x;
+  for (int k = 0; k < kUItems; k++) {
+    const uint32_t j = base + k * kUBlock + threadIdx.x;
     if (j >= n) continue;
     const uint32_t rank = prefix + wsum[k * NW + w] + before[k] + (head[k] ? 1u : 0u) - 1u;
     const int r = (int)(key[k] >> id_bits);
@@ -283,16 +303,16 @@ void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, co
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
                    const BatchView &b, uint32_t *block_heads, uint32_t *u_copy) {
   if (!b.n) return;
-  const unsigned nb = div_up(b.n, kTile);
+  const unsigned nb = unique_tiles(b.n);
   if (kl.wide) {
-    hipLaunchKernelGGL(head_count<uint64_t>, dim3(nb), dim3(kBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
+    hipLaunchKernelGGL(head_count<uint64_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
                        block_heads);
-    hipLaunchKernelGGL(unique_emit<uint64_t>, dim3(nb), dim3(kBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
+    hipLaunchKernelGGL(unique_emit<uint64_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
                        kl.id_bits, t.nrank, t.slot, block_heads, b, u_copy);
   } else {
-    hipLaunchKernelGGL(head_count<uint32_t>, dim3(nb), dim3(kBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
+    hipLaunchKernelGGL(head_count<uint32_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
                        block_heads);
-    hipLaunchKernelGGL(unique_emit<uint32_t>, dim3(nb), dim3(kBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
+    hipLaunchKernelGGL(unique_emit<uint32_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
                        kl.id_bits, t.nrank, t.slot, block_heads, b, u_copy);
   }
   HCTR_HIP(hipGetLastError());

@@ -59,16 +59,20 @@ __device__ __forceinline__ void count_digit(uint32_t *h, uint32_t d, bool in) {
 // first_counts_done: scratch.words already holds the per-tile counts of the first pass' digit
 // (sort_first_digit_bits(bits) low bits, rows of 1 << that many words, tiles of kSortTile keys), written by the
 // kernel that made the keys (see count_digit).
+// step_from / step_to: only the launches [step_from, step_to) of the sort are enqueued by this call, launch 3 * p + k
+// being the count (k = 0), the column scan (1) or the scatter (2) of pass p; a caller that enqueues the sort in
+// pieces passes the same other arguments every time.
 template <typename K>
 void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
                           uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
-                          const K **keys_sorted, bool first_counts_done = false);
+                          const K **keys_sorted, bool first_counts_done = false, int step_from = 0,
+                          int step_to = 1 << 30);
 
 extern template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *,
                                                     uint32_t *, uint32_t *, uint32_t *, uint32_t *,
-                                                    const SortScratch &, const uint32_t **, bool);
+                                                    const SortScratch &, const uint32_t **, bool, int, int);
 extern template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *,
                                                     uint64_t *, uint32_t *, uint32_t *, uint32_t *,
-                                                    const SortScratch &, const uint64_t **, bool);
+                                                    const SortScratch &, const uint64_t **, bool, int, int);
 
 } // namespace hctr

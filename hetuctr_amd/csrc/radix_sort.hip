@@ -16,6 +16,7 @@ namespace hctr {
 namespace {
 
 constexpr int kWaves = kSortBlock / kWave;
+constexpr uint32_t kXcds = 8;              // accelerator dies of the device, each with its own L2
 constexpr int kSub = kSortTile / kWaves; // keys per wave
 constexpr int kRounds = kSub / kWave;    // 64-key groups per wave
 static_assert(kRounds * kWave * kWaves == kSortTile, "tile shape");
@@ -96,9 +97,19 @@ __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ 
 template <typename K, bool kFirst>
 __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
                                                       K *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
-                                                      uint32_t n, int shift, int dbits,
+                                                      uint32_t n, int shift, int dbits, uint32_t tiles,
                                                       const uint32_t *__restrict__ tile_prefix,
                                                       const uint32_t *__restrict__ bin_total) {
+#ifndef HCTR_SORT_NO_XCD
+  // Workgroups go to the 8 XCDs of the device in turn, and each XCD has an L2 of its own.  XCD x takes the x-th
+  // eighth of the tiles: neighbouring tiles write neighbouring pieces of every bin, so the pieces meet in one L2 and
+  // leave it as whole lines.
+  const uint32_t tiles_per_xcd = gridDim.x / kXcds;
+  const uint32_t tile = (blockIdx.x % kXcds) * tiles_per_xcd + blockIdx.x / kXcds;
+  if (tile >= tiles) return;
+#else
+  const uint32_t tile = blockIdx.x;
+#endif
   // one LDS area, used twice: first the wave-private digit counters, then the tile sorted by digit
   constexpr int kCntWords = kWaves * kSortMaxBins;
   constexpr int kTileWords = kSortTile * (int)(sizeof(K) / 4 + 1);
@@ -112,7 +123,6 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
   const uint32_t nb = 1u << dbits, mask = nb - 1;
   const int w = threadIdx.x / kWave;
   const unsigned lane = lane_id();
-  const uint32_t tile = blockIdx.x;
   // consecutive bins per thread in the scans over the bins
   const uint32_t per = nb > (uint32_t)kSortBlock ? nb / kSortBlock : 1u;
   const uint32_t blo = min(threadIdx.x * per, nb), bhi = min(blo + per, nb);
@@ -245,13 +255,14 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
 template <typename K>
 void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int bits, K *tmp_k0, K *tmp_k1,
                           uint32_t *tmp_v0, uint32_t *tmp_v1, uint32_t *vals_out, const SortScratch &scratch,
-                          const K **keys_sorted, bool first_counts_done) {
+                          const K **keys_sorted, bool first_counts_done, int step_from, int step_to) {
   *keys_sorted = keys_in;
   if (n == 0) return;
   if (bits < 1) bits = 1;
   HCTR_CHECK(bits <= (int)sizeof(K) * 8, "sort key wider than its type");
   HCTR_CHECK(scratch.words != nullptr && n <= scratch.n_cap, "sort scratch too small");
   const uint32_t tiles = (uint32_t)sort_tiles(n);
+  const uint32_t sgrid = (tiles + kXcds - 1) / kXcds * kXcds; // whole rounds over the XCDs
   uint32_t *counts = scratch.words;
   uint32_t *bin_total = scratch.words + (size_t)tiles * kSortMaxBins;
   const int passes = (bits + kSortMaxDigitBits - 1) / kSortMaxDigitBits;
@@ -266,16 +277,20 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
     K *kout = ktmp[p & 1];
     uint32_t *vout = (p == passes - 1) ? vals_out : vtmp[p & 1];
     const uint32_t nb = 1u << dbits;
-    if (p > 0 || !first_counts_done)
+    auto wanted = [&](int kind) { return 3 * p + kind >= step_from && 3 * p + kind < step_to; };
+    if (wanted(0) && (p > 0 || !first_counts_done))
       hipLaunchKernelGGL(digit_histogram<K>, dim3(tiles), dim3(kSortBlock), 0, stream, kin, n, shift, dbits, counts);
-    hipLaunchKernelGGL(scan_tiles, dim3((nb + kScanCols - 1) / kScanCols), dim3(kScanBlock), 0, stream, counts, tiles, nb,
-                       bin_total);
-    if (p == 0)
-      hipLaunchKernelGGL((scatter<K, true>), dim3(tiles), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift,
-                         dbits, counts, bin_total);
-    else
-      hipLaunchKernelGGL((scatter<K, false>), dim3(tiles), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift,
-                         dbits, counts, bin_total);
+    if (wanted(1))
+      hipLaunchKernelGGL(scan_tiles, dim3((nb + kScanCols - 1) / kScanCols), dim3(kScanBlock), 0, stream, counts, tiles,
+                         nb, bin_total);
+    if (wanted(2)) {
+      if (p == 0)
+        hipLaunchKernelGGL((scatter<K, true>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift,
+                           dbits, tiles, counts, bin_total);
+      else
+        hipLaunchKernelGGL((scatter<K, false>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
+                           shift, dbits, tiles, counts, bin_total);
+    }
     HCTR_HIP(hipGetLastError());
     kin = kout;
     vin = vout;
@@ -286,9 +301,9 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
 
 template void radix_sort_positions<uint32_t>(hipStream_t, const uint32_t *, uint32_t, int, uint32_t *, uint32_t *,
                                              uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
-                                             const uint32_t **, bool);
+                                             const uint32_t **, bool, int, int);
 template void radix_sort_positions<uint64_t>(hipStream_t, const uint64_t *, uint32_t, int, uint64_t *, uint64_t *,
                                              uint32_t *, uint32_t *, uint32_t *, const SortScratch &,
-                                             const uint64_t **, bool);
+                                             const uint64_t **, bool, int, int);
 
 } // namespace hctr

@@ -82,6 +82,10 @@ struct HostMirror {
 
 class Group;
 
+// launches of the sort that a deferred preprocess of a single shard enqueues itself: the column scan and the scatter
+// of the first pass and the count of the second (the first count comes from the key kernel)
+constexpr int kEarlySortSteps = 4;
+
 // stages whose device time can be measured separately (HIP events on the group's stream)
 enum Stage { S_KEYS = 0, S_SORT, S_UNIQUE, S_PLAN, S_PUSH, S_QUERY, S_EXCHANGE, S_OWNER, S_REFRESH, S_GATHER, S_COUNT };
 const char *stage_name(int s);
@@ -109,7 +113,7 @@ class Shard {
   void ingest_keys(const int64_t *keys, size_t n, uint32_t *flag = nullptr);
   // sort, unique, run lists of the ingested batch; u_out: where the number of unique keys goes besides the batch's
   // own device word (default: the device block that is read back after the call)
-  void index_batch(uint32_t *u_out = nullptr);
+  void index_batch(uint32_t *u_out = nullptr, int part = 0);
   void preprocess_gradient();
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
@@ -174,7 +178,10 @@ class Group {
   hipEvent_t ev_index = nullptr, ev_keys = nullptr, ev_push = nullptr;
   bool defer_index = false;              // the mode is on (HETUCTR_DEFER_INDEX != 0)
   bool index_pending = false;            // a batch's index is enqueued and nobody has waited for it yet
+  bool index_rest_pending = false;       // single shard: preprocess enqueued only the first launches of the index
+  void enqueue_index_rest();             // enqueues the others
   void flush_index();                    // waits for a pending index and takes its results over
+  bool time_calls = false;               // bracket the two calls with events (hctr_last_times switches it on)
   std::vector<Shard *> members;
   DeviceBuf desc_dev;
   CopyDesc *desc_host = nullptr;

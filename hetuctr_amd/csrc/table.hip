@@ -226,32 +226,37 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag) {
   }
 }
 
-void Shard::index_batch(uint32_t *u_out) {
+void Shard::index_batch(uint32_t *u_out, int part) {
   hipStream_t s = group->stream;
+  // part 1: the first kEarlySortSteps launches of the sort; part 2: everything after them; 0: all of it
+  const int from = part == 2 ? kEarlySortSteps : 0, to = part == 1 ? kEarlySortSteps : (1 << 30);
   if (cur.n != 0) {
     SortScratch sc;
     sc.words = sortws.as<uint32_t>();
     sc.n_cap = cur.n;
     const void *sorted_keys = nullptr;
-    StageScope *sort_scope = new StageScope(*group, S_SORT);
-    if (kl.wide) {
-      const uint64_t *sk;
-      radix_sort_positions<uint64_t>(s, comp.as<uint64_t>(), cur.n, kl.total_bits, ktmp0.as<uint64_t>(),
-                                     ktmp1.as<uint64_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
-                                     cur.sorted_arg.as<uint32_t>(), sc, &sk, true);
-      sorted_keys = sk;
-    } else {
-      const uint32_t *sk;
-      radix_sort_positions<uint32_t>(s, comp.as<uint32_t>(), cur.n, kl.total_bits, ktmp0.as<uint32_t>(),
-                                     ktmp1.as<uint32_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
-                                     cur.sorted_arg.as<uint32_t>(), sc, &sk, true);
-      sorted_keys = sk;
+    {
+      StageScope sort_scope(*group, S_SORT);
+      if (kl.wide) {
+        const uint64_t *sk;
+        radix_sort_positions<uint64_t>(s, comp.as<uint64_t>(), cur.n, kl.total_bits, ktmp0.as<uint64_t>(),
+                                       ktmp1.as<uint64_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
+                                       cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
+        sorted_keys = sk;
+      } else {
+        const uint32_t *sk;
+        radix_sort_positions<uint32_t>(s, comp.as<uint32_t>(), cur.n, kl.total_bits, ktmp0.as<uint32_t>(),
+                                       ktmp1.as<uint32_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
+                                       cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
+        sorted_keys = sk;
+      }
     }
-    delete sort_scope;
+    if (part == 1) return;
     StageScope st(*group, S_UNIQUE);
     launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>(), u_out ? u_out : &dst_->U);
     launch_list_long_runs(s, cur.view());
   }
+  if (part == 1) return;
   if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt);
 }
 
@@ -619,8 +624,9 @@ void Group::join(Shard *s) {
 void Group::leave(Shard *s) {
   std::lock_guard<std::mutex> lk(mu_);
   if (members[s->cfg.rank] == s) members[s->cfg.rank] = nullptr;
-  if (index_pending) { // the shard's buffers are about to be freed: nothing of it may still be running
+  if (index_pending || index_rest_pending) { // the shard's buffers are about to be freed: nothing of it may still be running
     index_pending = false;
+    index_rest_pending = false;
     (void)hipStreamSynchronize(index_stream);
   }
 }
@@ -770,18 +776,29 @@ void wait_for(hipStream_t s) {
 }
 } // namespace
 
-// Enqueues the index stages of the ingested batch (single shard) on the stream the stages currently use.
+// Enqueues index stages of the ingested batch (single shard) on the stream the stages currently use.
 // The number of unique keys is written by its kernel straight into the pinned host block finish_preprocess() reads: no
 // copy stands between the last index kernel and the gather that waits for it.
-static void enqueue_index(Shard *m) {
+static void enqueue_index(Shard *m, int part) {
   if (m->cur.n == 0) m->mirror->st.U = 0; // nothing of this shard is in flight that writes the block
-  m->index_batch(&m->mirror->st.U);
+  m->index_batch(&m->mirror->st.U, part);
+}
+
+// single shard: the launches of the index that preprocess left to the next call
+void Group::enqueue_index_rest() {
+  if (!index_rest_pending) return;
+  index_rest_pending = false;
+  StreamSwitch on(*this, index_stream);
+  enqueue_index(members[0], 2);
+  HCTR_HIP(hipEventRecord(ev_index, stream));
+  index_pending = true;
 }
 
 void Group::flush_index() {
-  if (!index_pending) return;
-  index_pending = false;
+  if (!index_pending && !index_rest_pending) return;
   HCTR_HIP(hipSetDevice(device_id));
+  enqueue_index_rest();
+  index_pending = false;
   wait_for(index_stream);
   if (nrank == 1) members[0]->finish_preprocess();
   else
@@ -797,23 +814,27 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     // One shard: everything is enqueued on the second stream, and the call returns as soon as the caller's ids have
     // been read.  Sorting and deduplicating them does not depend on the pending gradient push, which the next
     // push_pull puts on the main stream while this is still running; the gather waits for both.
+    // The host returns as early as it can, because the caller's next call is what starts the gradient push: only
+    // the first launches of the index are enqueued here (they keep the GPU busy until that push arrives), the rest
+    // follows from push_pull once the push kernel is in its queue.
     Shard *m = members[0];
     StreamSwitch on(*this, index_stream);
-    HCTR_HIP(hipEventRecord(ev0, stream));
+    if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
     m->swap_batches();
     m->ingest_keys(keys[0], n[0], &m->mirror->key_err); // the flag lives in pinned host memory the kernel can write
-    HCTR_HIP(hipEventRecord(ev1, stream));
+    if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
     HCTR_HIP(hipEventRecord(ev_keys, stream));
-    enqueue_index(m);
-    HCTR_HIP(hipEventRecord(ev_index, stream));
-    index_pending = true;
+    enqueue_index(m, 1);
+    index_rest_pending = true;
     hipError_t e;
     while ((e = hipEventQuery(ev_keys)) == hipErrorNotReady) {
     }
     HCTR_HIP(e);
-    float ms = 0.f;
-    HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
-    m->last_pre_ms = ms;
+    if (time_calls) {
+      float ms = 0.f;
+      HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+      m->last_pre_ms = ms;
+    }
     if (m->mirror->key_err) {
       m->mirror->key_err = 0;
       throw Error("hetuCTR: preprocess: a key lies outside [0, length) (it was treated as id 0)");
@@ -825,7 +846,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     // call returns when that is done (the plan sizes the push buffers).  The index of the current batches runs on the
     // second stream; the next push_pull starts the pushes at once and waits for the index before it builds the
     // queries, which are the first thing that needs it.
-    HCTR_HIP(hipEventRecord(ev0, stream));
+    if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
     for (Shard *m : members) {
       m->swap_batches();
       m->ingest_keys(keys[m->cfg.rank], n[m->cfg.rank], &m->mirror->key_err);
@@ -835,7 +856,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
       m->preprocess_gradient();
       m->enqueue_readback_plan();
     }
-    HCTR_HIP(hipEventRecord(ev1, stream));
+    if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
     HCTR_HIP(hipStreamWaitEvent(index_stream, ev_keys, 0));
     {
       StreamSwitch on(*this, index_stream);
@@ -847,7 +868,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     index_pending = true;
     sync_stream();
     float ms = 0.f;
-    HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+    if (time_calls) HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
     bool bad_key = false;
     for (Shard *m : members) {
       m->last_pre_ms = ms;
@@ -859,17 +880,17 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     if (bad_key) throw Error("hetuCTR: preprocess: a key lies outside [0, length) (it was treated as id 0)");
     return;
   }
-  HCTR_HIP(hipEventRecord(ev0, stream));
+  if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) {
     m->swap_batches();
     m->preprocess_index(keys[m->cfg.rank], n[m->cfg.rank]);
     m->preprocess_gradient();
     m->enqueue_readback_preprocess();
   }
-  HCTR_HIP(hipEventRecord(ev1, stream));
+  if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
   sync_stream();
   float ms = 0.f;
-  HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+  if (time_calls) HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
   collect_marks();
   std::string first_error;
   for (Shard *m : members) {
@@ -897,9 +918,10 @@ void Group::exchange_shapes() {
 void Group::push_pull_all(const float *const *grads, float *const *dsts) {
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
-  HCTR_HIP(hipEventRecord(ev0, stream));
+  if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) m->generate_gradient(grads[m->cfg.rank]);
-  HCTR_HIP(hipEventRecord(ev_push, stream));
+  if (time_calls) HCTR_HIP(hipEventRecord(ev_push, stream));
+  enqueue_index_rest(); // single shard: the push is in its queue, now the rest of the current batch's index
   if (index_pending && nrank > 1) {
     // the pushes are queued; the queries are built from the index of the current batches, which the host needs too
     // (unique keys and queries per owner size the exchange)
@@ -926,17 +948,18 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
     exchange_return();
   }
   for (Shard *m : members) m->write_back(dsts[m->cfg.rank]);
-  HCTR_HIP(hipEventRecord(ev1, stream));
+  if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
   sync_stream();
-  float ms = 0.f;
-  HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
   collect_marks();
   if (join_index) {
     members[0]->finish_preprocess();
     exchange_shapes();
   }
-  float push_ms = 0.f;
-  HCTR_HIP(hipEventElapsedTime(&push_ms, ev0, ev_push));
+  float ms = 0.f, push_ms = 0.f;
+  if (time_calls) {
+    HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
+    HCTR_HIP(hipEventElapsedTime(&push_ms, ev0, ev_push));
+  }
   for (Shard *m : members) {
     m->last_pp_ms = ms;
     m->last_push_ms = push_ms;

@@ -99,7 +99,9 @@ int hctr_debug_fetch(hctr_table *t, int which, void *host_out, size_t cap_elems,
 int hctr_stream(hctr_table *t, void **stream_out);
 
 /* Device time of the last preprocess and push_pull calls in milliseconds, measured with HIP events on
- * that stream around the launched work (host-side waits excluded). */
+ * that stream around the launched work (host-side waits excluded).  The events cost host time in every call, so they
+ * are recorded only from the first call of this function (or of hctr_last_push_ms) on: it returns zeros and
+ * switches the measurement on for the calls that follow. */
 int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
 
 /* hctr_preprocess returns as soon as the caller's ids have been read (the buffer may be reused) and, with several

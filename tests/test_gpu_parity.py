@@ -227,6 +227,7 @@ def test_key_buffer_is_free_when_preprocess_returns():
     length, width, n = 40_000, 32, 30_000
     p = single(length, width, lr=0.05)
     t, o = p.tables[0], p.oracle
+    assert t.last_times() == (0.0, 0.0)                   # and from now on the calls are timed
     dev = torch.empty(n, dtype=torch.int64, device="cuda")
     host = np.empty(n, np.int64)
     dst = torch.empty((n, width), device="cuda")
