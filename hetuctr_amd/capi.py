@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # HETUCTR_LIB points at another build of the same library (kernel tuning experiments)
 LIB_PATH = os.environ.get("HETUCTR_LIB") or os.path.join(_HERE, "lib", "libhetuctr_hip.so")
 INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
-SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_push_pull", "hctr_group_preprocess",
+SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_preprocess_noalloc", "hctr_push_pull", "hctr_group_preprocess",
            "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch",
            "hctr_stream", "hctr_last_times", "hctr_last_push_ms", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
            "hctr_stage_times", "hctr_copy_probe", "hctr_version", "hctr_part_create", "hctr_part_destroy",
@@ -21,6 +21,7 @@ UNIQUE, SORTED_ARG, RUN_START, IDX_MAP, ROOT, OFFSET, SEND_CNT, RECV_CNT = range
 NEED_UPDATE, UPDATE_PREFIX, PUSH_CNT, PUSHRECV_CNT, OUTDATED, GOT, VERSION, UPDATES = range(8, 16)
 EMBEDDING, PENDING, STORE_IDS, STATS, SIZES, KEYS = range(16, 22)
 FLOAT_ITEMS = (EMBEDDING, PENDING)
+NOALLOC_MAX_KEYS = 262144
 
 
 class Config(C.Structure):
@@ -42,6 +43,7 @@ def lib():
         l.hctr_create.argtypes = [C.POINTER(Config), C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]
         l.hctr_destroy.argtypes = [C.c_void_p]
         l.hctr_preprocess.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        l.hctr_preprocess_noalloc.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         l.hctr_push_pull.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         l.hctr_group_preprocess.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         l.hctr_group_push_pull.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
@@ -109,6 +111,10 @@ class Table:
 
     def preprocess(self, ptr, n):
         _check(lib().hctr_preprocess(self._h, C.c_void_p(int(ptr)), n))
+
+    def preprocess_noalloc(self, ptr, n):
+        """preprocess that allocates nothing (device ids, at most NOALLOC_MAX_KEYS, buffers sized by earlier calls)."""
+        _check(lib().hctr_preprocess_noalloc(self._h, C.c_void_p(int(ptr)), n))
 
     def push_pull(self, grad_ptr, dst_ptr):
         _check(lib().hctr_push_pull(self._h, C.c_void_p(int(grad_ptr) or None), C.c_void_p(int(dst_ptr) or None)))

@@ -92,6 +92,13 @@ int hctr_preprocess(hctr_table *t, const int64_t *keys, size_t n) {
   });
 }
 
+int hctr_preprocess_noalloc(hctr_table *t, const int64_t *keys, size_t n) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->group->preprocess_noalloc(keys, n);
+  });
+}
+
 int hctr_push_pull(hctr_table *t, const float *grad, float *dst) {
   return guarded([&] {
     HCTR_CHECK(t && t->shard, "null table");

@@ -58,6 +58,7 @@ struct Batch {
   std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
   std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
   void reserve(uint32_t n_keys, int nrank, bool wide);
+  bool holds(uint32_t n_keys, int nrank, bool wide) const; // reserve() would not allocate
   void clear(hipStream_t s, int nrank); // make the device side an empty batch; does nothing if it already is
   BatchView view() const;
 };
@@ -110,7 +111,8 @@ class Shard {
     index_batch();
   }
   // the caller's ids -> device copy and sort keys; flag: where the range check reports (default: the device word)
-  void ingest_keys(const int64_t *keys, size_t n, uint32_t *flag = nullptr);
+  // scratch_area (default: the shard's own growable buffers): the index scratch of this batch is cut out of it
+  void ingest_keys(const int64_t *keys, size_t n, uint32_t *flag = nullptr, void *scratch_area = nullptr);
   // sort, unique, run lists of the ingested batch; u_out: where the number of unique keys goes besides the batch's
   // own device word (default: the device block that is read back after the call)
   void index_batch(uint32_t *u_out = nullptr, int part = 0);
@@ -138,6 +140,11 @@ class Shard {
   DeviceBuf root, slot, emb, ver, pend, upd, store_ids;
   // scratch shared by the stages
   DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, sortws, block_sums, dstat, stats;
+  // where the index stages of the current batch find their scratch: the buffers above or pieces of the static array
+  struct ScratchPtrs {
+    void *comp = nullptr, *ktmp0 = nullptr, *ktmp1 = nullptr;
+    uint32_t *vtmp0 = nullptr, *vtmp1 = nullptr, *sortws = nullptr, *block_sums = nullptr;
+  } sp;
   DeviceBuf need, prefix, plan_sums; // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
   DevStat *dst_ = nullptr; // == dstat.p
   uint32_t *err_ptr() const { return &dst_->err; }
@@ -157,7 +164,15 @@ class Shard {
 
  private:
   void reserve_batch_scratch(uint32_t n);
+  void use_scratch_area(void *area, uint32_t n);
 };
+
+// The entry point that allocates nothing takes batches of up to kNoAllocMaxKeys keys; kNoAllocScratchBytes is what
+// the index of such a batch needs with 64-bit sort keys (sort ping-pong buffers, per-tile digit counts, scan sums).
+constexpr size_t kNoAllocMaxKeys = 262144;
+size_t index_scratch_bytes(uint32_t n, bool wide);
+constexpr size_t kNoAllocScratchBytes = 3 * (kNoAllocMaxKeys * 8) + 2 * (kNoAllocMaxKeys * 4) +
+                                        (kNoAllocMaxKeys / kSortTile + 2) * kSortMaxBins * 4 + 4096;
 
 // All shards of one loopback group live in one process on one device and share one stream.  The group
 // carries the collective calls: every shard's thread deposits its arguments, the last one to arrive runs the
@@ -205,6 +220,8 @@ class Group {
 
   // lock-step bodies (one caller)
   void preprocess_all(const int64_t *const *keys, const size_t *n);
+  void preprocess_noalloc(const int64_t *keys, size_t n);
+  void *noalloc_scratch = nullptr;       // device address of this GPU's static scratch array
   void push_pull_all(const float *const *grads, float *const *dsts);
   // per-shard entry points: rendezvous of nrank callers
   void preprocess_one(int rank, const int64_t *keys, size_t n);

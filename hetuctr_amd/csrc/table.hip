@@ -18,6 +18,29 @@ const char *stage_name(int s) {
   return s >= 0 && s < S_COUNT ? names[s] : "?";
 }
 
+// ---- scratch of the entry point that allocates nothing (hctr_preprocess_noalloc) --------------------------------
+// One array per GPU, held from the moment the library is loaded on it until the process ends.  In host code the
+// array's name is only a handle: the device address comes from hipGetSymbolAddress, once per device, and that pointer
+// is what kernels and copies are given.
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+std::mutex g_scratch_mu;
+std::map<int, void *> g_scratch_ptr; // device ordinal -> address of that device's copy of `scratch`
+} // namespace
+
+// address of the current device's copy of the array (dev must be the current device)
+static void *noalloc_scratch_of(int dev) {
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  auto it = g_scratch_ptr.find(dev);
+  if (it != g_scratch_ptr.end()) return it->second;
+  void *ptr = nullptr;
+  HCTR_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+  HCTR_CHECK(ptr != nullptr, "no device address for the static scratch array");
+  g_scratch_ptr[dev] = ptr;
+  return ptr;
+}
+
 static int bits_for(uint64_t max_value) { // bits needed to represent values 0..max_value
   int b = 0;
   while (b < 64 && (max_value >> b)) b++;
@@ -27,6 +50,15 @@ static int bits_for(uint64_t max_value) { // bits needed to represent values 0..
 // ================================================================================================
 // Batch
 // ================================================================================================
+bool Batch::holds(uint32_t n_keys, int nrank, bool wide) const {
+  const size_t n = std::max<uint32_t>(n_keys, 1);
+  return keys.bytes >= n * sizeof(index_t) && sorted_arg.bytes >= n * 4 && rank_sorted.bytes >= n * 4 &&
+         idx_map.bytes >= n * 4 && ukey.bytes >= n * (wide ? 8 : 4) && run_start.bytes >= (n + 1) * 4 &&
+         uoff.bytes >= n * sizeof(slot_t) && bucket_lo.bytes >= (size_t)(nrank + 1) * 4 && dU.bytes >= 4 &&
+         long_list.bytes >= long_list_capacity((uint32_t)n) * sizeof(uint4) * kLongBuckets &&
+         dnlong.bytes >= 4 * kRunCounters && med_list.bytes >= med_list_capacity((uint32_t)n) * 4;
+}
+
 void Batch::reserve(uint32_t n_keys, int nrank, bool wide) {
   const size_t n = std::max<uint32_t>(n_keys, 1);
   keys.reserve(n * sizeof(index_t));
@@ -192,23 +224,57 @@ void Shard::reserve_batch_scratch(uint32_t n) {
   vtmp1.reserve(m * 4);
   sortws.reserve(sort_scratch_words(m) * 4);
   block_sums.reserve((scan_blocks(m) + 2) * 4);
+  sp.comp = comp.p;
+  sp.ktmp0 = ktmp0.p;
+  sp.ktmp1 = ktmp1.p;
+  sp.vtmp0 = vtmp0.as<uint32_t>();
+  sp.vtmp1 = vtmp1.as<uint32_t>();
+  sp.sortws = sortws.as<uint32_t>();
+  sp.block_sums = block_sums.as<uint32_t>();
+}
+
+// bytes of index scratch a batch of n keys needs, every piece a multiple of 256 bytes
+size_t index_scratch_bytes(uint32_t n, bool wide) {
+  const size_t m = std::max<uint32_t>(n, 1), ks = wide ? 8 : 4;
+  auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+  return 3 * up(m * ks) + 2 * up(m * 4) + up(sort_scratch_words(m) * 4) + up((scan_blocks(m) + 2) * 4);
+}
+
+// the same pieces cut out of one caller-provided area (the static array) instead of the shard's own buffers
+void Shard::use_scratch_area(void *area, uint32_t n) {
+  const size_t m = std::max<uint32_t>(n, 1), ks = kl.wide ? 8 : 4;
+  auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+  unsigned char *p = (unsigned char *)area;
+  auto take = [&](size_t bytes) {
+    void *r = p;
+    p += up(bytes);
+    return r;
+  };
+  sp.comp = take(m * ks);
+  sp.ktmp0 = take(m * ks);
+  sp.ktmp1 = take(m * ks);
+  sp.vtmp0 = (uint32_t *)take(m * 4);
+  sp.vtmp1 = (uint32_t *)take(m * 4);
+  sp.sortws = (uint32_t *)take(sort_scratch_words(m) * 4);
+  sp.block_sums = (uint32_t *)take((scan_blocks(m) + 2) * 4);
 }
 
 // csrc/core/preprocess.cu:92-141
-void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag) {
+void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scratch_area) {
   HCTR_CHECK(n < 0xfffffff0ull, "a batch holds fewer than 2^32 keys");
   HCTR_CHECK(keys != nullptr || n == 0, "null key pointer");
   hipStream_t s = group->stream;
   cur.n = (uint32_t)n;
   cur.U = 0;
   cur.idx_map_valid = false;
-  cur.reserve(cur.n, cfg.nrank, kl.wide);
+  if (!scratch_area) cur.reserve(cur.n, cfg.nrank, kl.wide); // else: the caller has checked that the buffers hold n keys
   if (n == 0) { // :93-95
     cur.clear(s, cfg.nrank);
   } else {
     cur.cleared = false;
     u_cleared = false;
-    reserve_batch_scratch(cur.n);
+    if (scratch_area) use_scratch_area(scratch_area, cur.n);
+    else reserve_batch_scratch(cur.n);
     {
       // ids -> device copy (:98-99) and sort keys.  When the caller's pointer is device-visible the copy is
       // written by the same kernel that reads the ids; a pageable host buffer goes through a transfer first.
@@ -218,10 +284,12 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag) {
                            (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged);
       if (!visible) {
         (void)hipGetLastError(); // an unregistered host pointer leaves a sticky "invalid value"
+        HCTR_CHECK(!scratch_area, "preprocess without allocations takes ids in device memory only (a transfer from "
+                                  "pageable host memory is staged by the runtime)");
         HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
       }
-      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, comp.p, flag ? flag : err_ptr(),
-                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), sortws.as<uint32_t>());
+      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, sp.comp, flag ? flag : err_ptr(),
+                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), sp.sortws);
     }
   }
 }
@@ -232,28 +300,28 @@ void Shard::index_batch(uint32_t *u_out, int part) {
   const int from = part == 2 ? kEarlySortSteps : 0, to = part == 1 ? kEarlySortSteps : (1 << 30);
   if (cur.n != 0) {
     SortScratch sc;
-    sc.words = sortws.as<uint32_t>();
+    sc.words = sp.sortws;
     sc.n_cap = cur.n;
     const void *sorted_keys = nullptr;
     {
       StageScope sort_scope(*group, S_SORT);
       if (kl.wide) {
         const uint64_t *sk;
-        radix_sort_positions<uint64_t>(s, comp.as<uint64_t>(), cur.n, kl.total_bits, ktmp0.as<uint64_t>(),
-                                       ktmp1.as<uint64_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
+        radix_sort_positions<uint64_t>(s, (const uint64_t *)sp.comp, cur.n, kl.total_bits, (uint64_t *)sp.ktmp0,
+                                       (uint64_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
                                        cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
         sorted_keys = sk;
       } else {
         const uint32_t *sk;
-        radix_sort_positions<uint32_t>(s, comp.as<uint32_t>(), cur.n, kl.total_bits, ktmp0.as<uint32_t>(),
-                                       ktmp1.as<uint32_t>(), vtmp0.as<uint32_t>(), vtmp1.as<uint32_t>(),
+        radix_sort_positions<uint32_t>(s, (const uint32_t *)sp.comp, cur.n, kl.total_bits, (uint32_t *)sp.ktmp0,
+                                       (uint32_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
                                        cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
         sorted_keys = sk;
       }
     }
     if (part == 1) return;
     StageScope st(*group, S_UNIQUE);
-    launch_unique(s, tv, kl, sorted_keys, cur.view(), block_sums.as<uint32_t>(), u_out ? u_out : &dst_->U);
+    launch_unique(s, tv, kl, sorted_keys, cur.view(), sp.block_sums, u_out ? u_out : &dst_->U);
     launch_list_long_runs(s, cur.view());
   }
   if (part == 1) return;
@@ -584,6 +652,7 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   HCTR_HIP(hipGetDeviceCount(&ndev));
   HCTR_CHECK(dev >= 0 && dev < ndev, "InCorrect device number."); // table_initialize.cu:144-146
   HCTR_HIP(hipSetDevice(dev));
+  noalloc_scratch = noalloc_scratch_of(dev); // this device's copy of the static array, looked up with it current
   // a blocking stream, like the reference's cudaStreamCreate (table_initialize.cu:16): work the caller queued on the
   // legacy default stream (torch's default) is ordered before ours without an explicit synchronisation
   HCTR_HIP(hipStreamCreate(&stream));
@@ -903,6 +972,38 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
   }
   exchange_shapes();
   if (!first_error.empty()) throw Error(first_error);
+}
+
+// hctr_preprocess_noalloc: the literal contract of HetuTable::preprocess (everything done when the call returns) for one
+// shard, with every piece of index scratch taken from the static array and no allocation anywhere on the way.
+void Group::preprocess_noalloc(const int64_t *keys, size_t n) {
+  HCTR_CHECK(nrank == 1, "preprocess without allocations is built for a table of one shard");
+  HCTR_CHECK(n <= kNoAllocMaxKeys, "preprocess without allocations takes at most " + std::to_string(kNoAllocMaxKeys) +
+                                       " keys per batch (the size of its static scratch)");
+  HCTR_CHECK(!stage_timing, "stage timing takes events from a growing pool: switch it off for calls that may not allocate");
+  HCTR_HIP(hipSetDevice(device_id));
+  flush_index(); // an earlier deferred batch is indexed before it becomes the previous one
+  Shard *m = members[0];
+  // after the swap the current batch lives in the buffers of the batch before the previous one
+  HCTR_CHECK(m->prev.holds((uint32_t)n, 1, m->kl.wide),
+             "preprocess without allocations: the table's batch buffers are smaller than this batch; they are sized by "
+             "ordinary hctr_preprocess calls (two in a row size both)");
+  HCTR_CHECK(index_scratch_bytes((uint32_t)n, m->kl.wide) <= kNoAllocScratchBytes, "internal: static scratch too small");
+  if (n) {
+    hipPointerAttribute_t attr;
+    const bool visible = keys != nullptr && hipPointerGetAttributes(&attr, keys) == hipSuccess &&
+                         (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged);
+    if (!visible) (void)hipGetLastError();
+    HCTR_CHECK(visible, "preprocess without allocations takes ids in device memory only (a transfer from pageable "
+                        "host memory is staged by the runtime)");
+  }
+  m->swap_batches();
+  m->ingest_keys(keys, n, nullptr, noalloc_scratch);
+  m->index_batch();
+  m->enqueue_readback_preprocess();
+  sync_stream();
+  m->finish_preprocess();
+  exchange_shapes();
 }
 
 // all2allExchangeShape, csrc/core/all2all.cu:6-16

@@ -57,6 +57,19 @@ int hctr_destroy(hctr_table *t);
  * Synchronous.  With nrank > 1 the call completes when every shard of the group has made it. */
 int hctr_preprocess(hctr_table *t, const int64_t *keys, size_t n);
 
+/* hctr_preprocess for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same result as hctr_preprocess, and like the
+ * reference's call it returns when all its work is done; it calls no hipMalloc / hipFree and no allocating routine:
+ *   - the index scratch (sort ping-pong buffers, per-tile digit counts, scan sums) lives in a static device array of
+ *     8.3 MiB that every GPU the library runs on holds until the process ends;
+ *   - n is at most 262144 keys (HCTR_NOALLOC_MAX_KEYS), larger batches are refused;
+ *   - keys must be DEVICE memory (a transfer from pageable host memory is staged by the runtime);
+ *   - the table has one shard, and its two batch buffers already hold n keys: they are sized by ordinary
+ *     hctr_preprocess calls (two in a row with the largest batch size both); otherwise the call is refused.
+ * All tables on one GPU share that GPU's array: calls that overlap on one GPU race. */
+#define HCTR_NOALLOC_MAX_KEYS 262144
+int hctr_preprocess_noalloc(hctr_table *t, const int64_t *keys, size_t n);
+
 /* Replaces HetuTable::pushPull (csrc/core/hetu_gpu_table.cu:9-41).  grad: DEVICE float[n_prev][width]
  * for the batch before the current one, or NULL (inference: nothing is pushed).  dst: DEVICE
  * float[n][width] receives the rows of the current batch.  Synchronous. */
