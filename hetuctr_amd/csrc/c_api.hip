@@ -181,13 +181,7 @@ int hctr_last_push_ms(hctr_table *t, float *push_ms) {
 int hctr_stage_timing(hctr_table *t, int on) {
   return guarded([&] {
     HCTR_CHECK(t && t->shard, "null table");
-    Group &g = *t->shard->group;
-    g.flush_index();
-    g.stage_timing = on != 0;
-    for (int i = 0; i < S_COUNT; i++) {
-      g.stage_ms[i] = 0;
-      g.stage_calls[i] = 0;
-    }
+    t->shard->group->set_stage_timing(on != 0);
   });
 }
 

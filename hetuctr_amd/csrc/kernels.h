@@ -17,7 +17,6 @@ struct KeyLayout {
 // csrc/core/preprocess_struct.h:7-24, with 32-bit positions and ranks).
 struct BatchView {
   uint32_t n;                // keys in the batch (host-known)
-  const index_t *keys;       // [n]   the ids as handed in                      (d_idx)
   uint32_t *sorted_arg;      // [n]   positions grouped by unique key, stable   (d_sorted_arg)
   uint32_t *rank_sorted;     // [n]   unique rank of sorted position j
   uint32_t *idx_map;         // [n]   unique rank of position i, filled on request only    (d_idx_map)
@@ -75,10 +74,10 @@ struct TableView {
 
 // ---- preprocess ---------------------------------------------------------------------------------
 // ids -> sort keys; flags ids outside [0, id_max) in *err (and sorts them as id 0)
-// keys_copy (optional): the ids are also copied there (the reference's d_idx); nlong (optional) is zeroed;
+// comp_keys is the batch's copy of the ids as well (the reference's d_idx); nlong (optional) is zeroed;
 // sort_counts: the sort's scratch, which receives the per-tile counts of the first pass' digit
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong, uint32_t *sort_counts);
+                      void *comp_keys, uint32_t *err, uint32_t *nlong, uint32_t *sort_counts);
 // sorted keys -> everything per unique key + inverse index.  block_heads: scratch of scan_blocks(n) words.
 // u_copy (optional) receives the number of unique keys as well (b.d_U always does)
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,

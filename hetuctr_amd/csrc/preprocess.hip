@@ -13,16 +13,16 @@ constexpr int kBlock = 256;
 constexpr int kItems = 8;
 constexpr int kTile = kBlock * kItems; // 2048: scan_blocks(n) sizes the scratch
 
-// ids -> sort keys (owner << id_bits | id), the copy of the ids, the range check, the reset of the batch's run
-// counters, and the per-tile counts of the first sort pass' digit: a block works on one sort tile, so the sort
+// ids -> sort keys (owner << id_bits | id; they are the batch's copy of the ids as well), the range check, the reset
+// of the batch's run counters, and the per-tile counts of the first sort pass' digit: a block works on one sort tile, so the sort
 // needs no counting launch of its own for that pass.  This is the one kernel that reads the caller's buffer: the
 // call may return when it is through.
 template <typename K>
 __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
                                                          int id_bits, int nrank, const worker_t *__restrict__ root,
                                                          K *__restrict__ comp, uint32_t *__restrict__ err,
-                                                         index_t *__restrict__ keys_copy, uint32_t *__restrict__ nlong,
-                                                         int dbits, uint32_t *__restrict__ counts) {
+                                                         uint32_t *__restrict__ nlong, int dbits,
+                                                         uint32_t *__restrict__ counts) {
   __shared__ uint32_t h[kSortMaxBins];
   const uint32_t nb = 1u << dbits, mask = nb - 1;
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
@@ -39,9 +39,7 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
 #pragma unroll
   for (int k = 0; k < kSortItems; k++) {
     const uint32_t i = base + k * kSortBlock + threadIdx.x;
-    if (i >= n) continue;
-    if (keys_copy) __builtin_nontemporal_store((index_t)id[k], &keys_copy[i]); // only read back on request
-    if (id[k] >= id_max) { // also catches negative ids
+    if (i < n && id[k] >= id_max) { // also catches negative ids
       bad = true;
       id[k] = 0;
     }
@@ -287,16 +285,16 @@ __global__ void bucket_sizes(BatchView b, int nrank, uint64_t *__restrict__ cnt_
 } // namespace
 
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err, index_t *keys_copy, uint32_t *nlong, uint32_t *sort_counts) {
+                      void *comp_keys, uint32_t *err, uint32_t *nlong, uint32_t *sort_counts) {
   if (!n) return;
   const unsigned nblocks = (unsigned)sort_tiles(n);
   const int dbits = sort_first_digit_bits(kl.total_bits);
   if (kl.wide)
     hipLaunchKernelGGL(make_keys<uint64_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
-                       t.root, (uint64_t *)comp_keys, err, keys_copy, nlong, dbits, sort_counts);
+                       t.root, (uint64_t *)comp_keys, err, nlong, dbits, sort_counts);
   else
     hipLaunchKernelGGL(make_keys<uint32_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
-                       t.root, (uint32_t *)comp_keys, err, keys_copy, nlong, dbits, sort_counts);
+                       t.root, (uint32_t *)comp_keys, err, nlong, dbits, sort_counts);
   HCTR_HIP(hipGetLastError());
 }
 

@@ -54,7 +54,9 @@ struct Batch {
   uint32_t U = 0;   // unique keys (host copy, valid after the preprocess call returned)
   bool idx_map_valid = false;
   bool cleared = false; // the device side reads as an empty batch (U = 0, no buckets, no runs) since clear()
-  DeviceBuf keys, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong, med_list;
+  // comp: the batch's sort keys in batch order (id and owner of every position); staged: ids that arrived in
+  // pageable host memory, on their way to the key kernel
+  DeviceBuf comp, staged, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong, med_list;
   std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
   std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
   void reserve(uint32_t n_keys, int nrank, bool wide);
@@ -139,10 +141,10 @@ class Shard {
   bool prev_active = false; // false: inference step or no previous batch, nothing is pushed
   DeviceBuf root, slot, emb, ver, pend, upd, store_ids;
   // scratch shared by the stages
-  DeviceBuf comp, ktmp0, ktmp1, vtmp0, vtmp1, sortws, block_sums, dstat, stats;
+  DeviceBuf ktmp0, ktmp1, vtmp0, vtmp1, sortws, block_sums, dstat, stats;
   // where the index stages of the current batch find their scratch: the buffers above or pieces of the static array
   struct ScratchPtrs {
-    void *comp = nullptr, *ktmp0 = nullptr, *ktmp1 = nullptr;
+    void *ktmp0 = nullptr, *ktmp1 = nullptr;
     uint32_t *vtmp0 = nullptr, *vtmp1 = nullptr, *sortws = nullptr, *block_sums = nullptr;
   } sp;
   DeviceBuf need, prefix, plan_sums; // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
@@ -171,7 +173,7 @@ class Shard {
 // the index of such a batch needs with 64-bit sort keys (sort ping-pong buffers, per-tile digit counts, scan sums).
 constexpr size_t kNoAllocMaxKeys = 262144;
 size_t index_scratch_bytes(uint32_t n, bool wide);
-constexpr size_t kNoAllocScratchBytes = 3 * (kNoAllocMaxKeys * 8) + 2 * (kNoAllocMaxKeys * 4) +
+constexpr size_t kNoAllocScratchBytes = 2 * (kNoAllocMaxKeys * 8) + 2 * (kNoAllocMaxKeys * 4) +
                                         (kNoAllocMaxKeys / kSortTile + 2) * kSortMaxBins * 4 + 4096;
 
 // All shards of one loopback group live in one process on one device and share one stream.  The group
@@ -213,6 +215,7 @@ class Group {
   std::vector<hipEvent_t> event_pool;
   hipEvent_t take_event();
   void collect_marks();                  // after a stream sync
+  void set_stage_timing(bool on);        // resets the accumulators; waits for a pending index under the group's lock
 
   void join(Shard *s);
   void leave(Shard *s);

@@ -52,7 +52,7 @@ static int bits_for(uint64_t max_value) { // bits needed to represent values 0..
 // ================================================================================================
 bool Batch::holds(uint32_t n_keys, int nrank, bool wide) const {
   const size_t n = std::max<uint32_t>(n_keys, 1);
-  return keys.bytes >= n * sizeof(index_t) && sorted_arg.bytes >= n * 4 && rank_sorted.bytes >= n * 4 &&
+  return comp.bytes >= n * (wide ? 8 : 4) && sorted_arg.bytes >= n * 4 && rank_sorted.bytes >= n * 4 &&
          idx_map.bytes >= n * 4 && ukey.bytes >= n * (wide ? 8 : 4) && run_start.bytes >= (n + 1) * 4 &&
          uoff.bytes >= n * sizeof(slot_t) && bucket_lo.bytes >= (size_t)(nrank + 1) * 4 && dU.bytes >= 4 &&
          long_list.bytes >= long_list_capacity((uint32_t)n) * sizeof(uint4) * kLongBuckets &&
@@ -61,7 +61,7 @@ bool Batch::holds(uint32_t n_keys, int nrank, bool wide) const {
 
 void Batch::reserve(uint32_t n_keys, int nrank, bool wide) {
   const size_t n = std::max<uint32_t>(n_keys, 1);
-  keys.reserve(n * sizeof(index_t));
+  comp.reserve(n * (wide ? 8 : 4));
   sorted_arg.reserve(n * 4);
   rank_sorted.reserve(n * 4);
   idx_map.reserve(n * 4);
@@ -88,7 +88,6 @@ void Batch::clear(hipStream_t s, int nrank) {
 BatchView Batch::view() const {
   BatchView v;
   v.n = n;
-  v.keys = keys.as<index_t>();
   v.sorted_arg = sorted_arg.as<uint32_t>();
   v.rank_sorted = rank_sorted.as<uint32_t>();
   v.idx_map = idx_map.as<uint32_t>();
@@ -217,14 +216,12 @@ Shard::~Shard() {
 void Shard::reserve_batch_scratch(uint32_t n) {
   const size_t m = std::max<uint32_t>(n, 1);
   const size_t ks = kl.wide ? 8 : 4;
-  comp.reserve(m * ks);
   ktmp0.reserve(m * ks);
   ktmp1.reserve(m * ks);
   vtmp0.reserve(m * 4);
   vtmp1.reserve(m * 4);
   sortws.reserve(sort_scratch_words(m) * 4);
   block_sums.reserve((scan_blocks(m) + 2) * 4);
-  sp.comp = comp.p;
   sp.ktmp0 = ktmp0.p;
   sp.ktmp1 = ktmp1.p;
   sp.vtmp0 = vtmp0.as<uint32_t>();
@@ -237,7 +234,7 @@ void Shard::reserve_batch_scratch(uint32_t n) {
 size_t index_scratch_bytes(uint32_t n, bool wide) {
   const size_t m = std::max<uint32_t>(n, 1), ks = wide ? 8 : 4;
   auto up = [](size_t b) { return (b + 255) / 256 * 256; };
-  return 3 * up(m * ks) + 2 * up(m * 4) + up(sort_scratch_words(m) * 4) + up((scan_blocks(m) + 2) * 4);
+  return 2 * up(m * ks) + 2 * up(m * 4) + up(sort_scratch_words(m) * 4) + up((scan_blocks(m) + 2) * 4);
 }
 
 // the same pieces cut out of one caller-provided area (the static array) instead of the shard's own buffers
@@ -250,7 +247,6 @@ void Shard::use_scratch_area(void *area, uint32_t n) {
     p += up(bytes);
     return r;
   };
-  sp.comp = take(m * ks);
   sp.ktmp0 = take(m * ks);
   sp.ktmp1 = take(m * ks);
   sp.vtmp0 = (uint32_t *)take(m * 4);
@@ -286,10 +282,11 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
         (void)hipGetLastError(); // an unregistered host pointer leaves a sticky "invalid value"
         HCTR_CHECK(!scratch_area, "preprocess without allocations takes ids in device memory only (a transfer from "
                                   "pageable host memory is staged by the runtime)");
-        HCTR_HIP(hipMemcpyAsync(cur.keys.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
+        cur.staged.reserve(n * sizeof(index_t));
+        HCTR_HIP(hipMemcpyAsync(cur.staged.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
       }
-      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.keys.as<index_t>(), cur.n, sp.comp, flag ? flag : err_ptr(),
-                       visible ? cur.keys.as<index_t>() : nullptr, cur.dnlong.as<uint32_t>(), sp.sortws);
+      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.staged.as<index_t>(), cur.n,
+                       cur.comp.p, flag ? flag : err_ptr(), cur.dnlong.as<uint32_t>(), sp.sortws);
     }
   }
 }
@@ -307,13 +304,13 @@ void Shard::index_batch(uint32_t *u_out, int part) {
       StageScope sort_scope(*group, S_SORT);
       if (kl.wide) {
         const uint64_t *sk;
-        radix_sort_positions<uint64_t>(s, (const uint64_t *)sp.comp, cur.n, kl.total_bits, (uint64_t *)sp.ktmp0,
+        radix_sort_positions<uint64_t>(s, cur.comp.as<uint64_t>(), cur.n, kl.total_bits, (uint64_t *)sp.ktmp0,
                                        (uint64_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
                                        cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
         sorted_keys = sk;
       } else {
         const uint32_t *sk;
-        radix_sort_positions<uint32_t>(s, (const uint32_t *)sp.comp, cur.n, kl.total_bits, (uint32_t *)sp.ktmp0,
+        radix_sort_positions<uint32_t>(s, cur.comp.as<uint32_t>(), cur.n, kl.total_bits, (uint32_t *)sp.ktmp0,
                                        (uint32_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
                                        cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
         sorted_keys = sk;
@@ -451,8 +448,8 @@ void Shard::generate_gradient(const float *grad) {
 void Shard::generate_query() {
   if (cfg.nrank == 1) return; // a shard never finds its own rows outdated (handle_query.cu:47-54)
   hipStream_t s = group->stream;
-  q_idx.reserve(std::max<uint32_t>(cur.U, 1) * sizeof(index_t));
-  q_ver.reserve(std::max<uint32_t>(cur.U, 1) * sizeof(version_t));
+  q_idx.reserve((size_t)std::max<uint32_t>(cur.U, 1) * sizeof(index_t));
+  q_ver.reserve((size_t)std::max<uint32_t>(cur.U, 1) * sizeof(version_t));
   StageScope st(*group, S_QUERY);
   launch_lookup_version(s, tv, cur.view(), q_ver.as<version_t>());
   launch_unique_ids(s, kl, cur.view(), q_idx.as<index_t>());
@@ -487,9 +484,9 @@ void Shard::handle_query() {
   hipStream_t s = group->stream;
   const int R = cfg.nrank;
   const uint32_t Q = (uint32_t)rq_seg[R];
-  outdated.reserve(std::max<uint32_t>(Q, 1) * 4);
-  out_pos.reserve(std::max<uint32_t>(Q, 1) * 4);
-  ret_ver.reserve(std::max<uint32_t>(Q, 1) * sizeof(version_t));
+  outdated.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
+  out_pos.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
+  ret_ver.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(version_t));
   ret_val.reserve((size_t)std::max<uint32_t>(Q, 1) * cfg.width * sizeof(embed_t));
   reserve_batch_scratch(Q);
   StageScope st(*group, S_OWNER);
@@ -533,7 +530,7 @@ void Shard::write_back(float *dst) {
   // distinct keys, where the gather reads as many rows as it writes; the previous batch is the predictor.
   a.stream_stores = !(prev.n != 0 && (double)prev.U >= 0.9 * (double)prev.n);
   if (cfg.nrank > 1) {
-    ret_i.reserve(std::max<uint32_t>(cur.U, 1) * 4);
+    ret_i.reserve((size_t)std::max<uint32_t>(cur.U, 1) * 4);
     reserve_batch_scratch(cur.U);
     StageScope st(*group, S_REFRESH);
     HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
@@ -626,7 +623,17 @@ size_t Shard::fetch(int which, void *out, size_t cap) {
     case HCTR_F_VERSION: return put64(download<version_t>(ver.p, tv.n_stored), tv.n_stored, out, cap);
     case HCTR_F_UPDATES: return put64(download<version_t>(upd.p, tv.n_cached), tv.n_cached, out, cap);
     case HCTR_F_STORE_IDS: return put64(download<index_t>(store_ids.p, tv.n_stored), tv.n_stored, out, cap);
-    case HCTR_F_KEYS: return put64(download<index_t>(cur.keys.p, cur.n), cur.n, out, cap);
+    case HCTR_F_KEYS: { // the ids of the batch as its sort keys hold them (an id outside the table reads as 0)
+      std::vector<uint64_t> k(cur.n);
+      if (kl.wide) {
+        auto h = download<uint64_t>(cur.comp.p, cur.n);
+        for (size_t i = 0; i < cur.n; i++) k[i] = h[i] & id_mask;
+      } else {
+        auto h = download<uint32_t>(cur.comp.p, cur.n);
+        for (size_t i = 0; i < cur.n; i++) k[i] = h[i] & id_mask;
+      }
+      return put64(k, cur.n, out, cap);
+    }
     case HCTR_F_EMBEDDING:
     case HCTR_F_PENDING: {
       const size_t n = (size_t)(which == HCTR_F_EMBEDDING ? tv.n_stored : tv.n_cached) * tv.width;
@@ -692,12 +699,20 @@ void Group::join(Shard *s) {
 
 void Group::leave(Shard *s) {
   std::lock_guard<std::mutex> lk(mu_);
-  if (members[s->cfg.rank] == s) members[s->cfg.rank] = nullptr;
-  if (index_pending || index_rest_pending) { // the shard's buffers are about to be freed: nothing of it may still be running
+  // The shard's buffers are about to be freed: nothing of it may still be running, and what a deferred preprocess
+  // left behind is taken over while every member is still there (the survivors of a group keep the sizes of their
+  // current batches; the group itself cannot step again without the rank that leaves).
+  if (index_pending || index_rest_pending) {
+    try {
+      if (complete()) flush_index();
+    } catch (const std::exception &) {
+      // a bad key of the abandoned batch: nobody is left to report it to
+    }
     index_pending = false;
     index_rest_pending = false;
     (void)hipStreamSynchronize(index_stream);
   }
+  if (members[s->cfg.rank] == s) members[s->cfg.rank] = nullptr;
 }
 
 bool Group::complete() const {
@@ -728,6 +743,16 @@ void Group::collect_marks() {
     event_pool.push_back(m.b);
   }
   marks.clear();
+}
+
+void Group::set_stage_timing(bool on) {
+  std::lock_guard<std::mutex> lk(mu_); // not while the ranks of the group are inside a collective call
+  flush_index();
+  stage_timing = on;
+  for (int i = 0; i < S_COUNT; i++) {
+    stage_ms[i] = 0;
+    stage_calls[i] = 0;
+  }
 }
 
 void Group::run_copies(std::vector<CopyDesc> &descs) {
@@ -805,7 +830,7 @@ void Group::exchange_return() {
     uint64_t rows = 0;
     for (int d = 0; d < R; d++) rows += members[d]->ret_seg[s + 1] - members[d]->ret_seg[s];
     req.in_rows = rows;
-    req.got.reserve(std::max<uint32_t>(req.cur.U, 1) * 4);
+    req.got.reserve((size_t)std::max<uint32_t>(req.cur.U, 1) * 4);
     req.in_ver.reserve(std::max<uint64_t>(rows, 1) * sizeof(version_t));
     req.in_val.reserve(std::max<uint64_t>(rows, 1) * W * sizeof(embed_t));
     uint64_t uoff = 0, roff = 0;
