@@ -10,9 +10,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("HETUCTR_LIB") or os.path.join(_HERE, "lib", "libhetuctr_hip.so")
 INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
 SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_preprocess_noalloc", "hctr_push_pull", "hctr_group_preprocess",
-           "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch",
+           "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch", "hctr_save", "hctr_load",
            "hctr_stream", "hctr_last_times", "hctr_last_push_ms", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
-           "hctr_stage_times", "hctr_copy_probe", "hctr_version", "hctr_part_create", "hctr_part_destroy",
+           "hctr_stage_times", "hctr_copy_probe", "hctr_sample_rows", "hctr_version", "hctr_part_create", "hctr_part_destroy",
            "hctr_part_sizes", "hctr_part_refine_data", "hctr_part_refine_embed", "hctr_part_get_communication",
            "hctr_part_get_priority", "hctr_part_get_result", "hctr_part_get_counts", "hctr_part_cache_lists"]
 
@@ -54,6 +54,8 @@ def lib():
         l.hctr_last_error.restype = C.c_char_p
         l.hctr_version.restype = C.c_char_p
         l.hctr_debug_fetch.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t)]
+        l.hctr_save.argtypes = [C.c_void_p, C.c_char_p]
+        l.hctr_load.argtypes = [C.c_void_p, C.c_char_p]
         l.hctr_stream.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         l.hctr_last_times.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
         l.hctr_last_push_ms.argtypes = [C.c_void_p, C.POINTER(C.c_float)]
@@ -62,6 +64,7 @@ def lib():
         l.hctr_stage_name.restype = C.c_char_p
         l.hctr_stage_times.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
         l.hctr_copy_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+        l.hctr_sample_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]
         l.hctr_part_create.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_uint,
                                        C.POINTER(C.c_void_p)]
         l.hctr_part_sizes.argtypes = [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_int)]
@@ -90,6 +93,11 @@ def copy_probe(dst_ptr, src_ptr, nbytes, repeats=5):
     ms = C.c_float(0)
     _check(lib().hctr_copy_probe(dst_ptr, src_ptr, nbytes, repeats, C.byref(ms)))
     return ms.value
+
+
+def sample_rows(log_ptr, n_samples, n_fields, rows_ptr, n_rows, out_ptr):
+    """out[r * n_fields + f] = log[rows[r] * n_fields + f] on the device (all pointers device memory)."""
+    _check(lib().hctr_sample_rows(log_ptr, n_samples, n_fields, rows_ptr, n_rows, out_ptr))
 
 
 class Table:
@@ -125,6 +133,14 @@ class Table:
         out = np.empty(n.value, dtype=np.float32 if which in FLOAT_ITEMS else np.int64)
         _check(lib().hctr_debug_fetch(self._h, which, out.ctypes.data, n.value, C.byref(n)))
         return out
+
+    def save(self, path):
+        """Rows, versions, pending gradients and update counters of this shard to one file."""
+        _check(lib().hctr_save(self._h, os.fsencode(path)))
+
+    def load(self, path):
+        """Restores what save() wrote into a table of the same configuration; its batches start empty."""
+        _check(lib().hctr_load(self._h, os.fsencode(path)))
 
     def stream(self):
         s = C.c_void_p()

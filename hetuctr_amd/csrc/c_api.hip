@@ -154,6 +154,20 @@ int hctr_debug_fetch(hctr_table *t, int which, void *host_out, size_t cap_elems,
   });
 }
 
+int hctr_save(hctr_table *t, const char *path) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->save(path);
+  });
+}
+
+int hctr_load(hctr_table *t, const char *path) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->load(path);
+  });
+}
+
 int hctr_stream(hctr_table *t, void **stream_out) {
   return guarded([&] {
     HCTR_CHECK(t && t->shard && stream_out, "null argument");
@@ -215,6 +229,30 @@ int hctr_copy_probe(void *dst, const void *src, size_t bytes, int repeats, float
     if (ms_avg) *ms_avg = ms / repeats;
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
+  });
+}
+
+int hctr_sample_rows(const int64_t *log, size_t n_samples, size_t n_fields, const int64_t *rows, size_t n_rows,
+                     int64_t *keys_out) {
+  return guarded([&] {
+    HCTR_CHECK(n_rows == 0 || (log && rows && keys_out), "null argument");
+    HCTR_CHECK(n_fields >= 1 && n_fields < (1u << 20), "fields out of range");
+    if (!n_rows) return;
+    uint32_t *err = nullptr;
+    HCTR_HIP(hipMalloc((void **)&err, 4));
+    uint32_t h = 0;
+    hipError_t e = hipMemsetAsync(err, 0, 4, nullptr);
+    try {
+      HCTR_HIP(e);
+      launch_sample_rows(nullptr, (const index_t *)log, n_samples, (uint32_t)n_fields, (const index_t *)rows, n_rows,
+                         (index_t *)keys_out, err);
+      HCTR_HIP(hipMemcpy(&h, err, 4, hipMemcpyDeviceToHost)); // waits for the kernel
+    } catch (...) {
+      (void)hipFree(err);
+      throw;
+    }
+    (void)hipFree(err);
+    HCTR_CHECK(h == 0, "sample_rows: a row number lies outside [0, n_samples) (its ids were written as 0)");
   });
 }
 

@@ -148,5 +148,8 @@ void launch_build_directory(hipStream_t s, const index_t *store_ids, uint32_t n_
 struct CopyDesc { const void *src; void *dst; size_t bytes; };
 void launch_copies(hipStream_t s, const CopyDesc *descs_device, uint32_t n, size_t max_bytes);
 void launch_plain_copy(hipStream_t s, const void *src, void *dst, size_t bytes); // bytes % 16 == 0
+// keys_out[r * fields + f] = log[rows[r] * fields + f]; a row number outside [0, n_samples) sets bit 0 of *err
+void launch_sample_rows(hipStream_t s, const index_t *log, uint64_t n_samples, uint32_t fields, const index_t *rows,
+                        uint64_t n_rows, index_t *keys_out, uint32_t *err);
 
 } // namespace hctr

@@ -136,6 +136,9 @@ class Shard {
   void finish_push_pull();
 
   size_t fetch(int which, void *host_out, size_t cap);
+  // rows, versions, pending gradients and update counters to / from one file (checkpoint.hip)
+  void save(const char *path);
+  void load(const char *path);
 
   Batch cur, prev;
   bool prev_active = false; // false: inference step or no previous batch, nothing is pushed

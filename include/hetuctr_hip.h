@@ -107,6 +107,16 @@ enum {
 };
 int hctr_debug_fetch(hctr_table *t, int which, void *host_out, size_t cap_elems, size_t *n_elems);
 
+/* Checkpoint of one shard.  No counterpart in the reference, whose table state lives in device memory only
+ * (csrc/core/hetu_gpu_table.h:38-70, freed in csrc/core/table_initialize.cu:231-245).  hctr_save writes the resident
+ * rows, their versions and, for cached rows, the pending gradients and update counters to `path` (one file per
+ * shard; format in hetuctr_amd/csrc/checkpoint.hip).  hctr_load restores them into a table created with the same
+ * rank, nrank, length, width, root_arr and storage_arr (checked; bounds and learning rate are the new table's) and
+ * empties its two batches: the next hctr_push_pull pushes nothing, as after hctr_create.  Call both between steps,
+ * from every shard of a group. */
+int hctr_save(hctr_table *t, const char *path);
+int hctr_load(hctr_table *t, const char *path);
+
 /* The HIP stream (hipStream_t) every kernel of this table's group is launched on, for callers that time
  * or order work against it (the reference's stream_main_, csrc/core/hetu_gpu_table.h:40). */
 int hctr_stream(hctr_table *t, void **stream_out);
@@ -142,6 +152,13 @@ int hctr_stage_times(hctr_table *t, double *ms_total, long long *launches, int c
  * plain 16-byte-lane kernel on the default stream, 1 + repeats times, and reports the average duration.  A launch
  * reads and writes exactly `bytes`, which is what hardware byte counters are scaled against. */
 int hctr_copy_probe(void *dst, const void *src, size_t bytes, int repeats, float *ms_avg);
+
+/* Batch sampling from a click log in device memory: keys_out[r * n_fields + f] = log[rows[r] * n_fields + f], i.e.
+ * data[idx].flatten() of the reference's benchmark driver (tests/benchmark.py:19-23) for an int64 log of
+ * n_samples x n_fields ids (the array its Criteo loader returns, tests/benchmark.py:26-31).  All three pointers are
+ * DEVICE memory; runs on the default stream and returns when the ids are written, ready for hctr_preprocess. */
+int hctr_sample_rows(const int64_t *log, size_t n_samples, size_t n_fields, const int64_t *rows, size_t n_rows,
+                     int64_t *keys_out);
 
 /* ---- offline partitioner ---------------------------------------------------------------------------------------
  * The C surface under the python module hetuCTR_partition (csrc/partition/pybind.cc:6-25).  Results are those of the
