@@ -34,6 +34,10 @@ def parse():
     ap.add_argument("--no-stage-timing", action="store_true")
     ap.add_argument("--host-keys", action="store_true",
                     help="hand the ids over as pageable host buffers (adds their transfer to the step)")
+    ap.add_argument("--pooled", action="store_true",
+                    help="multi-hot configs: sum-pool every bag of `hot` ids (hctr_push_pull_pooled): one gradient row "
+                         "and one output row per bag instead of per id")
+    ap.add_argument("--bag", type=int, default=0, help="--pooled: bag size (default: the config's ids per field)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the library's plain 1 GiB copy kernel (scale factor of the HBM byte counters)")
     ap.add_argument("--active-peers", action="store_true",
@@ -356,8 +360,9 @@ def main():
     dkeys = [torch.from_numpy(b).cuda() for b in batches]
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
-    grad = torch.randn((n, width), device="cuda", generator=gen) * 1e-3
-    dst = torch.empty((n, width), device="cuda")
+    bag = (a.bag or ks.hot) if a.pooled else 1       # sum-pooled bags: one gradient / output row per bag
+    grad = torch.randn((n // bag, width), device="cuda", generator=gen) * 1e-3
+    dst = torch.empty((n // bag, width), device="cuda")
     torch.cuda.synchronize()
     print("[bench] table + inputs resident in HBM after %.1fs" % (time.perf_counter() - t_init), file=sys.stderr, flush=True)
 
@@ -365,9 +370,14 @@ def main():
     # includes their transfer (never the reported headline: `value` is quoted with the ids resident in HBM)
     key_ptr = [b.ctypes.data for b in batches] if a.host_keys else [d.data_ptr() for d in dkeys]
 
-    def step(i):
-        table.preprocess(key_ptr[i % len(dkeys)], n)
-        table.push_pull(grad.data_ptr(), dst.data_ptr())
+    if bag > 1:
+        def step(i):
+            table.preprocess(key_ptr[i % len(dkeys)], n)
+            table.push_pull_pooled(grad.data_ptr(), dst.data_ptr(), bag)
+    else:
+        def step(i):
+            table.preprocess(key_ptr[i % len(dkeys)], n)
+            table.push_pull(grad.data_ptr(), dst.data_ptr())
 
     uniq = {}
     for i in range(max(a.warmup, 1)):
@@ -377,7 +387,7 @@ def main():
         if i not in uniq:
             table.preprocess(dkeys[i].data_ptr(), n)
             uniq[i] = int(table.fetch(capi.SIZES)[1])
-            table.push_pull(grad.data_ptr(), dst.data_ptr())
+            table.push_pull_pooled(grad.data_ptr(), dst.data_ptr(), bag)
     w0 = max(a.warmup, 1) + len(dkeys)
     # ---- timed region: K full steps, nothing else on the GPU and nothing but the two calls on the host
     torch.cuda.synchronize()
@@ -415,7 +425,7 @@ def main():
     # distinct keys of the batches the timed steps used (current batch = pulled, previous = pushed)
     u_cur = np.mean([uniq[(w0 + i) % len(dkeys)] for i in range(a.steps)])
     u_prev = np.mean([uniq[(w0 + i - 1) % len(dkeys)] for i in range(a.steps)])
-    bytes_step = workloads.algorithmic_bytes(n, 0.5 * (u_cur + u_prev), width)
+    bytes_step = workloads.algorithmic_bytes(n, 0.5 * (u_cur + u_prev), width, bag)
     step_gbs = bytes_step / (ms_step * 1e-3) / 1e9
 
     # HBM traffic per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (committed
@@ -429,7 +439,7 @@ def main():
     for k, (tot, cnt) in stages.items():
         if k in kernel_names and cnt > 0:
             avg_ms = tot / cnt
-            b = workloads.stage_bytes(k, n, u_cur, n, u_prev, width)
+            b = workloads.stage_bytes(k, n, u_cur, n, u_prev, width, bag)
             gbs = b / (avg_ms * 1e-3) / 1e9
             roof_all[k] = dict(bound="hbm", kernel=kernel_names[k], achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s",
                                frac=gbs / HBM_PEAK_GBS, traffic=traffic.get(k), avg_ms=avg_ms, algorithmic_bytes=int(b))
@@ -452,15 +462,22 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: %d-row x %d fp32 table, batch %d samples x %d fields x %d ids = %d keys, %s, "
-                               "SGD lr %g, one shard (all rows local)" %
+                               "SGD lr %g, one shard (all rows local)%s" %
                                (a.config, ks.rows, width, ks.samples, ks.fields, ks.hot, n,
-                                "uniform ids" if cfg["alpha"] is None else "per-field Zipf %.2f" % cfg["alpha"], lr),
+                                "uniform ids" if cfg["alpha"] is None else "per-field Zipf %.2f" % cfg["alpha"], lr,
+                                "" if bag == 1 else ", bags of %d ids sum-pooled" % bag),
                    "keys_per_step": n, "unique_keys_per_step": float(u_cur), "width": width, "rows": ks.rows,
                    "ids_handed_over_in": "pageable host memory" if a.host_keys else "HBM"},
         "unique_rows_per_sec": u_cur * a.steps / dt,
         "device_ms_per_step": {"preprocess_until_ids_are_read": pre_ms / a.steps, "push_pull": pp_ms / a.steps},
         "step_hbm": {"algorithmic_bytes": int(bytes_step), "achieved_GBps": step_gbs, "frac": step_gbs / HBM_PEAK_GBS},
         "stage_ms": {k: v[0] / max(v[1], 1) for k, v in stages.items() if v[1]},
+        "pooling": None if bag == 1 else {
+            "bag": bag, "gradient_rows_per_step": n // bag, "output_rows_per_step": n // bag,
+            "unpooled_output_bytes": 4 * width * n, "pooled_output_bytes": 4 * width * (n // bag),
+            "bytes_saved_per_step": 2 * 4 * width * (n - n // bag),
+            "note": "the reference hands one row per id both ways (its API has no pooling); pooled, the gradient and "
+                    "the output shrink by the bag size, the table rows read per id stay"},
         "ms_per_step_with_stage_events": ms_step_ev,
         "roofline": roof,
         "roofline_stages": roof_all,

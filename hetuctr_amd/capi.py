@@ -9,8 +9,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # HETUCTR_LIB points at another build of the same library (kernel tuning experiments)
 LIB_PATH = os.environ.get("HETUCTR_LIB") or os.path.join(_HERE, "lib", "libhetuctr_hip.so")
 INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
-SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_preprocess_noalloc", "hctr_push_pull", "hctr_group_preprocess",
-           "hctr_group_push_pull", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch", "hctr_save", "hctr_load",
+SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_preprocess_noalloc", "hctr_push_pull", "hctr_push_pull_pooled",
+           "hctr_group_preprocess", "hctr_group_push_pull", "hctr_group_push_pull_pooled", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch", "hctr_save", "hctr_load",
            "hctr_stream", "hctr_last_times", "hctr_last_push_ms", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
            "hctr_stage_times", "hctr_copy_probe", "hctr_sample_rows", "hctr_version", "hctr_part_create", "hctr_part_destroy",
            "hctr_part_sizes", "hctr_part_refine_data", "hctr_part_refine_embed", "hctr_part_get_communication",
@@ -45,6 +45,8 @@ def lib():
         l.hctr_preprocess.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         l.hctr_preprocess_noalloc.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         l.hctr_push_pull.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        l.hctr_push_pull_pooled.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        l.hctr_group_push_pull_pooled.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]
         l.hctr_group_preprocess.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         l.hctr_group_push_pull.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         l.hctr_seed.argtypes = [C.c_ulong]
@@ -127,6 +129,11 @@ class Table:
     def push_pull(self, grad_ptr, dst_ptr):
         _check(lib().hctr_push_pull(self._h, C.c_void_p(int(grad_ptr) or None), C.c_void_p(int(dst_ptr) or None)))
 
+    def push_pull_pooled(self, grad_ptr, dst_ptr, bag):
+        """push_pull with sum-pooled bags of `bag` consecutive keys: one gradient / output row per bag."""
+        _check(lib().hctr_push_pull_pooled(self._h, C.c_void_p(int(grad_ptr) or None),
+                                           C.c_void_p(int(dst_ptr) or None), bag))
+
     def fetch(self, which):
         n = C.c_size_t()
         _check(lib().hctr_debug_fetch(self._h, which, None, 0, C.byref(n)))
@@ -206,3 +213,8 @@ def group_preprocess(tables, key_ptrs, ns):
 def group_push_pull(tables, grad_ptrs, dst_ptrs):
     hs = (C.c_void_p * len(tables))(*[t._h for t in tables])
     _check(lib().hctr_group_push_pull(hs, len(tables), _ptrs(grad_ptrs), _ptrs(dst_ptrs)))
+
+
+def group_push_pull_pooled(tables, grad_ptrs, dst_ptrs, bag):
+    hs = (C.c_void_p * len(tables))(*[t._h for t in tables])
+    _check(lib().hctr_group_push_pull_pooled(hs, len(tables), _ptrs(grad_ptrs), _ptrs(dst_ptrs), bag))

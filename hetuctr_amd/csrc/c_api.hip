@@ -106,6 +106,13 @@ int hctr_push_pull(hctr_table *t, const float *grad, float *dst) {
   });
 }
 
+int hctr_push_pull_pooled(hctr_table *t, const float *grad_pooled, float *dst_pooled, size_t bag) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->group->push_pull_one(t->shard->cfg.rank, grad_pooled, dst_pooled, bag);
+  });
+}
+
 static Group *group_of(hctr_table *const *tables, int nrank) {
   HCTR_CHECK(tables && nrank >= 1, "null table list");
   for (int r = 0; r < nrank; r++) HCTR_CHECK(tables[r] && tables[r]->shard, "null table");
@@ -123,6 +130,11 @@ int hctr_group_preprocess(hctr_table *const *tables, int nrank, const int64_t *c
 
 int hctr_group_push_pull(hctr_table *const *tables, int nrank, const float *const *grads, float *const *dsts) {
   return guarded([&] { group_of(tables, nrank)->push_pull_all(grads, dsts); });
+}
+
+int hctr_group_push_pull_pooled(hctr_table *const *tables, int nrank, const float *const *grads_pooled,
+                                float *const *dsts_pooled, size_t bag) {
+  return guarded([&] { group_of(tables, nrank)->push_pull_all(grads_pooled, dsts_pooled, bag); });
 }
 
 // csrc/core/debug.cu:5-12

@@ -101,9 +101,46 @@ void launch_bucket_counts(hipStream_t s, const BatchView &b, const uint32_t *pre
                           int nrank, uint64_t *cnt_out);
 void launch_bucket_sizes(hipStream_t s, const BatchView &b, int nrank, uint64_t *cnt_out);
 
+// Division of a batch position by the bag size of sum-pooled lookups without a divide instruction: for any 32-bit
+// n and bag >= 2, n / bag == (((n - q) >> 1) + q) >> shift with q = high word of n * magic (the "round up, add back"
+// form of division by an invariant integer).  bag == 1 leaves positions alone (no shifts, magic 0).
+struct BagDiv {
+  uint32_t bag = 1, magic = 0, half = 0, shift = 0;
+  BagDiv() = default;
+  explicit BagDiv(uint32_t d) : bag(d) {
+    if (d < 2) return; // magic 0 and no shifts: the formula below returns n
+    half = 1;
+    int lg = 31;
+    while (!((d >> lg) & 1u)) lg--; // floor(log2 d)
+    if ((d & (d - 1)) == 0) {         // a power of two: q is 0 and the two shifts make up log2(d)
+      magic = 0;
+      shift = (uint32_t)lg - 1;
+      return;
+    }
+    const uint64_t num = (uint64_t)1 << (32 + lg);
+    uint64_t m = num / d;
+    const uint64_t rem = num - m * d;
+    m = (m + m) & 0xffffffffull;
+    const uint64_t twice = rem + rem;
+    if (twice >= d) m += 1;
+    magic = (uint32_t)(m + 1);
+    shift = (uint32_t)lg;
+  }
+  // straight-line code for every bag size (a branch here would sit inside the load pipelines of the push)
+  __host__ __device__ __forceinline__ uint32_t operator()(uint32_t n) const {
+#ifdef __HIP_DEVICE_COMPILE__
+    const uint32_t q = __umulhi(n, magic);
+#else
+    const uint32_t q = (uint32_t)(((uint64_t)n * magic) >> 32);
+#endif
+    return (((n - q) >> half) + q) >> shift;
+  }
+};
+
 // ---- push: segment-sum of gradients by unique key + fused SGD ----------------------------------------
 struct PushArgs {
-  const embed_t *grad;       // [n_prev][width]
+  const embed_t *grad;       // [n_prev / bag][width]
+  BagDiv bag;                // bag size of sum-pooled lookups (1: none): position i reads gradient row i / bag
   const uint32_t *need;      // [U_prev] or nullptr when nrank == 1
   const uint32_t *prefix;    // [U_prev] push slot
   index_t *g_idx;            // push buffers
@@ -138,6 +175,9 @@ struct PullArgs {
 void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
                     uint32_t *stats);
 void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a);
+// sum-pooled lookups: dst[b] = the rows of positions b * bag .. b * bag + bag - 1 added up in that order
+// (cur.idx_map must be filled: launch_idx_map)
+void launch_gather_pooled(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a, uint32_t bag);
 
 // ---- init -------------------------------------------------------------------------------------------------
 void launch_init_values(hipStream_t s, embed_t *out, size_t len, int type, float a, float b, unsigned seed);

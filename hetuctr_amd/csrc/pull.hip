@@ -188,6 +188,43 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
   }
 }
 
+// Sum-pooled lookups: one group per bag of `bag` consecutive batch positions.  The rows of the bag are requested
+// kPoolAhead at a time and added in position order (fp32, starting from the first row), so a bag costs one output
+// row instead of `bag`.  Works in batch order, through the inverse index of the batch.
+constexpr int kPoolAhead = 8;
+template <int VEC, int LPR, bool kLocalOnly>
+__global__ __launch_bounds__(kBlock) void gather_pooled(TableView t, BatchView c, PullArgs a, uint32_t bag,
+                                                        uint32_t n_bags) {
+  typedef typename RowVec<VEC>::T V;
+  constexpr int kGroups = kBlock / LPR;
+  const uint32_t b = blockIdx.x * kGroups + threadIdx.x / LPR;
+  if (b >= n_bags) return;
+  const uint32_t gl = threadIdx.x % LPR, W = t.width;
+  const uint32_t i0 = b * bag;
+  for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
+    V acc;
+    for (uint32_t h0 = 0; h0 < bag; h0 += kPoolAhead) {
+      const embed_t *src[kPoolAhead];
+#pragma unroll
+      for (int k = 0; k < kPoolAhead; k++) {
+        const uint32_t u = c.idx_map[i0 + min(h0 + k, bag - 1)];
+        const slot_t o = c.uoff[u];
+        if (kLocalOnly || o != kNoSlot) src[k] = t.emb + (size_t)o * W;
+        else src[k] = a.in_val + (size_t)a.ret_i[u] * W;
+      }
+      V v[kPoolAhead];
+#pragma unroll
+      for (int k = 0; k < kPoolAhead; k++) v[k] = *(const V *)(src[k] + col);
+#pragma unroll
+      for (int k = 0; k < kPoolAhead; k++) {
+        if (h0 + k == 0) acc = v[k];
+        else if (h0 + k < bag) acc = acc + v[k];
+      }
+    }
+    __builtin_nontemporal_store(acc, (V *)(a.dst + (size_t)b * W + col));
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void copy_segments(const CopyDesc *__restrict__ d) {
   const CopyDesc cd = d[blockIdx.y];
   const size_t stride = (size_t)gridDim.x * kBlock;
@@ -308,6 +345,23 @@ void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, cons
     else if (local_only) hipLaunchKernelGGL((gather<V, L, true, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a); \
     else if (a.stream_stores) hipLaunchKernelGGL((gather<V, L, false, true>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a); \
     else hipLaunchKernelGGL((gather<V, L, false, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a);          \
+  } while (0)
+  HCTR_DISPATCH_ROW(vec4, lpr, CALL);
+#undef CALL
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_gather_pooled(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a, uint32_t bag) {
+  if (!cur.n) return;
+  const uint32_t n_bags = cur.n / bag;
+  const bool vec4 = t.width % 4 == 0 && ((uintptr_t)a.dst % 16) == 0;
+  const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
+  const bool local_only = a.got == nullptr;
+#define CALL(V, L)                                                                                                  \
+  do {                                                                                                              \
+    const unsigned blocks = div_up(n_bags, kBlock / L);                                                             \
+    if (local_only) hipLaunchKernelGGL((gather_pooled<V, L, true>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a, bag, n_bags); \
+    else hipLaunchKernelGGL((gather_pooled<V, L, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a, bag, n_bags);  \
   } while (0)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL

@@ -73,22 +73,26 @@ __device__ __forceinline__ uint32_t div_up_dev(uint32_t a, uint32_t b) { return 
 #define HCTR_GRAD_NT 1
 #endif
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-// a gradient row is read exactly once per step
-__device__ __forceinline__ float4 grad_load(const float4 *p) {
-#if HCTR_GRAD_NT
-  const f32x4 r = __builtin_nontemporal_load((const f32x4 *)p);
-  return make_float4(r.x, r.y, r.z, r.w);
-#else
+// A gradient row is read exactly once per step: it is loaded past the caches.  With sum-pooled bags (kPooled) a row
+// is read once per key of its bag, so there it is loaded the ordinary way and the repeats hit the cache.
+template <bool kPooled> __device__ __forceinline__ float4 grad_load(const float4 *p) {
+  if (HCTR_GRAD_NT && !kPooled) {
+    const f32x4 r = __builtin_nontemporal_load((const f32x4 *)p);
+    return make_float4(r.x, r.y, r.z, r.w);
+  }
   return *p;
-#endif
 }
-__device__ __forceinline__ float grad_load(const float *p) {
-#if HCTR_GRAD_NT
-  return __builtin_nontemporal_load(p);
-#else
+template <bool kPooled> __device__ __forceinline__ float grad_load(const float *p) {
+  if (HCTR_GRAD_NT && !kPooled) return __builtin_nontemporal_load(p);
   return *p;
-#endif
 }
+// The gradient row of batch position `pos`: the position itself, or with sum-pooled bags of `bag` consecutive
+// positions the row of the position's bag (every key of a bag receives the bag's gradient).
+// kPooled is a compile-time switch: the plain push must not pay for the division in its load pipelines.
+template <bool kPooled> __device__ __forceinline__ uint32_t grad_row(uint32_t pos, const BagDiv &bag) {
+  return kPooled ? bag(pos) : pos;
+}
+
 template <int VEC> struct Vec;
 template <> struct Vec<4> {
   typedef float4 T;
@@ -171,7 +175,7 @@ constexpr int kRunsPerGroup = HCTR_RUNS_PER_GROUP;
 constexpr int kHead = 2; // occurrences per run fetched up front
 constexpr int kTail = 6; // occurrences per step after those
 
-template <int VEC, int LPR, typename K, bool kSingle>
+template <int VEC, int LPR, typename K, bool kSingle, bool kPooled>
 __device__ __forceinline__ void short_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
                                            uint32_t block, uint32_t U) {
   typedef typename Vec<VEC>::T V;
@@ -215,13 +219,13 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 #pragma unroll
     for (int i = 0; i < G; i++)
 #pragma unroll
-      for (int k = 0; k < kHead; k++) si[i][k] = sorted_arg[min(rs[i] + k, n - 1)];
+      for (int k = 0; k < kHead; k++) si[i][k] = grad_row<kPooled>(sorted_arg[min(rs[i] + k, n - 1)], a.bag);
 #pragma unroll
     for (int i = 0; i < G; i++)
 #pragma unroll
       for (int k = 0; k < kHead; k++) {
         v[i][k] = Vec<VEC>::zero();
-        if (mine[i] && (uint32_t)k < len[i]) v[i][k] = grad_load((const V *)(grad + (size_t)si[i][k] * W + col));
+        if (mine[i] && (uint32_t)k < len[i]) v[i][k] = grad_load<kPooled>((const V *)(grad + (size_t)si[i][k] * W + col));
       }
     V acc[G];
 #pragma unroll
@@ -239,9 +243,9 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
         uint32_t sj[kTail];
         V x[kTail];
 #pragma unroll
-        for (int k = 0; k < kTail; k++) sj[k] = sorted_arg[min(j + k, rs[i + 1] - 1)];
+        for (int k = 0; k < kTail; k++) sj[k] = grad_row<kPooled>(sorted_arg[min(j + k, rs[i + 1] - 1)], a.bag);
 #pragma unroll
-        for (int k = 0; k < kTail; k++) x[k] = grad_load((const V *)(grad + (size_t)sj[k] * W + col));
+        for (int k = 0; k < kTail; k++) x[k] = grad_load<kPooled>((const V *)(grad + (size_t)sj[k] * W + col));
 #pragma unroll
         for (int k = 0; k < kTail; k++)
           if (j + k < rs[i + 1]) Vec<VEC>::add(acc[i], x[k]);
@@ -263,7 +267,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
 // over it).  The group first copies the run's gradient-row indices into LDS with one coalesced load, so that no
 // later load waits for an index; then two batches of kBatch gradient rows are kept in flight while the rows are
 // added in order.
-template <int VEC, int LPR, typename K, bool kSingle>
+template <int VEC, int LPR, typename K, bool kSingle, bool kPooled>
 __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
                                             uint32_t *lds_idx, uint32_t block, uint32_t nblocks) {
   typedef typename Vec<VEC>::T V;
@@ -280,7 +284,7 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
     const uint32_t lo = p.run_start[u], hi = p.run_start[u + 1];
     const uint32_t len = hi - lo; // <= kLongRun
     const slot_t off = p.uoff[u];
-    for (uint32_t q = gl; q < len; q += LPR) my_idx[q] = sorted_arg[lo + q];
+    for (uint32_t q = gl; q < len; q += LPR) my_idx[q] = grad_row<kPooled>(sorted_arg[lo + q], a.bag);
     // a group never spans waves: the LDS writes above are ordered before the reads below in hardware; the
     // fence keeps the compiler from moving them
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -296,7 +300,7 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
       V xa[kBatch], xb[kBatch];
       auto fetch = [&](V(&x)[kBatch], uint32_t q0) { // rows q0 .. q0+kBatch-1 of the run (clamped to its end)
 #pragma unroll
-        for (int k = 0; k < kBatch; k++) x[k] = grad_load((const V *)(gcol + (size_t)my_idx[min(q0 + k, len - 1)] * W));
+        for (int k = 0; k < kBatch; k++) x[k] = grad_load<kPooled>((const V *)(gcol + (size_t)my_idx[min(q0 + k, len - 1)] * W));
       };
       auto add = [&](const V(&x)[kBatch], uint32_t q0) {
 #pragma unroll
@@ -356,7 +360,7 @@ __device__ __forceinline__ uint32_t bundle_runs(int cls) { // runs per bundle: c
   return cls <= 6 ? 1u : min(1u << (cls - 6), (uint32_t)kTable); // one run of 2048 or more, 2 of 1024.., 4, 8, 16
 }
 
-template <int VEC, typename K, int CSC> // CSC: columns per slice if known at compile time, else 0
+template <int VEC, typename K, int CSC, bool kPooled> // CSC: columns per slice if known at compile time, else 0
 __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
                                           float *lds, uint4 *table, uint32_t *shared, int c_lo, int c_hi,
                                           uint32_t bidx, uint32_t nblk, uint32_t *counters) {
@@ -464,7 +468,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       // Loads are unconditional and branch-free so that kDepth chunks stay in flight per thread: positions
       // past the end of a run re-read its last row (never summed), lanes outside the slice read column 0.
       const embed_t *gbase = a.grad + ((in_slice && col < W) ? col : 0);
-      auto row_load = [&](uint32_t idx) -> V { return grad_load((const V *)(gbase + (size_t)idx * W)); };
+      auto row_load = [&](uint32_t idx) -> V { return grad_load<kPooled>((const V *)(gbase + (size_t)idx * W)); };
       // cursor of the index stage, 2 * kDepth chunks ahead of the LDS stage; past the end of the stream it
       // stays on the last run
       uint32_t cj = 0, cc = 0;
@@ -477,7 +481,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       }
       auto next_chunk = [&](uint32_t(&dst)[kRPT]) {
 #pragma unroll
-        for (int q = 0; q < kRPT; q++) dst[q] = sorted_arg[min(clo + cc * CR + q * RPL + my_row, chi - 1)];
+        for (int q = 0; q < kRPT; q++) dst[q] = grad_row<kPooled>(sorted_arg[min(clo + cc * CR + q * RPL + my_row, chi - 1)], a.bag);
         cc++;
         if (cc >= cn && cj + 1 < J) {
           cj++;
@@ -624,7 +628,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
 
 // all roles in one launch: the long chains start first, medium and short blocks fill the machine behind them, the
 // version counters of a single shard come last
-template <int VEC, int LPR, typename K, bool kSingle>
+template <int VEC, int LPR, typename K, bool kSingle, bool kPooled>
 #ifndef HCTR_PUSH_WAVES
 #define HCTR_PUSH_WAVES 4
 #endif
@@ -642,21 +646,21 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
     // advances with the share of the block that feeds it), then tickets of the other long runs.
     uint32_t *tk = p.d_nlong + kTicketBase;
     if (VEC == 4 && t.width % kSlice == 0) {
-      long_role<VEC, K, (VEC == 4 ? kGiantSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, 0, kGiantClasses,
+      long_role<VEC, K, (VEC == 4 ? kGiantSlice : 0), kPooled>(t, id_bits, p, a, lds, run_table, run_totals, 0, kGiantClasses,
                                                       blockIdx.x, kLongBlocks, tk);
-      long_role<VEC, K, (VEC == 4 ? kSlice : 0)>(t, id_bits, p, a, lds, run_table, run_totals, kGiantClasses, kLongBuckets,
+      long_role<VEC, K, (VEC == 4 ? kSlice : 0), kPooled>(t, id_bits, p, a, lds, run_table, run_totals, kGiantClasses, kLongBuckets,
                                                  blockIdx.x, kLongBlocks, tk + kTicketLanes);
     } else {
-      long_role<VEC, K, 0>(t, id_bits, p, a, lds, run_table, run_totals, 0, kLongBuckets, blockIdx.x, kLongBlocks, tk);
+      long_role<VEC, K, 0, kPooled>(t, id_bits, p, a, lds, run_table, run_totals, 0, kLongBuckets, blockIdx.x, kLongBlocks, tk);
     }
   } else if (blockIdx.x < kLongBlocks + kMedBlocks) { // medium runs take long per block: they start early
-    medium_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, (uint32_t *)lds, blockIdx.x - kLongBlocks, kMedBlocks);
+    medium_role<VEC, LPR, K, kSingle, kPooled>(t, id_bits, p, a, (uint32_t *)lds, blockIdx.x - kLongBlocks, kMedBlocks);
   } else {
     constexpr int kGroups = kPushBlock / LPR;
     const uint32_t short_blocks = div_up_dev(U, kGroups * kRunsPerGroup);
     const uint32_t b = blockIdx.x - kLongBlocks - kMedBlocks;
     if (b < short_blocks) {
-      short_role<VEC, LPR, K, kSingle>(t, id_bits, p, a, b, U);
+      short_role<VEC, LPR, K, kSingle, kPooled>(t, id_bits, p, a, b, U);
     } else if (kSingle) {
       // Single shard: every key is owned, so the only counter is the row version, which grows by the number of
       // duplicates (generate_query.cu:68-69).  One thread per unique key, in the last blocks of the grid.
@@ -672,24 +676,31 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
   }
 }
 
-template <int VEC, int LPR, typename K, bool kSingle>
+template <int VEC, int LPR, typename K, bool kSingle, bool kPooled>
 void launch_push_t(hipStream_t st, const TableView &t, int id_bits, const BatchView &p, uint32_t U, const PushArgs &a) {
   constexpr int kGroups = kPushBlock / LPR;
   const unsigned ver_blocks = kSingle ? div_up(U, kPushBlock) : 0; // version counters of a single shard
   const unsigned rest = kMedBlocks + div_up(U, kGroups * kRunsPerGroup) + ver_blocks;
-  hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle>), dim3(kLongBlocks + rest), dim3(kPushBlock), 0, st, t, id_bits, p,
+  hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle, kPooled>), dim3(kLongBlocks + rest), dim3(kPushBlock), 0, st, t, id_bits, p,
                      a, U);
+}
+
+template <int VEC, typename K, bool kSingle, bool kPooled>
+void launch_push_p(hipStream_t ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
+                   const PushArgs &a) {
+  const uint32_t lanes = (t.width + VEC - 1) / VEC;
+  if (lanes <= 4) launch_push_t<VEC, 4, K, kSingle, kPooled>(ps, t, id_bits, p, U, a);
+  else if (lanes <= 8) launch_push_t<VEC, 8, K, kSingle, kPooled>(ps, t, id_bits, p, U, a);
+  else if (lanes <= 16) launch_push_t<VEC, 16, K, kSingle, kPooled>(ps, t, id_bits, p, U, a);
+  else if (lanes <= 32) launch_push_t<VEC, 32, K, kSingle, kPooled>(ps, t, id_bits, p, U, a);
+  else launch_push_t<VEC, 64, K, kSingle, kPooled>(ps, t, id_bits, p, U, a);
 }
 
 template <int VEC, typename K, bool kSingle>
 void launch_push_v(hipStream_t ps, const TableView &t, int id_bits, const BatchView &p, uint32_t U,
                    const PushArgs &a) {
-  const uint32_t lanes = (t.width + VEC - 1) / VEC;
-  if (lanes <= 4) launch_push_t<VEC, 4, K, kSingle>(ps, t, id_bits, p, U, a);
-  else if (lanes <= 8) launch_push_t<VEC, 8, K, kSingle>(ps, t, id_bits, p, U, a);
-  else if (lanes <= 16) launch_push_t<VEC, 16, K, kSingle>(ps, t, id_bits, p, U, a);
-  else if (lanes <= 32) launch_push_t<VEC, 32, K, kSingle>(ps, t, id_bits, p, U, a);
-  else launch_push_t<VEC, 64, K, kSingle>(ps, t, id_bits, p, U, a);
+  if (a.bag.bag > 1) launch_push_p<VEC, K, kSingle, true>(ps, t, id_bits, p, U, a);
+  else launch_push_p<VEC, K, kSingle, false>(ps, t, id_bits, p, U, a);
 }
 
 template <int VEC, typename K>

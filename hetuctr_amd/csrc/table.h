@@ -127,12 +127,12 @@ class Shard {
   void finish_plan();
   void finish_index();
   void check_key_error();                   // raises if the ingested batch held a key outside [0, length)
-  void generate_gradient(const float *grad);
+  void generate_gradient(const float *grad, uint32_t bag = 1);
   void generate_query();
   void handle_gradient();
   void handle_query();
   void finish_handle_query();               // after the mid-step sync
-  void write_back(float *dst);
+  void write_back(float *dst, uint32_t bag = 1);
   void finish_push_pull();
 
   size_t fetch(int which, void *host_out, size_t cap);
@@ -228,10 +228,11 @@ class Group {
   void preprocess_all(const int64_t *const *keys, const size_t *n);
   void preprocess_noalloc(const int64_t *keys, size_t n);
   void *noalloc_scratch = nullptr;       // device address of this GPU's static scratch array
-  void push_pull_all(const float *const *grads, float *const *dsts);
+  // bag > 1: sum-pooled lookups, grads and dsts hold one row per bag of `bag` consecutive keys
+  void push_pull_all(const float *const *grads, float *const *dsts, size_t bag = 1);
   // per-shard entry points: rendezvous of nrank callers
   void preprocess_one(int rank, const int64_t *keys, size_t n);
-  void push_pull_one(int rank, const float *grad, float *dst);
+  void push_pull_one(int rank, const float *grad, float *dst, size_t bag = 1);
 
  private:
   void exchange_shapes();
@@ -248,6 +249,7 @@ class Group {
   std::vector<size_t> a_n_;
   std::vector<const float *> a_grad_;
   std::vector<float *> a_dst_;
+  std::vector<size_t> a_bag_;
 };
 
 // brackets the launches of one stage with two events when stage timing is on

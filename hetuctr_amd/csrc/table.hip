@@ -407,7 +407,7 @@ void Shard::check_key_error() {
 }
 
 // csrc/core/generate_query.cu:85-89; inference rule of csrc/core/hetu_gpu_table.cu:14-21
-void Shard::generate_gradient(const float *grad) {
+void Shard::generate_gradient(const float *grad, uint32_t bag) {
   hipStream_t s = group->stream;
   if (grad == nullptr) {
     prev.n = 0;
@@ -423,8 +423,10 @@ void Shard::generate_gradient(const float *grad) {
   for (int i = 0; i < cfg.nrank; i++) pushes += prev.push_cnt[i];
   last_stats[3] = (long long)pushes;
   const size_t W = cfg.width;
+  HCTR_CHECK(prev.n % bag == 0, "pooled push: the previous batch is not a whole number of bags");
   PushArgs a;
   a.grad = grad;
+  a.bag = BagDiv(bag);
   a.need = nullptr;
   a.prefix = nullptr;
   a.g_idx = nullptr;
@@ -517,7 +519,7 @@ void Shard::finish_handle_query() {
 }
 
 // csrc/core/writeback.cu:43-56
-void Shard::write_back(float *dst) {
+void Shard::write_back(float *dst, uint32_t bag) {
   hipStream_t s = group->stream;
   PullArgs a;
   a.got = nullptr;
@@ -545,7 +547,16 @@ void Shard::write_back(float *dst) {
   }
   if (dst != nullptr) {
     StageScope st(*group, S_GATHER);
-    launch_gather(s, tv, cur.view(), a);
+    if (bag > 1) { // sum-pooled bags: in batch order, through the inverse index
+      HCTR_CHECK(cur.n % bag == 0, "pooled pull: the batch is not a whole number of bags");
+      if (!cur.idx_map_valid) {
+        launch_idx_map(s, cur.view());
+        cur.idx_map_valid = true;
+      }
+      launch_gather_pooled(s, tv, cur.view(), a, bag);
+    } else {
+      launch_gather(s, tv, cur.view(), a);
+    }
   }
 }
 
@@ -675,6 +686,7 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   a_n_.resize(nr);
   a_grad_.resize(nr);
   a_dst_.resize(nr);
+  a_bag_.resize(nr, 1);
   if (const char *w = getenv("HETUCTR_GROUP_WAIT_SECONDS")) wait_seconds = atof(w);
 }
 
@@ -1041,11 +1053,13 @@ void Group::exchange_shapes() {
 }
 
 // csrc/core/hetu_gpu_table.cu:9-41 for every shard of the group
-void Group::push_pull_all(const float *const *grads, float *const *dsts) {
+void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t bag_size) {
+  HCTR_CHECK(bag_size >= 1 && bag_size < (1u << 24), "bag size out of range");
+  const uint32_t bag = (uint32_t)bag_size;
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
   if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
-  for (Shard *m : members) m->generate_gradient(grads[m->cfg.rank]);
+  for (Shard *m : members) m->generate_gradient(grads[m->cfg.rank], bag);
   if (time_calls) HCTR_HIP(hipEventRecord(ev_push, stream));
   enqueue_index_rest(); // single shard: the push is in its queue, now the rest of the current batch's index
   if (index_pending && nrank > 1) {
@@ -1073,7 +1087,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts) {
     for (Shard *m : members) m->finish_handle_query();
     exchange_return();
   }
-  for (Shard *m : members) m->write_back(dsts[m->cfg.rank]);
+  for (Shard *m : members) m->write_back(dsts[m->cfg.rank], bag);
   if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
   sync_stream();
   collect_marks();
@@ -1134,17 +1148,22 @@ void Group::preprocess_one(int rank, const int64_t *keys, size_t n) {
   collective(rank, 1, [&] { preprocess_all(a_keys_.data(), a_n_.data()); });
 }
 
-void Group::push_pull_one(int rank, const float *grad, float *dst) {
+void Group::push_pull_one(int rank, const float *grad, float *dst, size_t bag) {
   if (nrank == 1) {
-    push_pull_all(&grad, &dst);
+    push_pull_all(&grad, &dst, bag);
     return;
   }
   {
     std::lock_guard<std::mutex> lk(mu_);
     a_grad_[rank] = grad;
     a_dst_[rank] = dst;
+    a_bag_[rank] = bag;
   }
-  collective(rank, 2, [&] { push_pull_all(a_grad_.data(), a_dst_.data()); });
+  collective(rank, 2, [&] {
+    for (int r = 1; r < nrank; r++)
+      HCTR_CHECK(a_bag_[r] == a_bag_[0], "the shards of a group must pool with the same bag size");
+    push_pull_all(a_grad_.data(), a_dst_.data(), a_bag_[0]);
+  });
 }
 
 // ---- registry of groups by (ip, port) --------------------------------------------------------------

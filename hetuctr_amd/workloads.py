@@ -154,21 +154,22 @@ def sharded_extra_bytes(width, touched_cached, pushed, received, queried, return
             queried * 2 * (8 + 8 + 16 + 8) + returned * (2 * row + 2 * row + 8) + refreshed * (3 * row + 8))
 
 
-def algorithmic_bytes(n_keys, n_unique, width):
+def algorithmic_bytes(n_keys, n_unique, width, bag=1):
     """Bytes one full step must move at least, all rows local (one shard): gradient read and output write per
-    key, one gather read and one read-modify-write per unique row, plus the index traffic per key (41 B) and
-    per unique key (81 B), counted with the reference's 8-byte indices."""
+    key (per bag of `bag` keys when the lookups are sum-pooled), one gather read and one read-modify-write per unique
+    row, plus the index traffic per key (41 B) and per unique key (81 B), counted with the reference's 8-byte
+    indices."""
     row = 4 * width
-    return row * (2 * n_keys + 3 * n_unique) + 41 * n_keys + 81 * n_unique
+    return row * (2 * (n_keys // bag) + 3 * n_unique) + 41 * n_keys + 81 * n_unique
 
 
-def stage_bytes(stage, n_keys, n_unique, n_prev, u_prev, width):
+def stage_bytes(stage, n_keys, n_unique, n_prev, u_prev, width, bag=1):
     """Algorithmic bytes of one launch of a W-wide stage (same accounting as algorithmic_bytes)."""
     row = 4 * width
     if stage == "segment_sum_apply":   # gradient rows + row RMW; sorted_arg read per key; offset, run_start, version RMW per unique
-        return row * n_prev + 2 * row * u_prev + 8 * n_prev + (8 + 8 + 16) * u_prev
+        return row * (n_prev // bag) + 2 * row * u_prev + 8 * n_prev + (8 + 8 + 16) * u_prev
     if stage == "gather":              # output write + unique-row read; idx_map read per key; offset read per unique
-        return row * n_keys + row * n_unique + 8 * n_keys + 8 * n_unique
+        return row * (n_keys // bag) + row * n_unique + 8 * n_keys + 8 * n_unique
     raise KeyError(stage)
 
 

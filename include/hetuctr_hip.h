@@ -75,11 +75,24 @@ int hctr_preprocess_noalloc(hctr_table *t, const int64_t *keys, size_t n);
  * float[n][width] receives the rows of the current batch.  Synchronous. */
 int hctr_push_pull(hctr_table *t, const float *grad, float *dst);
 
+/* hctr_push_pull for multi-hot lookups that are sum-pooled: the batch is a sequence of bags of `bag` consecutive keys
+ * (the layout the reference's drivers give a multi-hot field, tests/benchmark.py:19-23 flattens samples the same
+ * way).  No counterpart in the reference, whose API has no pooling: there a bag is just more keys, the caller adds the
+ * pulled rows up itself and hands back the bag's gradient once per key.  Here dst_pooled is DEVICE
+ * float[n / bag][width], row b = the rows of keys b*bag .. b*bag+bag-1 added in that order (fp32, starting from the
+ * first), and grad_pooled is DEVICE float[n_prev / bag][width] or NULL, every key of a bag receiving its bag's row;
+ * the table ends in exactly the state hctr_push_pull reaches with the replicated gradients.  bag = 1 is
+ * hctr_push_pull; n and n_prev must be multiples of bag.  The pooled forms move 1/bag of the gradient and output
+ * bytes. */
+int hctr_push_pull_pooled(hctr_table *t, const float *grad_pooled, float *dst_pooled, size_t bag);
+
 /* Single-caller forms of the two calls above for a whole loopback group: entry r of each array belongs
  * to tables[r], which must be rank r of one complete group.  What R reference processes do in
  * lock-step with NCCL between the stages (csrc/core/all2all.cu:6-130) happens inside one call. */
 int hctr_group_preprocess(hctr_table *const *tables, int nrank, const int64_t *const *keys, const size_t *n);
 int hctr_group_push_pull(hctr_table *const *tables, int nrank, const float *const *grads, float *const *dsts);
+int hctr_group_push_pull_pooled(hctr_table *const *tables, int nrank, const float *const *grads_pooled,
+                                float *const *dsts_pooled, size_t bag);
 
 /* Replaces the module function hetuCTR.seed (csrc/pybind/pybind.cu:77): seed of tables created later. */
 void hctr_seed(unsigned long seed);

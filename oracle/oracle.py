@@ -102,6 +102,25 @@ class Oracle:
             raise RuntimeError(lib().orc_last_error().decode())
         return dsts
 
+    def push_pull_pooled(self, grads_pooled, bag):
+        """Sum-pooled bags of `bag` consecutive keys (no counterpart in the reference's API, which has no pooling:
+        its drivers flatten a multi-hot sample into more keys, tests/benchmark.py:19-23, and pool outside).  Defined
+        through the reference's own step: every key of a bag receives the bag's gradient row, and a bag's output is
+        the sum of its keys' pulled rows in key order, one fp32 addition at a time, starting from the first row.
+        grads_pooled: list of R float32 [Nprev / bag, W] arrays or None.  Returns R arrays [N / bag, W].
+        Pinned by tests/test_oracle_update.py::test_pooled_* (bag 1 is the plain step; exact occurrence counts)."""
+        gs = [None if g is None else np.repeat(np.ascontiguousarray(g, dtype=np.float32), bag, axis=0)
+              for g in grads_pooled]
+        out = []
+        for d in self.push_pull(gs):
+            assert d.shape[0] % bag == 0
+            v = d.reshape(-1, bag, self.W)
+            acc = v[:, 0, :].copy()
+            for h in range(1, bag):
+                acc = acc + v[:, h, :]          # elementwise float32 additions, in key order
+            out.append(acc)
+        return out
+
     def push_pull_into(self, grads, dsts):
         """Like push_pull with caller-provided float32 C-contiguous arrays (no allocation, no copies)."""
         if lib().orc_push_pull(self._h, _ptr_array(grads), _ptr_array(dsts)):

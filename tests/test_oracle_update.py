@@ -181,3 +181,58 @@ def test_not_stored_rows_always_push_and_pull():
     assert out == [[0.0, 0.0, 0.0], [3.0, 10.0, 3.0], [6.0, 20.0, 6.0]]
     assert o.fetch(0, orc.NEED_UPDATE).tolist() == [0, 1] and o.fetch(0, orc.PUSH_CNT).tolist() == [0, 1]
     assert int(o.fetch(1, orc.VERSION)[0]) == 4
+
+
+# ---- sum-pooled bags (oracle.Oracle.push_pull_pooled): pinned by what the definition fixes -----------------------
+@pytest.mark.parametrize("nrank", [1, 4])
+def test_pooled_occurrence_count_closed_form(nrank):
+    # zero init, lr = -1, every bag's gradient == 1: a key's row counts its earlier occurrences (a key that sits
+    # twice in a bag is pushed twice), and a bag pulls the sum of its keys' counts; all integers, exact in fp32
+    length, width, bag, bags = 512, 6, 5, 200
+    o, root, _ = update_setup(nrank, length, width)
+    rngs = [np.random.RandomState(7 + r) for r in range(nrank)]
+    store = np.zeros(length)
+    prev = [np.zeros(0, np.int64)] * nrank
+    for step in range(20):
+        for r in range(nrank):
+            np.add.at(store, prev[r], 1.0)
+        keys = [rngs[r].randint(length, size=bags * bag).astype(np.int64) for r in range(nrank)]
+        o.preprocess(keys)
+        gp = [np.ones((prev[r].shape[0] // bag, width), np.float32) for r in range(nrank)]
+        dst = o.push_pull_pooled(gp, bag)
+        for r in range(nrank):
+            want = store[keys[r]].reshape(bags, bag).sum(axis=1)
+            assert dst[r].shape == (bags, width)
+            assert np.array_equal(dst[r][:, 0], want.astype(np.float32)), (step, r)
+            assert np.all(dst[r] == dst[r][:, :1])
+        prev = keys
+
+
+def test_pooled_bag_of_one_is_the_plain_step_and_the_sum_runs_in_key_order():
+    length, width = 64, 3
+    root = np.zeros(length, np.uint8)
+    st = [np.arange(length, dtype=np.int64)]
+    a = orc.Oracle(1, length, width, 0, 0, root, st, init=("Uniform", -1.0, 1.0), learning_rate=0.5)
+    b = orc.Oracle(1, length, width, 0, 0, root, st, init=("Uniform", -1.0, 1.0), learning_rate=0.5)
+    rs = np.random.RandomState(1)
+    prev_n = 0
+    for step in range(4):
+        keys = rs.randint(length, size=40).astype(np.int64)
+        g = rs.rand(prev_n, width).astype(np.float32)
+        a.preprocess([keys]); b.preprocess([keys])
+        assert np.array_equal(a.push_pull([g])[0], b.push_pull_pooled([g], 1)[0])
+        prev_n = 40
+    # order of the additions, with rows 0, 1, 2 holding 1e8, 1, -1e8 (1e8 + 1 == 1e8 in fp32):
+    # keys (1, 0, 2): (1 + 1e8) - 1e8 = 0 from left to right, 1 from right to left or pairwise;
+    # keys (2, 0, 1): (-1e8 + 1e8) + 1 = 1 from left to right, 0 from right to left
+    c = orc.Oracle(1, 3, 1, 0, 0, np.zeros(3, np.uint8), [np.arange(3, dtype=np.int64)], init=("Zero", 0, 0),
+                   learning_rate=-1.0)
+    c.preprocess([np.array([0, 1, 2], np.int64)])
+    c.push_pull([None])
+    c.preprocess([np.array([1, 0, 2, 2, 0, 1], np.int64)])
+    c.push_pull_pooled([np.array([[1e8], [1.0], [-1e8]], np.float32)], 1)   # lr = -1: the rows become 1e8, 1, -1e8
+    c.preprocess([np.array([1, 0, 2, 2, 0, 1], np.int64)])
+    pooled = c.push_pull_pooled([None], 3)[0]
+    assert pooled[:, 0].tolist() == [0.0, 1.0]
+    for x in (a, b, c):
+        x.close()
