@@ -457,6 +457,58 @@ def main():
                                           "note": "start of push_pull to end of the push kernel while the sort/unique "
                                                   "kernels of the current batch share the GPU with it"}
 
+    def variant(ptrs, timing=True):
+        """The same table stepped with other key batches or another call protocol: ms per step, and the push / gather
+        kernels alone (pass with stage events)."""
+        def vstep(i):
+            table.preprocess(ptrs[i % len(ptrs)], n)
+            table.push_pull_pooled(grad.data_ptr(), dst.data_ptr(), bag)
+        us = []
+        for i in range(len(ptrs) + 2):
+            vstep(i)
+            us.append(int(table.fetch(capi.SIZES)[1]))
+        torch.cuda.synchronize()
+        tv0 = time.perf_counter()
+        for i in range(a.steps):
+            vstep(i)
+        torch.cuda.synchronize()
+        ms = 1e3 * (time.perf_counter() - tv0) / a.steps
+        u = float(np.mean(us[2:]))
+        res = {"ms_per_step": ms, "value": n / (ms * 1e-3), "unique_keys_per_step": u,
+               "step_hbm_frac": workloads.algorithmic_bytes(n, u, width, bag) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        if timing and not a.no_stage_timing:
+            table.stage_timing(True)
+            for i in range(a.steps):
+                vstep(i)
+            st = table.stage_times()
+            table.stage_timing(False)
+            res["stage_ms"] = {k: v[0] / max(v[1], 1) for k, v in st.items() if v[1]}
+            for k in kernel_names:
+                if k in res["stage_ms"]:
+                    res[kernel_names[k] + "_frac"] = (workloads.stage_bytes(k, n, u, n, u, width, bag) /
+                                                      (res["stage_ms"][k] * 1e-3) / 1e9 / HBM_PEAK_GBS)
+        return res
+
+    # the reference's literal call protocol: preprocess returns when all its work is done (hetu_gpu_table.cu:64), so
+    # nothing of the batch's index runs beside the push
+    literal = None
+    if not a.host_keys:
+        table.defer_index(False)
+        literal = variant(key_ptr, timing=False)
+        table.defer_index(True)
+    # the same workload with the hot rows of every field scattered over the field instead of lying side by side
+    permuted = None
+    if a.config == "cfg2" and a.scale == 1.0 and not a.host_keys:
+        pcfg = workloads.CONFIGS["cfg2_permuted"]
+        pks = workloads.KeyStream(pcfg, seed=0, scale=a.scale)
+        pkeys = [torch.from_numpy(pks.batch()).cuda() for _ in range(len(dkeys))]
+        pks.release_tables()
+        torch.cuda.synchronize()
+        permuted = variant([k.data_ptr() for k in pkeys])
+        permuted["note"] = ("rank -> id through a seeded permutation per field (cfg2_permuted); the headline keeps "
+                            "the Zipf rank as the local id, i.e. every field's hot rows are its first rows")
+        del pkeys
+
     out = {
         "metric": "sparse IDs/sec per train step (pull+push)", "value": n * a.steps / dt, "unit": "IDs/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_step, "higher_is_better": True,
@@ -464,8 +516,9 @@ def main():
         "config": {"workload": "%s: %d-row x %d fp32 table, batch %d samples x %d fields x %d ids = %d keys, %s, "
                                "SGD lr %g, one shard (all rows local)%s" %
                                (a.config, ks.rows, width, ks.samples, ks.fields, ks.hot, n,
-                                "uniform ids" if cfg["alpha"] is None else "per-field Zipf %.2f" % cfg["alpha"], lr,
-                                "" if bag == 1 else ", bags of %d ids sum-pooled" % bag),
+                                "uniform ids" if cfg["alpha"] is None else "per-field Zipf %.2f (%s)" %
+                                (cfg["alpha"], "rank -> id permuted per field" if cfg.get("permute") else "rank = local id"),
+                                lr, "" if bag == 1 else ", bags of %d ids sum-pooled" % bag),
                    "keys_per_step": n, "unique_keys_per_step": float(u_cur), "width": width, "rows": ks.rows,
                    "ids_handed_over_in": "pageable host memory" if a.host_keys else "HBM"},
         "unique_rows_per_sec": u_cur * a.steps / dt,
@@ -481,6 +534,8 @@ def main():
         "ms_per_step_with_stage_events": ms_step_ev,
         "roofline": roof,
         "roofline_stages": roof_all,
+        "literal_contract": literal,
+        "permuted_ids": permuted,
     }
     if not a.no_cpu:
         del dst

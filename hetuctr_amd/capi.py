@@ -11,7 +11,7 @@ LIB_PATH = os.environ.get("HETUCTR_LIB") or os.path.join(_HERE, "lib", "libhetuc
 INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
 SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_preprocess_noalloc", "hctr_push_pull", "hctr_push_pull_pooled",
            "hctr_group_preprocess", "hctr_group_push_pull", "hctr_group_push_pull_pooled", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch", "hctr_save", "hctr_load",
-           "hctr_stream", "hctr_last_times", "hctr_last_push_ms", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
+           "hctr_stream", "hctr_last_times", "hctr_last_push_ms", "hctr_defer_index", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
            "hctr_stage_times", "hctr_copy_probe", "hctr_sample_rows", "hctr_version", "hctr_part_create", "hctr_part_destroy",
            "hctr_part_sizes", "hctr_part_refine_data", "hctr_part_refine_embed", "hctr_part_get_communication",
            "hctr_part_get_priority", "hctr_part_get_result", "hctr_part_get_counts", "hctr_part_cache_lists"]
@@ -61,6 +61,7 @@ def lib():
         l.hctr_stream.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         l.hctr_last_times.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
         l.hctr_last_push_ms.argtypes = [C.c_void_p, C.POINTER(C.c_float)]
+        l.hctr_defer_index.argtypes = [C.c_void_p, C.c_int]
         l.hctr_stage_timing.argtypes = [C.c_void_p, C.c_int]
         l.hctr_stage_name.argtypes = [C.c_int]
         l.hctr_stage_name.restype = C.c_char_p
@@ -164,6 +165,10 @@ class Table:
         a = C.c_float()
         _check(lib().hctr_last_push_ms(self._h, C.byref(a)))
         return a.value
+
+    def defer_index(self, on):
+        """False: preprocess returns only when all of its work is done (the reference's contract)."""
+        _check(lib().hctr_defer_index(self._h, int(on)))
 
     def stage_timing(self, on):
         """Switches per-stage HIP-event timing on (resetting the accumulators) or off."""

@@ -211,6 +211,13 @@ int hctr_stage_timing(hctr_table *t, int on) {
   });
 }
 
+int hctr_defer_index(hctr_table *t, int on) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->group->set_defer_index(on != 0);
+  });
+}
+
 int hctr_stage_count(void) { return S_COUNT; }
 const char *hctr_stage_name(int stage) { return stage_name(stage); }
 

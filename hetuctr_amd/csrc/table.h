@@ -218,6 +218,7 @@ class Group {
   std::vector<hipEvent_t> event_pool;
   hipEvent_t take_event();
   void collect_marks();                  // after a stream sync
+  void set_defer_index(bool on);         // switches the early return of preprocess; waits for a pending index first
   void set_stage_timing(bool on);        // resets the accumulators; waits for a pending index under the group's lock
 
   void join(Shard *s);

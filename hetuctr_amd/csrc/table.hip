@@ -757,6 +757,12 @@ void Group::collect_marks() {
   marks.clear();
 }
 
+void Group::set_defer_index(bool on) {
+  std::lock_guard<std::mutex> lk(mu_);
+  flush_index();
+  defer_index = on;
+}
+
 void Group::set_stage_timing(bool on) {
   std::lock_guard<std::mutex> lk(mu_); // not while the ranks of the group are inside a collective call
   flush_index();

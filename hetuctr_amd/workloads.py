@@ -2,8 +2,10 @@
 
 A table is a concatenation of categorical fields; a sample holds one id per field (or `hot` ids per field for
 multi-hot bags, flattened: the table API has no pooling, a bag is just more keys).  Ids of a field follow a
-truncated Zipf law over the field's own range; the Zipf rank IS the local id (rank 0 = local id 0), i.e. the
-hot rows of every field are its first rows.  Batches are laid out sample-major: key[s * nfields*hot + f*hot + h].
+truncated Zipf law over the field's own range; by default the Zipf rank IS the local id (rank 0 = local id 0), i.e.
+the hot rows of every field are its first rows and lie next to each other in HBM.  With `permute` every field maps
+its ranks to local ids through a seeded permutation, so the hot rows are spread over the field's whole range.
+Batches are laid out sample-major: key[s * nfields*hot + f*hot + h].
 """
 import numpy as np
 
@@ -15,6 +17,9 @@ CONFIGS = {
     # headline: ~33M rows in 26 log-uniform fields (10 .. 10M), dim 128
     "cfg2": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=1.05, lr=0.05,
                  init=("Normal", 0.0, 0.1), single_field=False),
+    # the headline with the hot rows of every field scattered over the field (rank -> id through a permutation)
+    "cfg2_permuted": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=1.05, lr=0.05,
+                          init=("Normal", 0.0, 0.1), single_field=False, permute=True),
     # the same table and batch with uniform ids: nearly every key of a batch is distinct (no duplicates to sum)
     "cfg2_uniform": dict(rows=33_762_577, width=128, samples=65536, fields=26, hot=1, alpha=None, lr=0.05,
                          init=("Normal", 0.0, 0.1), single_field=True),
@@ -59,6 +64,9 @@ class KeyStream:
             self.card = field_cardinalities(self.rows, self.fields, seed)
             self.base = np.concatenate([[0], np.cumsum(self.card)[:-1]]).astype(np.int64)
         self.rng = np.random.default_rng(seed + 1)
+        self.permute = bool(cfg.get("permute"))
+        self.seed = seed
+        self._perm = {}
         self._cdf = {}
         self.n = self.samples * self.fields * self.hot
 
@@ -72,7 +80,12 @@ class KeyStream:
             cdf /= cdf[-1]
             self._cdf[f] = cdf
         u = self.rng.random(count)
-        return np.minimum(np.searchsorted(self._cdf[f], u, side="left"), c - 1).astype(np.int64)
+        rank = np.minimum(np.searchsorted(self._cdf[f], u, side="left"), c - 1).astype(np.int64)
+        if not self.permute:
+            return rank
+        if f not in self._perm:
+            self._perm[f] = np.random.default_rng(self.seed + 1000 + f).permutation(c)
+        return self._perm[f][rank]
 
     def batch(self):
         out = np.empty((self.samples, self.fields, self.hot), dtype=np.int64)
@@ -82,6 +95,7 @@ class KeyStream:
 
     def release_tables(self):
         self._cdf.clear()
+        self._perm.clear()
 
 
 def shard_layout(ks, nrank, cache_frac, seed=0, cached_ranks=(0,)):

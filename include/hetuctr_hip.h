@@ -150,6 +150,9 @@ int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
  * hctr_last_push_ms: device time from the start of the last hctr_push_pull to the end of its push stage, i.e. the
  * push kernel while the index of the next batch runs beside it.  No counterpart in the reference. */
 int hctr_last_push_ms(hctr_table *t, float *push_ms);
+/* The same switch as HETUCTR_DEFER_INDEX for a table's group at run time: 0 makes hctr_preprocess return only when
+ * all of its work is done (the reference's contract, hetu_gpu_table.cu:64), non-zero restores the early return. */
+int hctr_defer_index(hctr_table *t, int on);
 
 /* Per-stage device time.  hctr_stage_timing(t, 1) resets the accumulators and makes every later call bracket
  * each stage's launches with HIP events on the table's stream; hctr_stage_times returns, per stage, the

@@ -90,6 +90,56 @@ def test_normal_vs_reference_build(kind):
     assert np.max(np.abs(ref - got)) <= 2e-5 * 2.0
 
 
+def _normal_by_inverse_cdf(n, mean, stddev, seed):
+    """Element n of the Normal initialiser from the definitions alone: the engine's draw x, thrust's direct sampling
+    (csrc/utils/initializer.cu:29-46 -> thrust::normal_distribution, device branch): u = x - 1 in [0, m - 2]; the
+    lower half maps to mean - stddev * sqrt(2) * erfcinv(2p), p = (u + 1/2) / (m - 2), the upper half is mirrored
+    (u -> m - 2 - u, sign flipped).  -sqrt(2) * erfcinv(2p) is the inverse normal CDF at p: python's own."""
+    from statistics import NormalDist
+    rng_range = M - 2
+    u = _state(seed) * pow(A, n + 1, M) % M - 1
+    if u > rng_range // 2:
+        return mean - stddev * NormalDist().inv_cdf((rng_range - u + 0.5) / rng_range), u
+    return mean + stddev * NormalDist().inv_cdf((u + 0.5) / rng_range), u
+
+
+@pytest.mark.parametrize("mean,stddev,seed", [(0.0, 1.0, 0), (0.5, 2.0, 11), (-3.0, 0.1, 12345)])
+def test_normal_against_the_inverse_normal_cdf(mean, stddev, seed):
+    # pins sign, scale and the mirror of the upper half independently of any erfcinv implementation
+    got = orc.init_values(3000, "Normal", mean, stddev, seed)
+    lower = upper = 0
+    for n in list(range(200)) + [777, 1500, 2999]:
+        want, u = _normal_by_inverse_cdf(n, mean, stddev, seed)
+        lower += u <= (M - 2) // 2
+        upper += u > (M - 2) // 2
+        assert abs(float(got[n]) - want) <= 1e-6 * stddev + 1.2e-7 * abs(want), (n, got[n], want)
+        # the lower half of the draws gives values below the mean, the upper half above
+        assert (got[n] < mean) == (u <= (M - 2) // 2) or abs(got[n] - mean) < 1e-6 * stddev
+    assert lower > 50 and upper > 50                       # both branches were exercised
+    # truncation: the first draw that lies within two sigma, redrawn from the engine reseeded with its own next
+    # output (initializer.cu:60-67)
+    t = orc.init_values(3000, "TruncatedNormal", mean, stddev, seed)
+    redrawn = 0
+    for n in range(300):
+        x = _state(seed) * pow(A, n + 1, M) % M
+        while True:
+            rng_range = M - 2
+            u = x - 1
+            from statistics import NormalDist
+            if u > rng_range // 2:
+                v = mean - stddev * NormalDist().inv_cdf((rng_range - u + 0.5) / rng_range)
+            else:
+                v = mean + stddev * NormalDist().inv_cdf((u + 0.5) / rng_range)
+            x = x * A % M                                  # rng(): the next output ...
+            x = 1 if x % M == 0 else x % M                 # ... becomes the seed
+            if not (v > mean + 2 * stddev or v < mean - 2 * stddev):
+                break
+            redrawn += 1
+            x = x * A % M                                  # the next dist(rng) draws from the reseeded engine
+        assert abs(float(t[n]) - v) <= 1e-6 * stddev + 1.2e-7 * abs(v), (n, t[n], v)
+    assert redrawn >= 5                                    # ~4.6 % of the draws fall outside two sigma
+
+
 def test_normal_moments_and_determinism():
     x = orc.init_values(400000, "Normal", 1.0, 3.0, 2)
     assert abs(x.mean() - 1.0) < 0.03 and abs(x.std() - 3.0) < 0.03
