@@ -154,15 +154,41 @@ void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const B
 // ---- query / owner side / pull -------------------------------------------------------------------------
 void launch_lookup_version(hipStream_t s, const TableView &t, const BatchView &cur, version_t *q_ver);
 void launch_unique_ids(hipStream_t s, const KeyLayout &kl, const BatchView &cur, index_t *q_idx);
-// owner: received pushes of ONE source, [lo, hi) of the receive buffers
-void launch_apply_remote(hipStream_t s, const TableView &t, const index_t *rg_idx, const version_t *rg_cnt,
-                         const embed_t *rg_val, uint32_t lo, uint32_t hi, uint32_t *err);
-// owner: outdated flag per received query; queries in [self_lo, self_hi) came from this shard itself
-void launch_decide_outdated(hipStream_t s, const TableView &t, const index_t *rq_idx, const version_t *rq_ver,
-                            uint32_t q, uint32_t self_lo, uint32_t self_hi, uint32_t *outdated, uint32_t *err);
-// owner: pack version + row of every flagged query at its compacted position
-void launch_pack_rows(hipStream_t s, const TableView &t, const index_t *rq_idx, const uint32_t *outdated,
-                      const uint32_t *out_pos, uint32_t q, version_t *ret_ver, embed_t *ret_val);
+// Owner side of a step: applying the received pushes (per target row in source order) and serving the received
+// queries (outdated flags, positions of the rows to return, rows packed, first returned row of every requester).
+// One entry per shard of the group; one set of launches serves them all.
+struct OwnerShard {
+  TableView t;
+  // received pushes, sources concatenated in rank order; rg_seg[0..nsrc]: first row of every source
+  const index_t *rg_idx;
+  const version_t *rg_cnt;
+  const embed_t *rg_val;
+  uint32_t rg_seg[258];
+  int longest;               // the source with the most rows
+  uint32_t push_blocks;      // blocks the push kernel needs for this shard (rows of `longest` / rows per block)
+  // received queries; rq_seg[0..nsrc]: first query of every requester; [rq_seg[rank], rq_seg[rank + 1]) are its own
+  const index_t *rq_idx;
+  const version_t *rq_ver;
+  uint32_t rq_seg[258];
+  uint32_t q, query_tiles;
+  uint32_t *outdated, *tile_cnt, *out_pos;
+  version_t *ret_ver;
+  embed_t *ret_val;
+  uint32_t *err;             // the shard's error word
+  uint32_t *seg_dev;         // [0..nsrc] first returned row of every requester's segment, device copy
+  uint32_t *seg_host;        // the same in memory the host reads; [257] = error flags
+};
+size_t query_tiles(uint32_t q);                       // tile_cnt needs this many words + 1
+uint32_t owner_push_rows_per_block(uint32_t width);   // rows of the longest source one block of the push kernel takes
+// shards_dev: the array in device memory; shards_host: the same values on the host (launch geometry)
+void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerShard *shards_host, int nshards, int nsrc);
+// return exchange on the loopback: descs[2 * (s * nrank + d)] (versions) and the one after it (rows) for requester s
+// and owner d, from the owners' segment tables on the device; the pointer arrays (nrank entries each) must be
+// readable by the device
+struct CopyDesc;
+void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, const version_t *const *ret_ver,
+                               const embed_t *const *ret_val, version_t *const *in_ver, embed_t *const *in_val,
+                               int nrank, uint32_t width, CopyDesc *descs);
 // requester: refresh cached rows that came back, then gather every key's row into dst
 struct PullArgs {
   const uint32_t *got;       // [U] or nullptr: nothing came back (nrank == 1)
@@ -172,8 +198,10 @@ struct PullArgs {
   embed_t *dst;              // [n][width]
   bool stream_stores;        // write dst with nontemporal stores (see Shard::write_back)
 };
+// stats: five device words that read zero before the first call (the launch leaves them zero again); host_stats: four
+// words the device can write (hit / miss / refreshed counts of the step, error bits)
 void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
-                    uint32_t *stats);
+                    uint32_t *stats, uint32_t *host_stats);
 void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a);
 // sum-pooled lookups: dst[b] = the rows of positions b * bag .. b * bag + bag - 1 added up in that order
 // (cur.idx_map must be filled: launch_idx_map)

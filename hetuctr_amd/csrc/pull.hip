@@ -29,104 +29,261 @@ __global__ __launch_bounds__(kBlock) void unique_ids(int id_bits, BatchView c, i
   q_idx[u] = (index_t)(((const K *)c.ukey)[u] & (K)(((uint64_t)1 << id_bits) - 1));
 }
 
-// one group of LPR lanes per received row
+// ---- owner side: every kernel below serves ALL shards of a loopback group in one launch (blockIdx.y = shard), the
+// way the shards' GPUs would work side by side; with one shard per process the grid is one row high.
+//
+// Received pushes (csrc/core/handle_query.cu:106-116 applies them source by source, in rank order).  The rows that hit
+// one target must be added in source order, so a target's rows all go to one block: every source's segment of the
+// receive buffer is ascending in id (it is a slice of the sender's sorted unique keys), block b takes the ids
+// between two splitters drawn from the longest segment, finds that id range in every other segment by binary search,
+// and walks the sources in order with a barrier between them.  Inside a source ids are distinct, so its rows are
+// applied in parallel, kAhead rows per group of LPR lanes at a time.
+__device__ __forceinline__ uint32_t lower_bound_id(const index_t *__restrict__ a, uint32_t lo, uint32_t hi, index_t x) {
+  while (lo < hi) { // first position in [lo, hi) whose id is >= x
+    const uint32_t mid = lo + (hi - lo) / 2;
+    if (a[mid] < x) lo = mid + 1;
+    else hi = mid;
+  }
+  return lo;
+}
 template <int VEC, int LPR>
-__global__ __launch_bounds__(kBlock) void apply_remote(TableView t, const index_t *__restrict__ rg_idx,
-                                                       const version_t *__restrict__ rg_cnt,
-                                                       const embed_t *__restrict__ rg_val, uint32_t lo, uint32_t hi,
-                                                       uint32_t *__restrict__ err) {
+__global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__restrict__ shards, int nsrc,
+                                                           uint32_t rows_per_block) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
-  const uint32_t k = lo + blockIdx.x * kGroups + threadIdx.x / LPR;
-  if (k >= hi) return;
-  const uint32_t gl = threadIdx.x % LPR, W = t.width;
-  const uint64_t id = (uint64_t)rg_idx[k];
-  slot_t o = kNoSlot;
-  if (id < t.id_max && t.root[id] == t.rank) o = t.slot[id];
-  if (o == kNoSlot) {
-    if (gl == 0) atomicOr(err, 2u);
-    return;
+  const OwnerShard &S = shards[blockIdx.y];
+  if (blockIdx.x >= S.push_blocks) return;
+  const TableView &t = S.t;
+  const index_t *__restrict__ rg_idx = S.rg_idx;
+  __shared__ uint32_t lo[256], hi[256];
+  const int longest = S.longest;
+  const uint32_t big_lo = S.rg_seg[longest], big_hi = S.rg_seg[longest + 1];
+  const uint32_t first = big_lo + blockIdx.x * rows_per_block, last = first + rows_per_block;
+  for (int s = threadIdx.x; s < nsrc; s += kBlock) {
+    const uint32_t a = S.rg_seg[s], b = S.rg_seg[s + 1];
+    if (s == longest) { // the splitters are this segment's own rows
+      lo[s] = first;
+      hi[s] = min(last, big_hi);
+    } else if (a == b) {
+      lo[s] = hi[s] = a;
+    } else {
+      // block 0 starts below every id, the last block ends above every id
+      lo[s] = blockIdx.x == 0 ? a : lower_bound_id(rg_idx, a, b, rg_idx[first]);
+      hi[s] = last >= big_hi ? b : lower_bound_id(rg_idx, lo[s], b, rg_idx[last]);
+    }
   }
-  if (gl == 0) t.ver[o] += rg_cnt[k];
-  for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
-    V *e = (V *)(t.emb + (size_t)o * W + col);
-    *e = *e + *(const V *)(rg_val + (size_t)k * W + col);
+  __syncthreads();
+  const uint32_t gl = threadIdx.x % LPR, W = t.width;
+  constexpr int kAhead = 4; // rows of one source a group works on together (distinct ids, hence distinct targets)
+  for (int s = 0; s < nsrc; s++) {
+    for (uint32_t k0 = lo[s] + threadIdx.x / LPR; k0 < hi[s]; k0 += kGroups * kAhead) {
+      slot_t o[kAhead];
+      uint64_t id[kAhead];
+#pragma unroll
+      for (int a = 0; a < kAhead; a++) id[a] = (uint64_t)rg_idx[min(k0 + a * kGroups, hi[s] - 1)];
+#pragma unroll
+      for (int a = 0; a < kAhead; a++) {
+        const bool mine = id[a] < t.id_max && t.root[min(id[a], t.id_max - 1)] == t.rank;
+        o[a] = mine ? t.slot[id[a]] : kNoSlot;
+      }
+      bool bad = false;
+#pragma unroll
+      for (int a = 0; a < kAhead; a++) {
+        const uint32_t k = k0 + a * kGroups;
+        if (k >= hi[s]) o[a] = kNoSlot;
+        else if (o[a] == kNoSlot) bad = true;
+      }
+      if (bad && gl == 0) atomicOr(S.err, 2u);
+      if (gl == 0) {
+#pragma unroll
+        for (int a = 0; a < kAhead; a++)
+          if (o[a] != kNoSlot) t.ver[o[a]] += S.rg_cnt[k0 + a * kGroups];
+      }
+      for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
+        V cur[kAhead], add[kAhead];
+#pragma unroll
+        for (int a = 0; a < kAhead; a++) {
+          if (o[a] == kNoSlot) continue;
+          cur[a] = *(const V *)(t.emb + (size_t)o[a] * W + col);
+          add[a] = *(const V *)(S.rg_val + (size_t)(k0 + a * kGroups) * W + col);
+        }
+#pragma unroll
+        for (int a = 0; a < kAhead; a++)
+          if (o[a] != kNoSlot) *(V *)(t.emb + (size_t)o[a] * W + col) = cur[a] + add[a];
+      }
+    }
+    __syncthreads(); // the next source may push to the same rows
   }
 }
 
-__global__ __launch_bounds__(kBlock) void decide_outdated(TableView t, const index_t *__restrict__ rq_idx,
-                                                          const version_t *__restrict__ rq_ver, uint32_t q,
-                                                          uint32_t self_lo, uint32_t self_hi,
-                                                          uint32_t *__restrict__ outdated, uint32_t *__restrict__ err) {
+// Owner side of the pull (csrc/core/handle_query.cu:7-78) in three launches; the first two work on tiles of kBlock
+// received queries, one query per thread.
+// decide_count: the outdated flag of every query (pull rule, self-exempt, :47-54) and the number of flags per tile.
+// scan_positions: a tile's flags scanned behind the tiles before it -> position of every flagged query among the
+// returned rows (:56-57, :74-75), and the first returned row of every requester's segment (:59-61) written both to
+// device memory, where the return exchange reads it, and to the host.
+// pack_rows: version and row of every flagged query packed at its position (:24-40).
+__global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restrict__ shards) {
+  const OwnerShard &S = shards[blockIdx.y];
+  if (blockIdx.x >= S.query_tiles) return;
+  const TableView &t = S.t;
+  __shared__ uint32_t wcnt[kBlock / kWave];
   const uint32_t k = blockIdx.x * kBlock + threadIdx.x;
-  if (k >= q) return;
-  const uint64_t id = (uint64_t)rq_idx[k];
-  slot_t o = kNoSlot;
-  if (id < t.id_max && t.root[id] == t.rank) o = t.slot[id];
-  if (o == kNoSlot) {
-    atomicOr(err, 4u);
-    outdated[k] = 0;
-    return;
+  uint32_t flag = 0;
+  if (k < S.q) {
+    const uint64_t id = (uint64_t)S.rq_idx[k];
+    slot_t o = kNoSlot;
+    if (id < t.id_max && t.root[id] == t.rank) o = t.slot[id];
+    if (o == kNoSlot) {
+      atomicOr(S.err, 4u);
+    } else {
+      const version_t local = S.rq_ver[k], global = t.ver[o];
+      const bool from_self = k >= S.rq_seg[t.rank] && k < S.rq_seg[t.rank + 1];
+      const bool out = local == kInvalidVersion || local + t.pull_bound < global;
+      flag = (out && !from_self) ? 1u : 0u;
+    }
+    S.outdated[k] = flag;
   }
-  const version_t local = rq_ver[k], global = t.ver[o];
-  const bool from_self = k >= self_lo && k < self_hi;
-  const bool out = local == kInvalidVersion || local + t.pull_bound < global;
-  outdated[k] = (out && !from_self) ? 1u : 0u;
+  const uint64_t m = __ballot(flag != 0);
+  if (lane_id() == 0) wcnt[threadIdx.x / kWave] = __popcll(m);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t c = 0;
+    for (int i = 0; i < kBlock / kWave; i++) c += wcnt[i];
+    S.tile_cnt[blockIdx.x] = c;
+  }
 }
 
+__global__ __launch_bounds__(kBlock) void scan_positions(const OwnerShard *__restrict__ shards, int nseg) {
+  const OwnerShard &S = shards[blockIdx.y];
+  if (blockIdx.x >= S.query_tiles) return;
+  __shared__ uint32_t sm[kBlock / kWave + 1];
+  __shared__ uint32_t excl[kBlock + 1]; // position of every query of the tile among the returned rows; [kBlock]: after it
+  const uint32_t q = S.q;
+  const uint32_t tile_lo = blockIdx.x * kBlock, k = tile_lo + threadIdx.x;
+  const uint32_t f = k < q ? S.outdated[k] : 0u;
+  uint32_t s = 0;
+  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlock) s += S.tile_cnt[i];
+  uint32_t before;
+  block_exclusive_scan<kBlock>(s, sm, before); // flagged queries in the tiles before this one
+  uint32_t total;
+  const uint32_t pos = before + block_exclusive_scan<kBlock>(f, sm, total);
+  if (k < q) S.out_pos[k] = pos;
+  excl[threadIdx.x] = pos;
+  if (threadIdx.x == 0) excl[kBlock] = before + total;
+  __syncthreads();
+  // the first returned row of a requester's segment is the position of the segment's first query
+  const bool last_block = blockIdx.x == S.query_tiles - 1;
+  for (int g = threadIdx.x; g <= nseg; g += kBlock) {
+    const uint32_t start = S.rq_seg[g];
+    uint32_t v = ~0u;
+    if (start >= tile_lo && start < tile_lo + kBlock && start < q) v = excl[start - tile_lo];
+    else if (last_block && start >= q) v = excl[kBlock]; // segments that start at the end: the total
+    if (v != ~0u) {
+      S.seg_dev[g] = v;
+      S.seg_host[g] = v;
+    }
+  }
+  if (last_block && threadIdx.x == 0) S.seg_host[257] = *S.err;
+}
+
+// one group of LPR lanes per received query
 template <int VEC, int LPR>
-__global__ __launch_bounds__(kBlock) void pack_rows(TableView t, const index_t *__restrict__ rq_idx,
-                                                    const uint32_t *__restrict__ outdated,
-                                                    const uint32_t *__restrict__ out_pos, uint32_t q,
-                                                    version_t *__restrict__ ret_ver, embed_t *__restrict__ ret_val) {
+__global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict__ shards) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
+  const OwnerShard &S = shards[blockIdx.y];
+  const TableView &t = S.t;
   const uint32_t k = blockIdx.x * kGroups + threadIdx.x / LPR;
-  if (k >= q || !outdated[k]) return;
+  if (k >= S.q || !S.outdated[k]) return;
   const uint32_t gl = threadIdx.x % LPR, W = t.width;
-  const slot_t o = t.slot[(uint64_t)rq_idx[k]];
-  const uint32_t pos = out_pos[k];
-  if (gl == 0) ret_ver[pos] = t.ver[o];
+  const slot_t o = t.slot[(uint64_t)S.rq_idx[k]];
+  const uint32_t pos = S.out_pos[k];
+  if (gl == 0) S.ret_ver[pos] = t.ver[o];
   for (uint32_t col = gl * VEC; col < W; col += LPR * VEC)
-    *(V *)(ret_val + (size_t)pos * W + col) = *(const V *)(t.emb + (size_t)o * W + col);
+    *(V *)(S.ret_val + (size_t)pos * W + col) = *(const V *)(t.emb + (size_t)o * W + col);
+}
+
+// The copies of the return exchange (csrc/core/all2all.cu:89-130) described on the device: how many rows an owner
+// returns to a requester is only known there.  Thread (requester s, owner d) writes the two descriptors (versions,
+// rows) of that pair; the rows of requester s arrive in owner order.
+struct ReturnPeers {
+  const uint32_t *const *ret_seg;   // [nrank] per owner: first returned row of every requester's segment, [nrank] = total
+  const version_t *const *ret_ver;  // [nrank] per owner
+  const embed_t *const *ret_val;    // [nrank] per owner
+  version_t *const *in_ver;         // [nrank] per requester
+  embed_t *const *in_val;           // [nrank] per requester
+};
+__global__ void build_return_descs(ReturnPeers p, int nrank, uint32_t width, CopyDesc *__restrict__ descs) {
+  const int s = blockIdx.x, d = threadIdx.x;
+  if (d >= nrank) return;
+  uint32_t before = 0;
+  for (int e = 0; e < d; e++) before += p.ret_seg[e][s + 1] - p.ret_seg[e][s];
+  const uint32_t lo = p.ret_seg[d][s], n = p.ret_seg[d][s + 1] - lo;
+  CopyDesc *o = descs + 2 * ((size_t)s * nrank + d);
+  o[0].src = p.ret_ver[d] + lo;
+  o[0].dst = p.in_ver[s] + before;
+  o[0].bytes = (size_t)n * sizeof(version_t);
+  o[1].src = p.ret_val[d] + (size_t)lo * width;
+  o[1].dst = p.in_val[s] + (size_t)before * width;
+  o[1].bytes = (size_t)n * width * sizeof(embed_t);
 }
 
 // Counts of the step's remote unique keys: [0] cached and fresh enough, [1] not stored here, [2] cached and
-// refreshed.  Atomics on one address are served one after the other, so every thread counts its strided share in
-// registers and a block adds its three totals once.
+// refreshed; [3] bit 3: an owned row came back as outdated (it never may).  Atomics on one address are served one
+// after the other, so every thread counts its strided share in registers and a block adds its totals once.  The block
+// that finishes last hands the totals to the host (pinned memory) and puts the device counters back to zero for the
+// next step: no clearing launch before, no copy after.
 constexpr int kCountBlocks = 128;
 __global__ __launch_bounds__(kBlock) void count_remote(TableView t, BatchView c, const uint32_t *__restrict__ got,
-                                                       uint32_t *__restrict__ stats) {
-  __shared__ uint32_t tot[3];
-  if (threadIdx.x < 3) tot[threadIdx.x] = 0;
+                                                       uint32_t *__restrict__ stats, uint32_t *__restrict__ host_stats) {
+  __shared__ uint32_t tot[4];
+  __shared__ bool last;
+  if (threadIdx.x < 4) tot[threadIdx.x] = 0;
   __syncthreads();
   const uint32_t U = *c.d_U;
-  uint32_t n0 = 0, n1 = 0, n2 = 0;
+  uint32_t n0 = 0, n1 = 0, n2 = 0, bad = 0;
   for (uint32_t u = blockIdx.x * kBlock + threadIdx.x; u < U; u += kCountBlocks * kBlock) {
     const slot_t o = c.uoff[u];
     if (o == kNoSlot) n1++;
     else if ((uint32_t)o < t.n_cached) {
       if (got[u]) n2++;
       else n0++;
+    } else if (got[u]) {
+      bad = 8u;
     }
   }
   for (int d = 32; d; d >>= 1) {
     n0 += __shfl_down(n0, d);
     n1 += __shfl_down(n1, d);
     n2 += __shfl_down(n2, d);
+    bad |= __shfl_down(bad, d);
   }
   if (threadIdx.x % 64 == 0) {
     atomicAdd(&tot[0], n0);
     atomicAdd(&tot[1], n1);
     atomicAdd(&tot[2], n2);
+    atomicOr(&tot[3], bad);
   }
   __syncthreads();
   if (threadIdx.x < 3 && tot[threadIdx.x]) atomicAdd(&stats[threadIdx.x], tot[threadIdx.x]);
+  if (threadIdx.x == 3 && tot[3]) atomicOr(&stats[3], tot[3]);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    last = atomicAdd(&stats[4], 1u) == gridDim.x - 1;
+  }
+  __syncthreads();
+  if (last && threadIdx.x < 4) {
+    __threadfence();
+    host_stats[threadIdx.x] = atomicExch(&stats[threadIdx.x], 0u);
+    if (threadIdx.x == 0) stats[4] = 0;
+  }
 }
 
 // one group per unique rank of the current batch
 template <int VEC, int LPR>
-__global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, PullArgs a, uint32_t *__restrict__ stats) {
+__global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, PullArgs a) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
   const uint32_t u = blockIdx.x * kGroups + threadIdx.x / LPR;
@@ -134,11 +291,7 @@ __global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, Pull
   const uint32_t gl = threadIdx.x % LPR, W = t.width;
   const slot_t o = c.uoff[u];
   const bool got = a.got[u] != 0;
-  if (!got || o == kNoSlot) return;
-  if ((uint32_t)o >= t.n_cached) { // an owned row can never come back as outdated
-    if (gl == 0) atomicOr(&stats[3], 8u);
-    return;
-  }
+  if (!got || o == kNoSlot || (uint32_t)o >= t.n_cached) return; // (an owned row that came back is reported by count_remote)
   const uint32_t k = a.ret_i[u];
   if (gl == 0) t.ver[o] = a.in_ver[k];
   for (uint32_t col = gl * VEC; col < W; col += LPR * VEC)
@@ -288,46 +441,57 @@ void launch_unique_ids(hipStream_t s, const KeyLayout &kl, const BatchView &cur,
   HCTR_HIP(hipGetLastError());
 }
 
-void launch_apply_remote(hipStream_t s, const TableView &t, const index_t *rg_idx, const version_t *rg_cnt,
-                         const embed_t *rg_val, uint32_t lo, uint32_t hi, uint32_t *err) {
-  if (hi <= lo) return;
-  const bool vec4 = t.width % 4 == 0;
-  const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
+size_t query_tiles(uint32_t q) { return std::max<size_t>(1, div_up(q, kBlock)); }
+
+uint32_t owner_push_rows_per_block(uint32_t width) {
+  const int lpr = lanes_for(width, width % 4 == 0 ? 4 : 1);
+  return 4 * 4 * (kBlock / lpr); // four batches of kAhead rows per group
+}
+
+void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerShard *shards_host, int nshards, int nsrc) {
+  uint32_t push_blocks = 0, tiles = 0, q_max = 0;
+  const uint32_t width = shards_host[0].t.width;
+  for (int i = 0; i < nshards; i++) {
+    push_blocks = std::max(push_blocks, shards_host[i].push_blocks);
+    tiles = std::max(tiles, shards_host[i].query_tiles);
+    q_max = std::max(q_max, shards_host[i].q);
+  }
+  const bool vec4 = width % 4 == 0;
+  const int lpr = lanes_for(width, vec4 ? 4 : 1);
+  if (push_blocks) {
+    const uint32_t rpb = owner_push_rows_per_block(width);
 #define CALL(V, L) \
-  hipLaunchKernelGGL((apply_remote<V, L>), dim3(div_up(hi - lo, kBlock / L)), dim3(kBlock), 0, s, t, rg_idx, rg_cnt, rg_val, lo, hi, err)
-  HCTR_DISPATCH_ROW(vec4, lpr, CALL);
+  hipLaunchKernelGGL((apply_remote_all<V, L>), dim3(push_blocks, nshards), dim3(kBlock), 0, s, shards_dev, nsrc, rpb)
+    HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
+  }
+  hipLaunchKernelGGL(decide_count, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev);
+  hipLaunchKernelGGL(scan_positions, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
+  if (q_max) {
+#define CALL(V, L) \
+  hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q_max, kBlock / L), nshards), dim3(kBlock), 0, s, shards_dev)
+    HCTR_DISPATCH_ROW(vec4, lpr, CALL);
+#undef CALL
+  }
   HCTR_HIP(hipGetLastError());
 }
 
-void launch_decide_outdated(hipStream_t s, const TableView &t, const index_t *rq_idx, const version_t *rq_ver,
-                            uint32_t q, uint32_t self_lo, uint32_t self_hi, uint32_t *outdated, uint32_t *err) {
-  if (!q) return;
-  hipLaunchKernelGGL(decide_outdated, dim3(div_up(q, kBlock)), dim3(kBlock), 0, s, t, rq_idx, rq_ver, q, self_lo,
-                     self_hi, outdated, err);
-  HCTR_HIP(hipGetLastError());
-}
-
-void launch_pack_rows(hipStream_t s, const TableView &t, const index_t *rq_idx, const uint32_t *outdated,
-                      const uint32_t *out_pos, uint32_t q, version_t *ret_ver, embed_t *ret_val) {
-  if (!q) return;
-  const bool vec4 = t.width % 4 == 0;
-  const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
-#define CALL(V, L) \
-  hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q, kBlock / L)), dim3(kBlock), 0, s, t, rq_idx, outdated, out_pos, q, ret_ver, ret_val)
-  HCTR_DISPATCH_ROW(vec4, lpr, CALL);
-#undef CALL
+void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, const version_t *const *ret_ver,
+                               const embed_t *const *ret_val, version_t *const *in_ver, embed_t *const *in_val,
+                               int nrank, uint32_t width, CopyDesc *descs) {
+  ReturnPeers p{ret_seg, ret_ver, ret_val, in_ver, in_val};
+  hipLaunchKernelGGL(build_return_descs, dim3(nrank), dim3(std::max(64, (nrank + 63) / 64 * 64)), 0, s, p, nrank, width, descs);
   HCTR_HIP(hipGetLastError());
 }
 
 void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
-                    uint32_t *stats) {
+                    uint32_t *stats, uint32_t *host_stats) {
   if (!n_unique || !a.got) return;
-  hipLaunchKernelGGL(count_remote, dim3(kCountBlocks), dim3(kBlock), 0, s, t, cur, a.got, stats);
+  hipLaunchKernelGGL(count_remote, dim3(kCountBlocks), dim3(kBlock), 0, s, t, cur, a.got, stats, host_stats);
   const bool vec4 = t.width % 4 == 0;
   const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
 #define CALL(V, L) \
-  hipLaunchKernelGGL((refresh<V, L>), dim3(div_up(n_unique, kBlock / L)), dim3(kBlock), 0, s, t, cur, a, stats)
+  hipLaunchKernelGGL((refresh<V, L>), dim3(div_up(n_unique, kBlock / L)), dim3(kBlock), 0, s, t, cur, a)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   HCTR_HIP(hipGetLastError());

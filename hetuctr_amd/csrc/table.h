@@ -129,9 +129,8 @@ class Shard {
   void check_key_error();                   // raises if the ingested batch held a key outside [0, length)
   void generate_gradient(const float *grad, uint32_t bag = 1);
   void generate_query();
-  void handle_gradient();
-  void handle_query();
-  void finish_handle_query();               // after the mid-step sync
+  void fill_owner_args(OwnerShard &o);      // handleGradient + handleQuery: what the group's owner-side launches need
+  void finish_handle_query();               // after the step: return counts and error flags from the pinned block
   void write_back(float *dst, uint32_t bag = 1);
   void finish_push_pull();
 
@@ -150,7 +149,7 @@ class Shard {
     void *ktmp0 = nullptr, *ktmp1 = nullptr;
     uint32_t *vtmp0 = nullptr, *vtmp1 = nullptr, *sortws = nullptr, *block_sums = nullptr;
   } sp;
-  DeviceBuf need, prefix, plan_sums; // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
+  DeviceBuf need, prefix, plan_sums, query_sums; // query_sums: flags per tile of received queries // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
   DevStat *dst_ = nullptr; // == dstat.p
   uint32_t *err_ptr() const { return &dst_->err; }
   // send side
@@ -160,7 +159,6 @@ class Shard {
   std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
   // requester side of the return
   DeviceBuf got, ret_i, in_ver, in_val;
-  uint64_t in_rows = 0;
   HostMirror *mirror = nullptr;
   long long last_stats[6] = {0, 0, 0, 0, 0, 0};
   float last_pre_ms = 0.f, last_pp_ms = 0.f, last_push_ms = 0.f;
@@ -201,11 +199,17 @@ class Group {
   bool index_rest_pending = false;       // single shard: preprocess enqueued only the first launches of the index
   void enqueue_index_rest();             // enqueues the others
   void flush_index();                    // waits for a pending index and takes its results over
+  // owner-side arguments of every shard: pinned staging and the device copy the kernels read
+  OwnerShard *owner_host = nullptr;
+  DeviceBuf owner_dev;
+  void owner_side();
   bool time_calls = false;               // bracket the two calls with events (hctr_last_times switches it on)
   std::vector<Shard *> members;
-  DeviceBuf desc_dev;
-  CopyDesc *desc_host = nullptr;
-  size_t desc_cap = 0;
+  DeviceBuf desc_dev[2];                 // copy descriptors of the query exchange [0] and of the return exchange [1]
+  CopyDesc *desc_host[2] = {nullptr, nullptr};
+  void **peer_tab = nullptr;             // pinned: per-shard buffer addresses the return exchange reads on the device
+  CopyDesc *reserve_descs(size_t n, int which);
+  size_t desc_cap[2] = {0, 0};
   double wait_seconds = 120.0;
   void sync_stream();
 

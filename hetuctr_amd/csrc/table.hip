@@ -172,11 +172,11 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
 
   dstat.reserve(sizeof(DevStat));
   dst_ = dstat.as<DevStat>();
-  stats.reserve(16);
+  stats.reserve(32);
   ret_total.reserve(4);
   ret_seg_dev.reserve(2 * 258 * 4);
   HCTR_HIP(hipMemsetAsync(dstat.p, 0, dstat.bytes, s));
-  HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
+  HCTR_HIP(hipMemsetAsync(stats.p, 0, 32, s));
   for (Batch *b : {&cur, &prev}) {
     b->reserve(1, c.nrank, kl.wide);
     b->clear(s, c.nrank);
@@ -457,54 +457,43 @@ void Shard::generate_query() {
   launch_unique_ids(s, kl, cur.view(), q_idx.as<index_t>());
 }
 
-// csrc/core/handle_query.cu:106-116: one source after the other, in rank order
-void Shard::handle_gradient() {
-  hipStream_t s = group->stream;
-  last_stats[5] = (long long)rg_seg[cfg.nrank];
-  StageScope st(*group, S_OWNER);
-  for (int src = 0; src < cfg.nrank; src++)
-    launch_apply_remote(s, tv, rg_idx.as<index_t>(), rg_cnt.as<version_t>(), rg_val.as<embed_t>(),
-                        (uint32_t)rg_seg[src], (uint32_t)rg_seg[src + 1], err_ptr());
-}
-
-// rows to return per requester: where the segments of the query start in the compacted order of the rows that are
-// sent back; the last word carries the shard's error flags so that one transfer brings both to the host
-struct SegmentStarts {
-  uint32_t v[258];
-};
-__global__ void segment_bounds(const uint32_t *__restrict__ out_pos, const uint32_t *__restrict__ total, SegmentStarts seg,
-                               int nseg, uint32_t q, const uint32_t *__restrict__ err, uint32_t *__restrict__ out) {
-  const int i = threadIdx.x;
-  if (i == 0) out[257] = *err;
-  if (i > nseg) return;
-  const uint32_t k = seg.v[i];
-  out[i] = k >= q ? *total : out_pos[k];
-}
-
-// csrc/core/handle_query.cu:42-78
-void Shard::handle_query() {
-  hipStream_t s = group->stream;
+// What the owner-side kernels need of this shard for the step (csrc/core/handle_query.cu:7-116): the received pushes
+// and queries, the buffers of the rows that go back.  The number of rows that go back to every requester stays on the
+// device, where the return exchange reads it; the host copy (statistics, error flags) is written by the same kernel
+// into pinned memory and read when the step is over.
+void Shard::fill_owner_args(OwnerShard &o) {
   const int R = cfg.nrank;
   const uint32_t Q = (uint32_t)rq_seg[R];
   outdated.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
   out_pos.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
   ret_ver.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(version_t));
   ret_val.reserve((size_t)std::max<uint32_t>(Q, 1) * cfg.width * sizeof(embed_t));
-  reserve_batch_scratch(Q);
-  StageScope st(*group, S_OWNER);
-  launch_decide_outdated(s, tv, rq_idx.as<index_t>(), rq_ver.as<version_t>(), Q, (uint32_t)rq_seg[cfg.rank],
-                         (uint32_t)rq_seg[cfg.rank + 1], outdated.as<uint32_t>(), err_ptr());
-  launch_exclusive_scan(s, outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q, nullptr, block_sums.as<uint32_t>(),
-                        ret_total.as<uint32_t>());
-  launch_pack_rows(s, tv, rq_idx.as<index_t>(), outdated.as<uint32_t>(), out_pos.as<uint32_t>(), Q,
-                   ret_ver.as<version_t>(), ret_val.as<embed_t>());
-  SegmentStarts seg;
-  for (int i = 0; i <= R; i++) seg.v[i] = (uint32_t)rq_seg[i];
-  uint32_t *out = ret_seg_dev.as<uint32_t>();
-  hipLaunchKernelGGL(segment_bounds, dim3(1), dim3(R + 1), 0, s, out_pos.as<uint32_t>(), ret_total.as<uint32_t>(), seg, R, Q,
-                     err_ptr(), out);
-  HCTR_HIP(hipGetLastError());
-  HCTR_HIP(hipMemcpyAsync(mirror->ret_seg, out, 258 * 4, hipMemcpyDeviceToHost, s));
+  query_sums.reserve((query_tiles(Q) + 2) * 4);
+  last_stats[5] = (long long)rg_seg[R];
+  o.t = tv;
+  o.rg_idx = rg_idx.as<index_t>();
+  o.rg_cnt = rg_cnt.as<version_t>();
+  o.rg_val = rg_val.as<embed_t>();
+  o.longest = 0;
+  for (int i = 0; i <= R; i++) {
+    o.rg_seg[i] = (uint32_t)rg_seg[i];
+    o.rq_seg[i] = (uint32_t)rq_seg[i];
+  }
+  for (int i = 1; i < R; i++)
+    if (rg_seg[i + 1] - rg_seg[i] > rg_seg[o.longest + 1] - rg_seg[o.longest]) o.longest = i;
+  o.push_blocks = div_up(rg_seg[o.longest + 1] - rg_seg[o.longest], owner_push_rows_per_block(tv.width));
+  o.rq_idx = rq_idx.as<index_t>();
+  o.rq_ver = rq_ver.as<version_t>();
+  o.q = Q;
+  o.query_tiles = (uint32_t)query_tiles(Q); // one tile even without queries: the segment table is written
+  o.outdated = outdated.as<uint32_t>();
+  o.tile_cnt = query_sums.as<uint32_t>();
+  o.out_pos = out_pos.as<uint32_t>();
+  o.ret_ver = ret_ver.as<version_t>();
+  o.ret_val = ret_val.as<embed_t>();
+  o.err = err_ptr();
+  o.seg_dev = ret_seg_dev.as<uint32_t>();
+  o.seg_host = mirror->ret_seg;
 }
 
 void Shard::finish_handle_query() {
@@ -531,19 +520,19 @@ void Shard::write_back(float *dst, uint32_t bag) {
   // batch there for the push that updates them next.  The one case where that loses is a batch of (almost) all
   // distinct keys, where the gather reads as many rows as it writes; the previous batch is the predictor.
   a.stream_stores = !(prev.n != 0 && (double)prev.U >= 0.9 * (double)prev.n);
-  if (cfg.nrank > 1) {
+  if (cfg.nrank > 1 && cur.U == 0) {
+    memset(mirror->stats, 0, sizeof mirror->stats); // no keys: nothing came back (nothing in flight writes the block)
+  } else if (cfg.nrank > 1) {
     ret_i.reserve((size_t)std::max<uint32_t>(cur.U, 1) * 4);
     reserve_batch_scratch(cur.U);
     StageScope st(*group, S_REFRESH);
-    HCTR_HIP(hipMemsetAsync(stats.p, 0, 16, s));
     launch_exclusive_scan(s, got.as<uint32_t>(), ret_i.as<uint32_t>(), cur.U, nullptr, block_sums.as<uint32_t>(),
                           nullptr);
     a.got = got.as<uint32_t>();
     a.ret_i = ret_i.as<uint32_t>();
     a.in_ver = in_ver.as<version_t>();
     a.in_val = in_val.as<embed_t>();
-    launch_refresh(s, tv, cur.view(), cur.U, a, stats.as<uint32_t>());
-    HCTR_HIP(hipMemcpyAsync(mirror->stats, stats.p, 16, hipMemcpyDeviceToHost, s));
+    launch_refresh(s, tv, cur.view(), cur.U, a, stats.as<uint32_t>(), mirror->stats);
   }
   if (dst != nullptr) {
     StageScope st(*group, S_GATHER);
@@ -691,7 +680,9 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
 }
 
 Group::~Group() {
-  if (desc_host) (void)hipHostFree(desc_host);
+  for (CopyDesc *d : desc_host)
+    if (d) (void)hipHostFree(d);
+  if (peer_tab) (void)hipHostFree(peer_tab);
   if (ev0) (void)hipEventDestroy(ev0);
   if (ev1) (void)hipEventDestroy(ev1);
   for (auto &m : marks) { (void)hipEventDestroy(m.a); (void)hipEventDestroy(m.b); }
@@ -701,6 +692,7 @@ Group::~Group() {
   if (ev_index) (void)hipEventDestroy(ev_index);
   if (ev_keys) (void)hipEventDestroy(ev_keys);
   if (ev_push) (void)hipEventDestroy(ev_push);
+  if (owner_host) (void)hipHostFree(owner_host);
 }
 
 void Group::join(Shard *s) {
@@ -757,6 +749,18 @@ void Group::collect_marks() {
   marks.clear();
 }
 
+// handleGradient + handleQuery of every shard (csrc/core/hetu_gpu_table.cu:27-31): one set of launches for the group
+void Group::owner_side() {
+  if (!owner_host) {
+    HCTR_HIP(hipHostMalloc((void **)&owner_host, (size_t)nrank * sizeof(OwnerShard), hipHostMallocDefault));
+    owner_dev.reserve((size_t)nrank * sizeof(OwnerShard));
+  }
+  for (Shard *m : members) m->fill_owner_args(owner_host[m->cfg.rank]);
+  StageScope st(*this, S_OWNER);
+  HCTR_HIP(hipMemcpyAsync(owner_dev.p, owner_host, (size_t)nrank * sizeof(OwnerShard), hipMemcpyHostToDevice, stream));
+  launch_owner_side(stream, owner_dev.as<OwnerShard>(), owner_host, nrank, nrank);
+}
+
 void Group::set_defer_index(bool on) {
   std::lock_guard<std::mutex> lk(mu_);
   flush_index();
@@ -773,22 +777,31 @@ void Group::set_stage_timing(bool on) {
   }
 }
 
+// Descriptors travel host -> pinned staging -> device with an asynchronous copy.  The two exchanges of a step have a
+// staging area and a device array each: nothing waits between them any more, so the second must not overwrite what the
+// first one's copy has not read yet.  A step ends with a wait, which is what makes reuse in the next step safe.
+CopyDesc *Group::reserve_descs(size_t n, int which) {
+  if (n > desc_cap[which]) {
+    HCTR_HIP(hipStreamSynchronize(stream)); // the old arrays may still be read by a copy or a launch in flight
+    if (desc_host[which]) HCTR_HIP(hipHostFree(desc_host[which]));
+    desc_host[which] = nullptr;
+    desc_cap[which] = n * 2;
+    HCTR_HIP(hipHostMalloc((void **)&desc_host[which], desc_cap[which] * sizeof(CopyDesc), hipHostMallocDefault));
+  }
+  desc_dev[which].reserve(desc_cap[which] * sizeof(CopyDesc));
+  return desc_dev[which].as<CopyDesc>();
+}
+
 void Group::run_copies(std::vector<CopyDesc> &descs) {
   if (descs.empty()) return;
   StageScope st(*this, S_EXCHANGE);
-  if (descs.size() > desc_cap) {
-    if (desc_host) HCTR_HIP(hipHostFree(desc_host));
-    desc_host = nullptr;
-    desc_cap = descs.size() * 2;
-    HCTR_HIP(hipHostMalloc((void **)&desc_host, desc_cap * sizeof(CopyDesc), hipHostMallocDefault));
-  }
-  desc_dev.reserve(desc_cap * sizeof(CopyDesc));
-  memcpy(desc_host, descs.data(), descs.size() * sizeof(CopyDesc));
-  HCTR_HIP(hipMemcpyAsync(desc_dev.p, desc_host, descs.size() * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
+  CopyDesc *dev = reserve_descs(descs.size(), 0);
+  memcpy(desc_host[0], descs.data(), descs.size() * sizeof(CopyDesc));
+  HCTR_HIP(hipMemcpyAsync(dev, desc_host[0], descs.size() * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
   size_t max_bytes = 0;
   for (auto &d : descs) max_bytes = std::max(max_bytes, d.bytes);
   for (size_t lo = 0; lo < descs.size(); lo += 32768)
-    launch_copies(stream, desc_dev.as<CopyDesc>() + lo, (uint32_t)std::min<size_t>(32768, descs.size() - lo), max_bytes);
+    launch_copies(stream, dev + lo, (uint32_t)std::min<size_t>(32768, descs.size() - lo), max_bytes);
   descs.clear();
 }
 
@@ -838,35 +851,52 @@ void Group::exchange_query() {
   run_copies(descs);
 }
 
-// csrc/core/all2all.cu:89-130: flags go back to the requesters, then versions and rows of the flagged queries
+// csrc/core/all2all.cu:89-130: flags go back to the requesters, then versions and rows of the flagged queries.
+// How many queries a requester sent to an owner is known on the host; how many of them come back with a row is only
+// known on the device, so the descriptors of those copies are written there (no wait in the middle of the step) and
+// the requester's buffers are sized for the most that can come back (every query it sent).
 void Group::exchange_return() {
   const int R = nrank;
   std::vector<CopyDesc> descs;
+  size_t max_bytes = 0;
+  if (!peer_tab) HCTR_HIP(hipHostMalloc((void **)&peer_tab, 5 * 256 * sizeof(void *), hipHostMallocDefault));
+  const uint32_t **tab_seg = (const uint32_t **)peer_tab;
+  const version_t **tab_rver = (const version_t **)(peer_tab + 256);
+  const embed_t **tab_rval = (const embed_t **)(peer_tab + 512);
+  version_t **tab_iver = (version_t **)(peer_tab + 768);
+  embed_t **tab_ival = (embed_t **)(peer_tab + 1024);
   for (int s = 0; s < R; s++) { // requester
     Shard &req = *members[s];
     const size_t W = req.cfg.width;
-    uint64_t rows = 0;
-    for (int d = 0; d < R; d++) rows += members[d]->ret_seg[s + 1] - members[d]->ret_seg[s];
-    req.in_rows = rows;
-    req.got.reserve((size_t)std::max<uint32_t>(req.cur.U, 1) * 4);
-    req.in_ver.reserve(std::max<uint64_t>(rows, 1) * sizeof(version_t));
-    req.in_val.reserve(std::max<uint64_t>(rows, 1) * W * sizeof(embed_t));
-    uint64_t uoff = 0, roff = 0;
+    const size_t rows_ub = std::max<uint32_t>(req.cur.U, 1); // a row per unique key at most
+    req.got.reserve(rows_ub * 4);
+    req.in_ver.reserve(rows_ub * sizeof(version_t));
+    req.in_val.reserve(rows_ub * W * sizeof(embed_t));
+    uint64_t uoff = 0;
     for (int d = 0; d < R; d++) { // owner, in rank order
       Shard &own = *members[d];
       const uint64_t qn = own.rq_seg[s + 1] - own.rq_seg[s];
       if (qn) descs.push_back({own.outdated.as<uint32_t>() + own.rq_seg[s], req.got.as<uint32_t>() + uoff, qn * 4});
-      const uint64_t rn = own.ret_seg[s + 1] - own.ret_seg[s];
-      if (rn) {
-        descs.push_back({own.ret_ver.as<version_t>() + own.ret_seg[s], req.in_ver.as<version_t>() + roff, rn * sizeof(version_t)});
-        descs.push_back({own.ret_val.as<embed_t>() + own.ret_seg[s] * W, req.in_val.as<embed_t>() + roff * W, rn * W * sizeof(embed_t)});
-      }
+      max_bytes = std::max(max_bytes, (size_t)qn * W * sizeof(embed_t));
       uoff += qn;
-      roff += rn;
     }
     HCTR_CHECK(uoff == req.cur.U, "internal: returned flags do not cover the unique keys");
+    tab_seg[s] = req.ret_seg_dev.as<uint32_t>();
+    tab_rver[s] = req.ret_ver.as<version_t>();
+    tab_rval[s] = req.ret_val.as<embed_t>();
+    tab_iver[s] = req.in_ver.as<version_t>();
+    tab_ival[s] = req.in_val.as<embed_t>();
   }
-  run_copies(descs);
+  StageScope st(*this, S_EXCHANGE);
+  const size_t n_host = descs.size(), n_dev = 2 * (size_t)R * R;
+  CopyDesc *dev = reserve_descs(n_host + n_dev, 1);
+  if (n_host) {
+    memcpy(desc_host[1], descs.data(), n_host * sizeof(CopyDesc));
+    HCTR_HIP(hipMemcpyAsync(dev, desc_host[1], n_host * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
+  }
+  launch_build_return_descs(stream, tab_seg, tab_rver, tab_rval, tab_iver, tab_ival, R, members[0]->tv.width, dev + n_host);
+  for (size_t lo = 0; lo < n_host + n_dev; lo += 32768)
+    launch_copies(stream, dev + lo, (uint32_t)std::min<size_t>(32768, n_host + n_dev - lo), max_bytes);
 }
 
 // csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
@@ -973,6 +1003,11 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     {
       StreamSwitch on(*this, index_stream);
       for (Shard *m : members) {
+        if (m->cur.n == 0) { // an empty batch (a shard that only serves): nothing to launch, nothing to read back
+          m->mirror->st.U = 0;
+          for (int i = 0; i <= nrank; i++) m->mirror->st.send_cnt[i] = 0;
+          continue;
+        }
         m->index_batch();
         m->enqueue_readback_index();
       }
@@ -1086,11 +1121,8 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
   }
   if (nrank > 1) {
     exchange_query();
-    for (Shard *m : members) m->handle_gradient();
-    for (Shard *m : members) m->handle_query();
-    sync_stream(); // hetu_gpu_table.cu:33: the return counts size the next exchange
-    collect_marks();
-    for (Shard *m : members) m->finish_handle_query();
+    owner_side();
+    // the reference waits here for the return counts (hetu_gpu_table.cu:33); they stay on the device
     exchange_return();
   }
   for (Shard *m : members) m->write_back(dsts[m->cfg.rank], bag);
@@ -1106,11 +1138,18 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
     HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
     HCTR_HIP(hipEventElapsedTime(&push_ms, ev0, ev_push));
   }
+  std::string first_error;
   for (Shard *m : members) {
     m->last_pp_ms = ms;
     m->last_push_ms = push_ms;
-    m->finish_push_pull();
+    try {
+      if (nrank > 1) m->finish_handle_query();
+      m->finish_push_pull();
+    } catch (const Error &e) {
+      if (first_error.empty()) first_error = e.what();
+    }
   }
+  if (!first_error.empty()) throw Error(first_error);
 }
 
 // Rendezvous of the nrank per-shard callers: the last one to arrive runs the step for all.
