@@ -98,8 +98,10 @@ void launch_decide_update(hipStream_t s, const TableView &t, const KeyLayout &kl
                           uint32_t *need);
 // pushed rows per owner from the scanned plan: cnt[d] = prefix[lo[d+1]] - prefix[lo[d]]
 void launch_bucket_counts(hipStream_t s, const BatchView &b, const uint32_t *prefix, const uint32_t *total,
-                          int nrank, uint64_t *cnt_out);
-void launch_bucket_sizes(hipStream_t s, const BatchView &b, int nrank, uint64_t *cnt_out);
+                          int nrank, uint64_t *cnt_out, uint64_t *host_out);
+// both also write their counts to host_out (pinned host memory), bucket_sizes the number of unique keys to host_U
+void launch_bucket_sizes(hipStream_t s, const BatchView &b, int nrank, uint64_t *cnt_out, uint64_t *host_out,
+                         uint32_t *host_U);
 
 // Division of a batch position by the bag size of sum-pooled lookups without a divide instruction: for any 32-bit
 // n and bag >= 2, n / bag == (((n - q) >> 1) + q) >> shift with q = high word of n * magic (the "round up, add back"
@@ -172,6 +174,7 @@ struct OwnerShard {
   uint32_t rq_seg[258];
   uint32_t q, query_tiles;
   uint32_t *outdated, *tile_cnt, *out_pos;
+  slot_t *q_slot;            // slot of every received query (kNoSlot: not owned here)
   version_t *ret_ver;
   embed_t *ret_val;
   uint32_t *err;             // the shard's error word

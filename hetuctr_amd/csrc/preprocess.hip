@@ -265,21 +265,29 @@ __global__ __launch_bounds__(kBlock) void decide_update(TableView t, int id_bits
 }
 
 __global__ void bucket_counts(BatchView b, const uint32_t *__restrict__ prefix, const uint32_t *__restrict__ total,
-                              int nrank, uint64_t *__restrict__ cnt_out) {
+                              int nrank, uint64_t *__restrict__ cnt_out, uint64_t *__restrict__ host_out) {
   const int d = threadIdx.x;
   if (d > nrank) return;
-  if (d == nrank) { cnt_out[d] = 0; return; }
-  const uint32_t U = *b.d_U;
-  const uint32_t lo = b.bucket_lo[d], hi = b.bucket_lo[d + 1];
-  const uint32_t a = lo >= U ? *total : prefix[lo];
-  const uint32_t e = hi >= U ? *total : prefix[hi];
-  cnt_out[d] = U ? (uint64_t)(e - a) : 0;
+  uint64_t c = 0;
+  if (d < nrank) {
+    const uint32_t U = *b.d_U;
+    const uint32_t lo = b.bucket_lo[d], hi = b.bucket_lo[d + 1];
+    const uint32_t a = lo >= U ? *total : prefix[lo];
+    const uint32_t e = hi >= U ? *total : prefix[hi];
+    c = U ? (uint64_t)(e - a) : 0;
+  }
+  cnt_out[d] = c;
+  host_out[d] = c; // pinned host memory: the caller sizes the push buffers from it, no copy in between
 }
 
-__global__ void bucket_sizes(BatchView b, int nrank, uint64_t *__restrict__ cnt_out) {
+__global__ void bucket_sizes(BatchView b, int nrank, uint64_t *__restrict__ cnt_out, uint64_t *__restrict__ host_out,
+                             uint32_t *__restrict__ host_U) {
   const int d = threadIdx.x;
   if (d > nrank) return;
-  cnt_out[d] = d == nrank ? 0 : (uint64_t)(b.bucket_lo[d + 1] - b.bucket_lo[d]);
+  const uint64_t c = d == nrank ? 0 : (uint64_t)(b.bucket_lo[d + 1] - b.bucket_lo[d]);
+  cnt_out[d] = c;
+  host_out[d] = c; // pinned host memory, like the number of unique keys beside it
+  if (d == 0) *host_U = *b.d_U;
 }
 
 } // namespace
@@ -351,13 +359,14 @@ void launch_decide_update(hipStream_t s, const TableView &t, const KeyLayout &kl
 }
 
 void launch_bucket_counts(hipStream_t s, const BatchView &b, const uint32_t *prefix, const uint32_t *total,
-                          int nrank, uint64_t *cnt_out) {
-  hipLaunchKernelGGL(bucket_counts, dim3(1), dim3(nrank + 1), 0, s, b, prefix, total, nrank, cnt_out);
+                          int nrank, uint64_t *cnt_out, uint64_t *host_out) {
+  hipLaunchKernelGGL(bucket_counts, dim3(1), dim3(nrank + 1), 0, s, b, prefix, total, nrank, cnt_out, host_out);
   HCTR_HIP(hipGetLastError());
 }
 
-void launch_bucket_sizes(hipStream_t s, const BatchView &b, int nrank, uint64_t *cnt_out) {
-  hipLaunchKernelGGL(bucket_sizes, dim3(1), dim3(nrank + 1), 0, s, b, nrank, cnt_out);
+void launch_bucket_sizes(hipStream_t s, const BatchView &b, int nrank, uint64_t *cnt_out, uint64_t *host_out,
+                         uint32_t *host_U) {
+  hipLaunchKernelGGL(bucket_sizes, dim3(1), dim3(nrank + 1), 0, s, b, nrank, cnt_out, host_out, host_U);
   HCTR_HIP(hipGetLastError());
 }
 

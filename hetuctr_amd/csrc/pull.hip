@@ -46,6 +46,24 @@ __device__ __forceinline__ uint32_t lower_bound_id(const index_t *__restrict__ a
   }
   return lo;
 }
+#ifndef HCTR_APPLY_AHEAD
+#define HCTR_APPLY_AHEAD 2
+#endif
+#ifndef HCTR_APPLY_BATCHES
+#define HCTR_APPLY_BATCHES 1
+#endif
+// Rows of one source a group works on together (distinct ids, hence distinct targets), and batches of that many rows
+// per group and block.  Small blocks measured fastest: the kernel is a stream of independent read-modify-writes, and
+// what limits it is how evenly the blocks spread over the chip, not the loads one wave keeps in flight.
+constexpr int kApplyAhead = HCTR_APPLY_AHEAD;
+constexpr int kApplyBatches = HCTR_APPLY_BATCHES;
+// The slot of an id the shard owns, kNoSlot for any other id.  Slots below n_cached hold the cached copies of rows
+// other shards own, so the slot alone tells (no look at the owner table).
+__device__ __forceinline__ slot_t owned_slot(const slot_t *__restrict__ slot, uint64_t id, uint64_t id_max, uint32_t n_cached) {
+  if (id >= id_max) return kNoSlot;
+  const slot_t o = slot[id];
+  return (o != kNoSlot && (uint32_t)o >= n_cached) ? o : kNoSlot;
+}
 template <int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__restrict__ shards, int nsrc,
                                                            uint32_t rows_per_block) {
@@ -53,8 +71,14 @@ __global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__r
   constexpr int kGroups = kBlock / LPR;
   const OwnerShard &S = shards[blockIdx.y];
   if (blockIdx.x >= S.push_blocks) return;
-  const TableView &t = S.t;
   const index_t *__restrict__ rg_idx = S.rg_idx;
+  const version_t *__restrict__ rg_cnt = S.rg_cnt;
+  const embed_t *__restrict__ rg_val = S.rg_val;
+  const slot_t *__restrict__ slot = S.t.slot;
+  embed_t *__restrict__ emb = S.t.emb;
+  version_t *__restrict__ ver = S.t.ver;
+  const uint64_t id_max = S.t.id_max;
+  const uint32_t n_cached = S.t.n_cached, W = S.t.width;
   __shared__ uint32_t lo[256], hi[256];
   const int longest = S.longest;
   const uint32_t big_lo = S.rg_seg[longest], big_hi = S.rg_seg[longest + 1];
@@ -73,47 +97,43 @@ __global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__r
     }
   }
   __syncthreads();
-  const uint32_t gl = threadIdx.x % LPR, W = t.width;
-  constexpr int kAhead = 4; // rows of one source a group works on together (distinct ids, hence distinct targets)
+  const uint32_t gl = threadIdx.x % LPR;
+  constexpr int kAhead = kApplyAhead;
+  bool bad = false;
   for (int s = 0; s < nsrc; s++) {
-    for (uint32_t k0 = lo[s] + threadIdx.x / LPR; k0 < hi[s]; k0 += kGroups * kAhead) {
+    const uint32_t end = hi[s];
+    for (uint32_t k0 = lo[s] + threadIdx.x / LPR; k0 < end; k0 += kGroups * kAhead) {
       slot_t o[kAhead];
       uint64_t id[kAhead];
 #pragma unroll
-      for (int a = 0; a < kAhead; a++) id[a] = (uint64_t)rg_idx[min(k0 + a * kGroups, hi[s] - 1)];
+      for (int a = 0; a < kAhead; a++) id[a] = (uint64_t)rg_idx[min(k0 + a * kGroups, end - 1)];
 #pragma unroll
       for (int a = 0; a < kAhead; a++) {
-        const bool mine = id[a] < t.id_max && t.root[min(id[a], t.id_max - 1)] == t.rank;
-        o[a] = mine ? t.slot[id[a]] : kNoSlot;
-      }
-      bool bad = false;
-#pragma unroll
-      for (int a = 0; a < kAhead; a++) {
-        const uint32_t k = k0 + a * kGroups;
-        if (k >= hi[s]) o[a] = kNoSlot;
+        o[a] = owned_slot(slot, id[a], id_max, n_cached);
+        if (k0 + a * kGroups >= end) o[a] = kNoSlot;
         else if (o[a] == kNoSlot) bad = true;
       }
-      if (bad && gl == 0) atomicOr(S.err, 2u);
       if (gl == 0) {
 #pragma unroll
         for (int a = 0; a < kAhead; a++)
-          if (o[a] != kNoSlot) t.ver[o[a]] += S.rg_cnt[k0 + a * kGroups];
+          if (o[a] != kNoSlot) ver[o[a]] += load_once(rg_cnt + k0 + a * kGroups);
       }
       for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
         V cur[kAhead], add[kAhead];
 #pragma unroll
         for (int a = 0; a < kAhead; a++) {
           if (o[a] == kNoSlot) continue;
-          cur[a] = *(const V *)(t.emb + (size_t)o[a] * W + col);
-          add[a] = *(const V *)(S.rg_val + (size_t)(k0 + a * kGroups) * W + col);
+          cur[a] = *(const V *)(emb + (size_t)o[a] * W + col);
+          add[a] = load_once((const V *)(rg_val + (size_t)(k0 + a * kGroups) * W + col)); // read once: keep it out of the caches
         }
 #pragma unroll
         for (int a = 0; a < kAhead; a++)
-          if (o[a] != kNoSlot) *(V *)(t.emb + (size_t)o[a] * W + col) = cur[a] + add[a];
+          if (o[a] != kNoSlot) *(V *)(emb + (size_t)o[a] * W + col) = cur[a] + add[a];
       }
     }
     __syncthreads(); // the next source may push to the same rows
   }
+  if (bad && gl == 0) atomicOr(S.err, 2u);
 }
 
 // Owner side of the pull (csrc/core/handle_query.cu:7-78) in three launches; the first two work on tiles of kBlock
@@ -131,9 +151,8 @@ __global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restr
   const uint32_t k = blockIdx.x * kBlock + threadIdx.x;
   uint32_t flag = 0;
   if (k < S.q) {
-    const uint64_t id = (uint64_t)S.rq_idx[k];
-    slot_t o = kNoSlot;
-    if (id < t.id_max && t.root[id] == t.rank) o = t.slot[id];
+    const slot_t o = owned_slot(t.slot, (uint64_t)S.rq_idx[k], t.id_max, t.n_cached);
+    S.q_slot[k] = o;
     if (o == kNoSlot) {
       atomicOr(S.err, 4u);
     } else {
@@ -187,21 +206,41 @@ __global__ __launch_bounds__(kBlock) void scan_positions(const OwnerShard *__res
   if (last_block && threadIdx.x == 0) S.seg_host[257] = *S.err;
 }
 
-// one group of LPR lanes per received query
+// kPackAhead received queries per group of LPR lanes; the slot of every query was left by decide_count
+constexpr int kPackAhead = 2;
 template <int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict__ shards) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
   const OwnerShard &S = shards[blockIdx.y];
-  const TableView &t = S.t;
-  const uint32_t k = blockIdx.x * kGroups + threadIdx.x / LPR;
-  if (k >= S.q || !S.outdated[k]) return;
-  const uint32_t gl = threadIdx.x % LPR, W = t.width;
-  const slot_t o = t.slot[(uint64_t)S.rq_idx[k]];
-  const uint32_t pos = S.out_pos[k];
-  if (gl == 0) S.ret_ver[pos] = t.ver[o];
-  for (uint32_t col = gl * VEC; col < W; col += LPR * VEC)
-    *(V *)(S.ret_val + (size_t)pos * W + col) = *(const V *)(t.emb + (size_t)o * W + col);
+  const uint32_t q = S.q;
+  const uint32_t k0 = blockIdx.x * (kGroups * kPackAhead) + threadIdx.x / LPR;
+  if (k0 >= q) return;
+  const embed_t *__restrict__ emb = S.t.emb;
+  embed_t *__restrict__ ret_val = S.ret_val;
+  const uint32_t gl = threadIdx.x % LPR, W = S.t.width;
+  slot_t o[kPackAhead];
+  uint32_t pos[kPackAhead];
+#pragma unroll
+  for (int a = 0; a < kPackAhead; a++) {
+    const uint32_t k = min(k0 + a * kGroups, q - 1);
+    o[a] = (k0 + a * kGroups < q && S.outdated[k]) ? S.q_slot[k] : kNoSlot;
+    pos[a] = S.out_pos[k];
+  }
+  if (gl == 0) {
+#pragma unroll
+    for (int a = 0; a < kPackAhead; a++)
+      if (o[a] != kNoSlot) S.ret_ver[pos[a]] = S.t.ver[o[a]];
+  }
+  for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
+    V v[kPackAhead];
+#pragma unroll
+    for (int a = 0; a < kPackAhead; a++)
+      if (o[a] != kNoSlot) v[a] = *(const V *)(emb + (size_t)o[a] * W + col);
+#pragma unroll
+    for (int a = 0; a < kPackAhead; a++)
+      if (o[a] != kNoSlot) *(V *)(ret_val + (size_t)pos[a] * W + col) = v[a];
+  }
 }
 
 // The copies of the return exchange (csrc/core/all2all.cu:89-130) described on the device: how many rows an owner
@@ -445,7 +484,7 @@ size_t query_tiles(uint32_t q) { return std::max<size_t>(1, div_up(q, kBlock)); 
 
 uint32_t owner_push_rows_per_block(uint32_t width) {
   const int lpr = lanes_for(width, width % 4 == 0 ? 4 : 1);
-  return 4 * 4 * (kBlock / lpr); // four batches of kAhead rows per group
+  return kApplyBatches * kApplyAhead * (kBlock / lpr);
 }
 
 void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerShard *shards_host, int nshards, int nsrc) {
@@ -469,7 +508,7 @@ void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerS
   hipLaunchKernelGGL(scan_positions, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
   if (q_max) {
 #define CALL(V, L) \
-  hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q_max, kBlock / L), nshards), dim3(kBlock), 0, s, shards_dev)
+  hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q_max, kPackAhead * (kBlock / L)), nshards), dim3(kBlock), 0, s, shards_dev)
     HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   }

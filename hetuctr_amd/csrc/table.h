@@ -77,7 +77,6 @@ struct DevStat {
 };
 struct HostMirror {
   DevStat st;
-  uint32_t ret_total;
   uint32_t stats[4];
   uint32_t ret_seg[258];
   uint32_t key_err; // written by the kernel that reads the caller's ids when preprocess returns early (no copy)
@@ -122,8 +121,6 @@ class Shard {
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
   // the same in two halves, for a preprocess whose push plan and index run on different streams
-  void enqueue_readback_plan();
-  void enqueue_readback_index();
   void finish_plan();
   void finish_index();
   void check_key_error();                   // raises if the ingested batch held a key outside [0, length)
@@ -155,7 +152,7 @@ class Shard {
   // send side
   DeviceBuf q_idx, q_ver, g_idx, g_cnt, g_val;
   // receive side (owner role)
-  DeviceBuf rq_idx, rq_ver, rg_idx, rg_cnt, rg_val, outdated, out_pos, ret_total, ret_ver, ret_val, ret_seg_dev;
+  DeviceBuf rq_idx, rq_ver, rg_idx, rg_cnt, rg_val, outdated, out_pos, q_slot, ret_ver, ret_val, ret_seg_dev;
   std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
   // requester side of the return
   DeviceBuf got, ret_i, in_ver, in_val;

@@ -173,7 +173,6 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   dstat.reserve(sizeof(DevStat));
   dst_ = dstat.as<DevStat>();
   stats.reserve(32);
-  ret_total.reserve(4);
   ret_seg_dev.reserve(2 * 258 * 4);
   HCTR_HIP(hipMemsetAsync(dstat.p, 0, dstat.bytes, s));
   HCTR_HIP(hipMemsetAsync(stats.p, 0, 32, s));
@@ -322,7 +321,7 @@ void Shard::index_batch(uint32_t *u_out, int part) {
     launch_list_long_runs(s, cur.view());
   }
   if (part == 1) return;
-  if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt);
+  if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt, mirror->st.send_cnt, &mirror->st.U);
 }
 
 // csrc/core/preprocess.cu:148-182
@@ -336,6 +335,7 @@ void Shard::preprocess_gradient() {
       HCTR_HIP(hipMemsetAsync(&dst_->push_total, 0, 4, s));
       plan_cleared = true;
     }
+    for (int i = 0; i <= cfg.nrank; i++) mirror->st.push_cnt[i] = 0; // nothing in flight writes the block
     return;
   }
   plan_cleared = false;
@@ -346,7 +346,7 @@ void Shard::preprocess_gradient() {
   launch_decide_update(s, tv, kl, prev.view(), need.as<uint32_t>());
   launch_exclusive_scan(s, need.as<uint32_t>(), prefix.as<uint32_t>(), prev.n, prev.dU.as<uint32_t>(),
                         plan_sums.as<uint32_t>(), &dst_->push_total);
-  launch_bucket_counts(s, prev.view(), prefix.as<uint32_t>(), &dst_->push_total, cfg.nrank, cnt);
+  launch_bucket_counts(s, prev.view(), prefix.as<uint32_t>(), &dst_->push_total, cfg.nrank, cnt, mirror->st.push_cnt);
 }
 
 void Shard::enqueue_readback_preprocess() {
@@ -364,24 +364,9 @@ void Shard::finish_preprocess() {
   finish_index();
 }
 
-// The two halves of the read-back: what the push plan of the previous batch produced (rows pushed per owner) and what
-// the index of the current batch produced (unique keys, queries per owner, the error word).
-void Shard::enqueue_readback_plan() {
-  if (cfg.nrank == 1) return;
-  HCTR_HIP(hipMemcpyAsync(mirror->st.push_cnt, dst_->push_cnt, (size_t)(cfg.nrank + 1) * sizeof(uint64_t),
-                          hipMemcpyDeviceToHost, group->stream));
-}
-
-void Shard::enqueue_readback_index() {
-  hipStream_t s = group->stream;
-  if (cur.n == 0 && !u_cleared) {
-    HCTR_HIP(hipMemsetAsync(&dst_->U, 0, 4, s));
-    u_cleared = true;
-  }
-  const size_t bytes = offsetof(DevStat, send_cnt) + (size_t)(cfg.nrank + 1) * sizeof(uint64_t);
-  HCTR_HIP(hipMemcpyAsync(&mirror->st, dstat.p, bytes, hipMemcpyDeviceToHost, s));
-}
-
+// The two halves of what preprocess hands to the host, each written to the pinned block by the kernel that computes it:
+// what the push plan of the previous batch produced (rows pushed per owner) and what the index of the current batch
+// produced (unique keys, queries per owner).
 void Shard::finish_plan() {
   prev_active = prev.n > 0;
   if (cfg.nrank == 1) prev.push_cnt[0] = 0;
@@ -466,6 +451,7 @@ void Shard::fill_owner_args(OwnerShard &o) {
   const uint32_t Q = (uint32_t)rq_seg[R];
   outdated.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
   out_pos.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
+  q_slot.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(slot_t));
   ret_ver.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(version_t));
   ret_val.reserve((size_t)std::max<uint32_t>(Q, 1) * cfg.width * sizeof(embed_t));
   query_sums.reserve((query_tiles(Q) + 2) * 4);
@@ -489,6 +475,7 @@ void Shard::fill_owner_args(OwnerShard &o) {
   o.outdated = outdated.as<uint32_t>();
   o.tile_cnt = query_sums.as<uint32_t>();
   o.out_pos = out_pos.as<uint32_t>();
+  o.q_slot = q_slot.as<slot_t>();
   o.ret_ver = ret_ver.as<version_t>();
   o.ret_val = ret_val.as<embed_t>();
   o.err = err_ptr();
@@ -996,7 +983,6 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     HCTR_HIP(hipEventRecord(ev_keys, stream));
     for (Shard *m : members) {
       m->preprocess_gradient();
-      m->enqueue_readback_plan();
     }
     if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
     HCTR_HIP(hipStreamWaitEvent(index_stream, ev_keys, 0));
@@ -1009,7 +995,6 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
           continue;
         }
         m->index_batch();
-        m->enqueue_readback_index();
       }
     }
     index_pending = true;
