@@ -132,6 +132,7 @@ void Shard::load(const char *path) {
     b->n = 0;
     b->U = 0;
     b->idx_map_valid = false;
+    b->planned = false;
     b->clear(s, cfg.nrank);
     std::fill(b->send_cnt.begin(), b->send_cnt.end(), 0);
     std::fill(b->recv_cnt.begin(), b->recv_cnt.end(), 0);

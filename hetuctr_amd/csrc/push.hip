@@ -107,6 +107,28 @@ template <> struct Vec<1> {
   static __device__ __forceinline__ T scale(const T &a, float s) { return a * s; }
 };
 
+// The version / update counters of unique rank u and its entry among the pushed rows (gradient_index_kernel,
+// generate_query.cu:51-83).  type: the update type of generate_query.cu:18-25; q: the row's place among the pushed rows.
+template <typename K>
+__device__ __forceinline__ void move_counters(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
+                                              uint32_t u, slot_t o, int type, uint32_t q) {
+  version_t cnt = (version_t)(p.run_start[u + 1] - p.run_start[u]);
+  if (type == 1) t.ver[o] += cnt;
+  else if (type >= 2) {
+    version_t up = t.upd[o] + cnt;
+    if (type == 2) {
+      cnt = up;
+      up = 0;
+      t.ver[o] += cnt;
+    }
+    t.upd[o] = up;
+  }
+  if (type == 0 || type == 2) { // the rows the plan marks as pushed
+    a.g_idx[q] = (index_t)(((const K *)p.ukey)[u] & (K)(((uint64_t)1 << id_bits) - 1));
+    a.g_cnt[q] = cnt;
+  }
+}
+
 // Applies the finished sum of unique rank u (already multiplied by -lr) to column(s) `col`.
 // `counters`: this lane also moves the version / update counters.  Update types as in generate_query.cu:18-25.
 template <int VEC, typename K>
@@ -144,23 +166,7 @@ __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const
     }
     *g = pg;
   }
-  if (counters) { // gradient_index_kernel, generate_query.cu:51-83
-    version_t cnt = (version_t)(p.run_start[u + 1] - p.run_start[u]);
-    if (type == 1) t.ver[o] += cnt;
-    else if (type >= 2) {
-      version_t up = t.upd[o] + cnt;
-      if (type == 2) {
-        cnt = up;
-        up = 0;
-        t.ver[o] += cnt;
-      }
-      t.upd[o] = up;
-    }
-    if (need) {
-      a.g_idx[q] = (index_t)(((const K *)p.ukey)[u] & (K)(((uint64_t)1 << id_bits) - 1));
-      a.g_cnt[q] = cnt;
-    }
-  }
+  if (counters) move_counters<K>(t, id_bits, p, a, u, o, type, q);
 }
 
 // ---- short role ----------------------------------------------------------------------------------------
@@ -194,6 +200,20 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
   for (int i = 0; i <= G; i++) rs[i] = run_start[min(u0 + i, U)];
 #pragma unroll
   for (int i = 0; i < G; i++) off[i] = p.uoff[min(u0 + i, U - 1)];
+  // several shards: the update type of every run (generate_query.cu:18-25) and its place among the pushed rows
+  int type[G];
+  uint32_t q[G];
+  if (!kSingle) {
+    uint32_t nd[G];
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+      nd[i] = a.need[min(u0 + i, U - 1)];
+      q[i] = a.prefix[min(u0 + i, U - 1)];
+    }
+#pragma unroll
+    for (int i = 0; i < G; i++)
+      type[i] = off[i] == kNoSlot ? 0 : ((uint32_t)off[i] >= t.n_cached ? 1 : (nd[i] ? 2 : 3));
+  }
   const float neg_lr = t.neg_lr;
 
   for (uint32_t c0 = 0; c0 < W; c0 += LPR * VEC) {
@@ -201,7 +221,7 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
     const bool active = col < W;
     uint32_t len[G];
     bool mine[G];
-    V e[G];
+    V e[G], pg[G];
     uint32_t si[G][kHead];
     V v[G][kHead];
 #pragma unroll
@@ -209,11 +229,17 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
       len[i] = rs[i + 1] - rs[i];
       mine[i] = u0 + i < U && len[i] <= kTinyRun && active;
     }
-    if (kSingle) {
+    // the rows the sums will be added to are requested before the gradient rows, not after the sums are done
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+      e[i] = Vec<VEC>::zero();
+      if (mine[i] && (kSingle || type[i] != 0)) e[i] = *(const V *)(t.emb + (size_t)off[i] * W + col);
+    }
+    if (!kSingle) {
 #pragma unroll
       for (int i = 0; i < G; i++) {
-        e[i] = Vec<VEC>::zero();
-        if (mine[i]) e[i] = *(const V *)(t.emb + (size_t)off[i] * W + col);
+        pg[i] = Vec<VEC>::zero();
+        if (mine[i] && type[i] >= 2) pg[i] = *(const V *)(t.pend + (size_t)off[i] * W + col);
       }
     }
 #pragma unroll
@@ -256,7 +282,24 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
         Vec<VEC>::add(r, scaled);
         *(V *)(t.emb + (size_t)off[i] * W + col) = r; // the version counters move in the last blocks of the launch
       } else {
-        apply_row<VEC, K>(t, id_bits, p, a, u0 + i, scaled, col, c0 == 0 && gl == 0);
+        // the same updates as apply_row(), with the rows already here
+        if (type[i] != 0) {
+          V r = e[i];
+          Vec<VEC>::add(r, scaled);
+          *(V *)(t.emb + (size_t)off[i] * W + col) = r;
+        } else {
+          *(V *)(a.g_val + (size_t)q[i] * W + col) = scaled;
+        }
+        if (type[i] >= 2) {
+          V g = pg[i];
+          Vec<VEC>::add(g, scaled);
+          if (type[i] == 2) {
+            *(V *)(a.g_val + (size_t)q[i] * W + col) = g;
+            g = Vec<VEC>::zero();
+          }
+          *(V *)(t.pend + (size_t)off[i] * W + col) = g;
+        }
+        if (c0 == 0 && gl == 0) move_counters<K>(t, id_bits, p, a, u0 + i, off[i], type[i], q[i]);
       }
     }
   }

@@ -54,9 +54,11 @@ struct Batch {
   uint32_t U = 0;   // unique keys (host copy, valid after the preprocess call returned)
   bool idx_map_valid = false;
   bool cleared = false; // the device side reads as an empty batch (U = 0, no buckets, no runs) since clear()
+  bool planned = false; // the push plan (need, prefix, push_cnt) has been computed for the batch as it stands
   // comp: the batch's sort keys in batch order (id and owner of every position); staged: ids that arrived in
   // pageable host memory, on their way to the key kernel
   DeviceBuf comp, staged, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong, med_list;
+  DeviceBuf need, prefix, plan_total; // push plan per unique key: pushed or not, position among the pushed rows; their number
   std::vector<uint64_t> send_cnt, recv_cnt;       // queries per owner / per requester
   std::vector<uint64_t> push_cnt, pushrecv_cnt;   // pushed rows per owner / per source
   void reserve(uint32_t n_keys, int nrank, bool wide);
@@ -117,11 +119,11 @@ class Shard {
   // sort, unique, run lists of the ingested batch; u_out: where the number of unique keys goes besides the batch's
   // own device word (default: the device block that is read back after the call)
   void index_batch(uint32_t *u_out = nullptr, int part = 0);
-  void preprocess_gradient();
+  void plan_batch(Batch &b);  // enqueues the push plan of b; its counts reach the host when the stream has run it
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
   // the same in two halves, for a preprocess whose push plan and index run on different streams
-  void finish_plan();
+  void finish_plan(Batch &b); // takes the counts over into b once they are there
   void finish_index();
   void check_key_error();                   // raises if the ingested batch held a key outside [0, length)
   void generate_gradient(const float *grad, uint32_t bag = 1);
@@ -146,7 +148,7 @@ class Shard {
     void *ktmp0 = nullptr, *ktmp1 = nullptr;
     uint32_t *vtmp0 = nullptr, *vtmp1 = nullptr, *sortws = nullptr, *block_sums = nullptr;
   } sp;
-  DeviceBuf need, prefix, plan_sums, query_sums; // query_sums: flags per tile of received queries // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
+  DeviceBuf plan_sums, query_sums; // query_sums: flags per tile of received queries // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
   DevStat *dst_ = nullptr; // == dstat.p
   uint32_t *err_ptr() const { return &dst_->err; }
   // send side
@@ -159,7 +161,6 @@ class Shard {
   HostMirror *mirror = nullptr;
   long long last_stats[6] = {0, 0, 0, 0, 0, 0};
   float last_pre_ms = 0.f, last_pp_ms = 0.f, last_push_ms = 0.f;
-  bool plan_cleared = false; // the device-side push counts read as zero
   bool u_cleared = false;    // the device-side copy of the number of unique keys reads as zero
 
  private:
@@ -190,11 +191,12 @@ class Group {
   // sorting and deduplicating them has no dependence on the pending gradient push, so the next push_pull starts the
   // push on the main stream right away and only the gather waits for both.
   hipStream_t index_stream = nullptr;
-  hipEvent_t ev_index = nullptr, ev_keys = nullptr, ev_push = nullptr;
+  hipEvent_t ev_index = nullptr, ev_keys = nullptr, ev_push = nullptr, ev_pushed = nullptr, ev_plan = nullptr;
   bool defer_index = false;              // the mode is on (HETUCTR_DEFER_INDEX != 0)
   bool index_pending = false;            // a batch's index is enqueued and nobody has waited for it yet
   bool index_rest_pending = false;       // single shard: preprocess enqueued only the first launches of the index
-  void enqueue_index_rest();             // enqueues the others
+  void enqueue_index_rest();
+  void enqueue_index_all(int part);             // enqueues the others
   void flush_index();                    // waits for a pending index and takes its results over
   // owner-side arguments of every shard: pinned staging and the device copy the kernels read
   OwnerShard *owner_host = nullptr;

@@ -262,6 +262,7 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
   cur.n = (uint32_t)n;
   cur.U = 0;
   cur.idx_map_valid = false;
+  cur.planned = false;
   if (!scratch_area) cur.reserve(cur.n, cfg.nrank, kl.wide); // else: the caller has checked that the buffers hold n keys
   if (n == 0) { // :93-95
     cur.clear(s, cfg.nrank);
@@ -324,29 +325,28 @@ void Shard::index_batch(uint32_t *u_out, int part) {
   if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt, mirror->st.send_cnt, &mirror->st.U);
 }
 
-// csrc/core/preprocess.cu:148-182
-void Shard::preprocess_gradient() {
+// The push plan of a batch (csrc/core/preprocess.cu:148-182): which of its remote unique keys are pushed when it is
+// the previous batch, and how many rows go to every owner.  It depends on the batch's index and on the update counters
+// of the cached rows as the push of the step before left them, and nothing changes either between the end of that
+// step and the preprocess call the reference computes the plan in: push_pull computes it for its current batch (beside
+// the owner-side work, on the second stream), and the next preprocess finds it done.
+void Shard::plan_batch(Batch &b) {
   hipStream_t s = group->stream;
-  uint64_t *cnt = dst_->push_cnt;
   if (cfg.nrank == 1) return; // single shard: every key is owned, nothing is ever pushed
-  if (prev.n == 0) {
-    if (!plan_cleared) {
-      HCTR_HIP(hipMemsetAsync(cnt, 0, (size_t)(cfg.nrank + 1) * sizeof(uint64_t), s));
-      HCTR_HIP(hipMemsetAsync(&dst_->push_total, 0, 4, s));
-      plan_cleared = true;
-    }
+  if (b.n == 0) {
     for (int i = 0; i <= cfg.nrank; i++) mirror->st.push_cnt[i] = 0; // nothing in flight writes the block
     return;
   }
-  plan_cleared = false;
-  need.reserve((size_t)prev.n * 4);
-  prefix.reserve((size_t)prev.n * 4);
-  plan_sums.reserve((scan_blocks(prev.n) + 2) * 4); // its own: the index of the current batch may be running beside it
+  b.need.reserve((size_t)b.n * 4);
+  b.prefix.reserve((size_t)b.n * 4);
+  b.plan_total.reserve(4);
+  plan_sums.reserve((scan_blocks(b.n) + 2) * 4); // its own: the index of the next batch may be running beside it
   StageScope st(*group, S_PLAN);
-  launch_decide_update(s, tv, kl, prev.view(), need.as<uint32_t>());
-  launch_exclusive_scan(s, need.as<uint32_t>(), prefix.as<uint32_t>(), prev.n, prev.dU.as<uint32_t>(),
-                        plan_sums.as<uint32_t>(), &dst_->push_total);
-  launch_bucket_counts(s, prev.view(), prefix.as<uint32_t>(), &dst_->push_total, cfg.nrank, cnt, mirror->st.push_cnt);
+  launch_decide_update(s, tv, kl, b.view(), b.need.as<uint32_t>());
+  launch_exclusive_scan(s, b.need.as<uint32_t>(), b.prefix.as<uint32_t>(), b.n, b.dU.as<uint32_t>(),
+                        plan_sums.as<uint32_t>(), b.plan_total.as<uint32_t>());
+  launch_bucket_counts(s, b.view(), b.prefix.as<uint32_t>(), b.plan_total.as<uint32_t>(), cfg.nrank, dst_->push_cnt,
+                       mirror->st.push_cnt);
 }
 
 void Shard::enqueue_readback_preprocess() {
@@ -355,23 +355,24 @@ void Shard::enqueue_readback_preprocess() {
     HCTR_HIP(hipMemsetAsync(&dst_->U, 0, 4, s));
     u_cleared = true;
   }
-  const size_t bytes = cfg.nrank == 1 ? 16 : sizeof(DevStat);
+  // unique keys, error word, queries per owner; the pushed rows per owner reach the host from their own kernel
+  const size_t bytes = cfg.nrank == 1 ? 16 : offsetof(DevStat, send_cnt) + (size_t)(cfg.nrank + 1) * sizeof(uint64_t);
   HCTR_HIP(hipMemcpyAsync(&mirror->st, dstat.p, bytes, hipMemcpyDeviceToHost, s));
 }
 
 void Shard::finish_preprocess() {
-  finish_plan();
+  if (!prev.planned) finish_plan(prev);
   finish_index();
 }
 
 // The two halves of what preprocess hands to the host, each written to the pinned block by the kernel that computes it:
 // what the push plan of the previous batch produced (rows pushed per owner) and what the index of the current batch
 // produced (unique keys, queries per owner).
-void Shard::finish_plan() {
-  prev_active = prev.n > 0;
-  if (cfg.nrank == 1) prev.push_cnt[0] = 0;
+void Shard::finish_plan(Batch &b) {
+  if (cfg.nrank == 1) b.push_cnt[0] = 0;
   else
-    for (int i = 0; i <= cfg.nrank; i++) prev.push_cnt[i] = mirror->st.push_cnt[i];
+    for (int i = 0; i <= cfg.nrank; i++) b.push_cnt[i] = mirror->st.push_cnt[i];
+  b.planned = true;
 }
 
 void Shard::finish_index() {
@@ -421,8 +422,8 @@ void Shard::generate_gradient(const float *grad, uint32_t bag) {
     g_idx.reserve(std::max<uint64_t>(pushes, 1) * sizeof(index_t));
     g_cnt.reserve(std::max<uint64_t>(pushes, 1) * sizeof(version_t));
     g_val.reserve(std::max<uint64_t>(pushes, 1) * W * sizeof(embed_t));
-    a.need = need.as<uint32_t>();
-    a.prefix = prefix.as<uint32_t>();
+    a.need = prev.need.as<uint32_t>();
+    a.prefix = prev.prefix.as<uint32_t>();
     a.g_idx = g_idx.as<index_t>();
     a.g_cnt = g_cnt.as<version_t>();
     a.g_val = g_val.as<embed_t>();
@@ -595,7 +596,7 @@ size_t Shard::fetch(int which, void *out, size_t cap) {
     case HCTR_F_NEED_UPDATE:
     case HCTR_F_UPDATE_PREFIX: {
       if (R == 1 || prev.U == 0) { std::vector<long long> z(prev.U, 0); return put64(z, prev.U, out, cap); }
-      return put64(download<uint32_t>(which == HCTR_F_NEED_UPDATE ? need.p : prefix.p, prev.U), prev.U, out, cap);
+      return put64(download<uint32_t>(which == HCTR_F_NEED_UPDATE ? prev.need.p : prev.prefix.p, prev.U), prev.U, out, cap);
     }
     case HCTR_F_PUSH_CNT: return put64(prev.push_cnt, R, out, cap);
     case HCTR_F_PUSHRECV_CNT: return put64(prev.pushrecv_cnt, R, out, cap);
@@ -654,6 +655,8 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
   HCTR_HIP(hipEventCreateWithFlags(&ev_index, hipEventDisableTiming));
   HCTR_HIP(hipEventCreateWithFlags(&ev_keys, hipEventDisableTiming));
   HCTR_HIP(hipEventCreate(&ev_push));
+  HCTR_HIP(hipEventCreateWithFlags(&ev_pushed, hipEventDisableTiming));
+  HCTR_HIP(hipEventCreateWithFlags(&ev_plan, hipEventDisableTiming));
   const char *defer = getenv("HETUCTR_DEFER_INDEX");
   defer_index = !(defer && atoi(defer) == 0);
   HCTR_HIP(hipEventCreate(&ev0));
@@ -679,6 +682,8 @@ Group::~Group() {
   if (ev_index) (void)hipEventDestroy(ev_index);
   if (ev_keys) (void)hipEventDestroy(ev_keys);
   if (ev_push) (void)hipEventDestroy(ev_push);
+  if (ev_pushed) (void)hipEventDestroy(ev_pushed);
+  if (ev_plan) (void)hipEventDestroy(ev_plan);
   if (owner_host) (void)hipHostFree(owner_host);
 }
 
@@ -913,13 +918,30 @@ static void enqueue_index(Shard *m, int part) {
   m->index_batch(&m->mirror->st.U, part);
 }
 
-// single shard: the launches of the index that preprocess left to the next call
+// several shards: one part of the index of every shard's current batch, on the second stream
+void Group::enqueue_index_all(int part) {
+  StreamSwitch on(*this, index_stream);
+  for (Shard *m : members) {
+    if (m->cur.n == 0) { // an empty batch (a shard that only serves): nothing to launch, nothing to read back
+      m->mirror->st.U = 0;
+      for (int i = 0; i <= nrank; i++) m->mirror->st.send_cnt[i] = 0;
+      continue;
+    }
+    m->index_batch(nullptr, part);
+  }
+}
+
+// the launches of the index that preprocess left to the next call
 void Group::enqueue_index_rest() {
   if (!index_rest_pending) return;
   index_rest_pending = false;
-  StreamSwitch on(*this, index_stream);
-  enqueue_index(members[0], 2);
-  HCTR_HIP(hipEventRecord(ev_index, stream));
+  if (nrank == 1) {
+    StreamSwitch on(*this, index_stream);
+    enqueue_index(members[0], 2);
+    HCTR_HIP(hipEventRecord(ev_index, stream));
+  } else {
+    enqueue_index_all(2);
+  }
   index_pending = true;
 }
 
@@ -981,30 +1003,33 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
       m->ingest_keys(keys[m->cfg.rank], n[m->cfg.rank], &m->mirror->key_err);
     }
     HCTR_HIP(hipEventRecord(ev_keys, stream));
-    for (Shard *m : members) {
-      m->preprocess_gradient();
-    }
-    if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
-    HCTR_HIP(hipStreamWaitEvent(index_stream, ev_keys, 0));
-    {
-      StreamSwitch on(*this, index_stream);
-      for (Shard *m : members) {
-        if (m->cur.n == 0) { // an empty batch (a shard that only serves): nothing to launch, nothing to read back
-          m->mirror->st.U = 0;
-          for (int i = 0; i <= nrank; i++) m->mirror->st.send_cnt[i] = 0;
-          continue;
-        }
-        m->index_batch();
+    // a previous batch that no push_pull has seen yet (two preprocess calls in a row) is planned here
+    std::vector<Shard *> late;
+    for (Shard *m : members)
+      if (!m->prev.planned) {
+        m->plan_batch(m->prev);
+        late.push_back(m);
       }
+    if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
+    // Only the first launches of the index go out here (they keep the GPU busy until the pushes arrive); the rest
+    // follows from push_pull once the push kernels are in their queue.
+    HCTR_HIP(hipStreamWaitEvent(index_stream, ev_keys, 0));
+    enqueue_index_all(1);
+    index_rest_pending = true;
+    if (!late.empty() || time_calls) {
+      sync_stream();
+    } else { // the ids have been read: the caller may reuse its buffers
+      hipError_t e;
+      while ((e = hipEventQuery(ev_keys)) == hipErrorNotReady) {
+      }
+      HCTR_HIP(e);
     }
-    index_pending = true;
-    sync_stream();
+    for (Shard *m : late) m->finish_plan(m->prev);
     float ms = 0.f;
     if (time_calls) HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
     bool bad_key = false;
     for (Shard *m : members) {
       m->last_pre_ms = ms;
-      m->finish_plan();
       bad_key |= m->mirror->key_err != 0;
       m->mirror->key_err = 0;
     }
@@ -1016,7 +1041,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
   for (Shard *m : members) {
     m->swap_batches();
     m->preprocess_index(keys[m->cfg.rank], n[m->cfg.rank]);
-    m->preprocess_gradient();
+    if (!m->prev.planned) m->plan_batch(m->prev);
     m->enqueue_readback_preprocess();
   }
   if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
@@ -1087,6 +1112,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
   if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) m->generate_gradient(grads[m->cfg.rank], bag);
   if (time_calls) HCTR_HIP(hipEventRecord(ev_push, stream));
+  if (nrank > 1) HCTR_HIP(hipEventRecord(ev_pushed, stream));
   enqueue_index_rest(); // single shard: the push is in its queue, now the rest of the current batch's index
   if (index_pending && nrank > 1) {
     // the pushes are queued; the queries are built from the index of the current batches, which the host needs too
@@ -1095,6 +1121,14 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
     wait_for(index_stream);
     for (Shard *m : members) m->finish_index();
     exchange_shapes();
+  }
+  if (nrank > 1) {
+    // the push plans of the current batches, for the step in which they are the previous ones: after the pushes of
+    // this step (they move the update counters the plan reads), beside everything else the step still does
+    StreamSwitch on(*this, index_stream);
+    HCTR_HIP(hipStreamWaitEvent(stream, ev_pushed, 0));
+    for (Shard *m : members) m->plan_batch(m->cur);
+    HCTR_HIP(hipEventRecord(ev_plan, stream));
   }
   for (Shard *m : members) m->generate_query();
   const bool join_index = index_pending;
@@ -1112,8 +1146,11 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
   }
   for (Shard *m : members) m->write_back(dsts[m->cfg.rank], bag);
   if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
+  if (nrank > 1) HCTR_HIP(hipStreamWaitEvent(stream, ev_plan, 0));
   sync_stream();
   collect_marks();
+  if (nrank > 1)
+    for (Shard *m : members) m->finish_plan(m->cur);
   if (join_index) {
     members[0]->finish_preprocess();
     exchange_shapes();
