@@ -94,6 +94,38 @@ def cpu_baseline(cfg, ks, batches, width, lr, steps):
                        "OpenMP oracle, warm" % (steps, n, rows, width))
 
 
+def cpu_baseline_sharded(ks, R, width, lr, bounds, root, storage, batches, active, steps):
+    """Times the CPU oracle with the same R logical ranks on the same batches (bounded number of steps, table
+    zero-initialised so that only the rows the batches reach cost memory)."""
+    from oracle import oracle as orc
+    o = orc.Oracle(R, ks.rows, width, bounds[0], bounds[1], root, storage, init=("Zero", 0.0, 0.0), learning_rate=lr)
+    o.set_parallel(True)
+    nb = len(batches[active[0]])
+    n = batches[active[0]][0].shape[0]
+    empty = np.zeros(0, np.int64)
+    rng = np.random.default_rng(7)
+    grad = rng.normal(0, 1e-3, size=(n, width)).astype(np.float32)
+
+    def step(i, with_grad=True):
+        o.preprocess([batches[r][i % nb] if r in batches else empty for r in range(R)])
+        o.push_pull([grad if (r in batches and with_grad) else None for r in range(R)])
+
+    step(0, False)
+    for i in range(1, nb + 1):                            # warm: every batch's rows have been touched once
+        step(i)
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(nb + 1 + i)
+    dt = time.perf_counter() - t0
+    cores = o.num_threads()
+    o.close()
+    keys = n * len(active)
+    return dict(value=keys * steps / dt, unit="IDs/s", cores=cores, kind="port", ms_per_step=1e3 * dt / steps,
+                sample="%d full-size steps of the same batches (%d keys per step over %d feeding ranks, %d logical "
+                       "ranks, %d-row x %d table, zero-initialised), OpenMP oracle, warm" %
+                       (steps, keys, len(active), R, ks.rows, width))
+
+
 def reference_partitioner():
     """The reference's partitioner built from its own sources WITH OpenMP (as shipped), or None."""
     import importlib.util
@@ -310,6 +342,22 @@ def main_sharded(a, cfg):
     }
     for t in tables:
         t.close()
+    # measured HBM bytes per launch of the dominant kernels (rocprofv3 --pmc runs of this same command, summarised
+    # under profiles/), valid for the default invocation only
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath) and a.scale == 1.0 and not a.active_peers and a.layout == "random" and bounds == (0, 0):
+        measured = json.load(open(tpath)).get(a.config)
+        if measured:
+            out["roofline"]["traffic"] = measured.get("whole_step")
+            out["kernels"] = {k: v for k, v in measured.items() if k != "whole_step"}
+    if not a.no_cpu:
+        del dkeys, grad, dsts
+        torch.cuda.empty_cache()
+        try:
+            out["cpu_baseline"] = cpu_baseline_sharded(ks, R, width, lr, bounds, root, storage, batches, active,
+                                                       a.cpu_steps)
+        except Exception as e:  # the GPU line stands without it
+            out["cpu_baseline"] = {"value": None, "error": str(e)}
     print(json.dumps(out), flush=True)
 
 

@@ -173,8 +173,9 @@ struct OwnerShard {
   const version_t *rq_ver;
   uint32_t rq_seg[258];
   uint32_t q, query_tiles;
-  uint32_t *outdated, *tile_cnt, *out_pos;
+  uint32_t *outdated, *tile_cnt;
   slot_t *q_slot;            // slot of every received query (kNoSlot: not owned here)
+  slot_t *ret_slot;          // slots of the rows to return, in return order
   version_t *ret_ver;
   embed_t *ret_val;
   uint32_t *err;             // the shard's error word
@@ -196,6 +197,7 @@ void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, co
 struct PullArgs {
   const uint32_t *got;       // [U] or nullptr: nothing came back (nrank == 1)
   const uint32_t *ret_i;     // [U] index into the returned rows
+  uint32_t *src_row;         // [U] where the gather reads a key's row (written by launch_refresh): offset or returned row
   const version_t *in_ver;
   const embed_t *in_val;
   embed_t *dst;              // [n][width]

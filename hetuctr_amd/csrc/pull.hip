@@ -142,7 +142,8 @@ __global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__r
 // scan_positions: a tile's flags scanned behind the tiles before it -> position of every flagged query among the
 // returned rows (:56-57, :74-75), and the first returned row of every requester's segment (:59-61) written both to
 // device memory, where the return exchange reads it, and to the host.
-// pack_rows: version and row of every flagged query packed at its position (:24-40).
+// pack_rows: version and row of every flagged query packed at its position (:24-40), from the list of their slots
+// that scan_positions leaves.
 __global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restrict__ shards) {
   const OwnerShard &S = shards[blockIdx.y];
   if (blockIdx.x >= S.query_tiles) return;
@@ -187,7 +188,7 @@ __global__ __launch_bounds__(kBlock) void scan_positions(const OwnerShard *__res
   block_exclusive_scan<kBlock>(s, sm, before); // flagged queries in the tiles before this one
   uint32_t total;
   const uint32_t pos = before + block_exclusive_scan<kBlock>(f, sm, total);
-  if (k < q) S.out_pos[k] = pos;
+  if (f) S.ret_slot[pos] = S.q_slot[k]; // the rows to return, in the order they go back
   excl[threadIdx.x] = pos;
   if (threadIdx.x == 0) excl[kBlock] = before + total;
   __syncthreads();
@@ -206,31 +207,26 @@ __global__ __launch_bounds__(kBlock) void scan_positions(const OwnerShard *__res
   if (last_block && threadIdx.x == 0) S.seg_host[257] = *S.err;
 }
 
-// kPackAhead received queries per group of LPR lanes; the slot of every query was left by decide_count
+// kPackAhead rows to return per group of LPR lanes; which rows, scan_positions has listed
 constexpr int kPackAhead = 2;
 template <int VEC, int LPR>
-__global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict__ shards) {
+__global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict__ shards, int nseg) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
   const OwnerShard &S = shards[blockIdx.y];
-  const uint32_t q = S.q;
+  const uint32_t total = S.seg_dev[nseg]; // rows this shard returns
   const uint32_t k0 = blockIdx.x * (kGroups * kPackAhead) + threadIdx.x / LPR;
-  if (k0 >= q) return;
+  if (k0 >= total) return;
   const embed_t *__restrict__ emb = S.t.emb;
   embed_t *__restrict__ ret_val = S.ret_val;
   const uint32_t gl = threadIdx.x % LPR, W = S.t.width;
   slot_t o[kPackAhead];
-  uint32_t pos[kPackAhead];
 #pragma unroll
-  for (int a = 0; a < kPackAhead; a++) {
-    const uint32_t k = min(k0 + a * kGroups, q - 1);
-    o[a] = (k0 + a * kGroups < q && S.outdated[k]) ? S.q_slot[k] : kNoSlot;
-    pos[a] = S.out_pos[k];
-  }
+  for (int a = 0; a < kPackAhead; a++) o[a] = k0 + a * kGroups < total ? S.ret_slot[k0 + a * kGroups] : kNoSlot;
   if (gl == 0) {
 #pragma unroll
     for (int a = 0; a < kPackAhead; a++)
-      if (o[a] != kNoSlot) S.ret_ver[pos[a]] = S.t.ver[o[a]];
+      if (o[a] != kNoSlot) S.ret_ver[k0 + a * kGroups] = S.t.ver[o[a]];
   }
   for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
     V v[kPackAhead];
@@ -239,7 +235,7 @@ __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict
       if (o[a] != kNoSlot) v[a] = *(const V *)(emb + (size_t)o[a] * W + col);
 #pragma unroll
     for (int a = 0; a < kPackAhead; a++)
-      if (o[a] != kNoSlot) *(V *)(ret_val + (size_t)pos[a] * W + col) = v[a];
+      if (o[a] != kNoSlot) *(V *)(ret_val + (size_t)(k0 + a * kGroups) * W + col) = v[a];
   }
 }
 
@@ -274,7 +270,11 @@ __global__ void build_return_descs(ReturnPeers p, int nrank, uint32_t width, Cop
 // that finishes last hands the totals to the host (pinned memory) and puts the device counters back to zero for the
 // next step: no clearing launch before, no copy after.
 constexpr int kCountBlocks = 128;
+// The same pass leaves, per unique key, where the gather finds its row: the resident offset, or (top bit set) the
+// index among the returned rows; the gather then reaches a row in as many dependent loads as on a single shard.
+constexpr uint32_t kReturnedRow = 0x80000000u;
 __global__ __launch_bounds__(kBlock) void count_remote(TableView t, BatchView c, const uint32_t *__restrict__ got,
+                                                       const uint32_t *__restrict__ ret_i, uint32_t *__restrict__ src_row,
                                                        uint32_t *__restrict__ stats, uint32_t *__restrict__ host_stats) {
   __shared__ uint32_t tot[4];
   __shared__ bool last;
@@ -284,6 +284,7 @@ __global__ __launch_bounds__(kBlock) void count_remote(TableView t, BatchView c,
   uint32_t n0 = 0, n1 = 0, n2 = 0, bad = 0;
   for (uint32_t u = blockIdx.x * kBlock + threadIdx.x; u < U; u += kCountBlocks * kBlock) {
     const slot_t o = c.uoff[u];
+    src_row[u] = o == kNoSlot ? (kReturnedRow | ret_i[u]) : (uint32_t)o;
     if (o == kNoSlot) n1++;
     else if ((uint32_t)o < t.n_cached) {
       if (got[u]) n2++;
@@ -362,9 +363,12 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
     const uint32_t j = min(j0 + k, n - 1);
     const uint32_t u = c.rank_sorted[j];
     const uint32_t i = c.sorted_arg[j];
-    const slot_t o = c.uoff[u];
-    if (kLocalOnly || o != kNoSlot) src[k] = t.emb + (size_t)o * W;
-    else src[k] = a.in_val + (size_t)a.ret_i[u] * W;
+    if (kLocalOnly) {
+      src[k] = t.emb + (size_t)c.uoff[u] * W;
+    } else {
+      const uint32_t r = a.src_row[u];
+      src[k] = (r & kReturnedRow) ? a.in_val + (size_t)(r & ~kReturnedRow) * W : t.emb + (size_t)r * W;
+    }
     dst[k] = a.dst + (size_t)i * W;
   }
   for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
@@ -400,9 +404,12 @@ __global__ __launch_bounds__(kBlock) void gather_pooled(TableView t, BatchView c
 #pragma unroll
       for (int k = 0; k < kPoolAhead; k++) {
         const uint32_t u = c.idx_map[i0 + min(h0 + k, bag - 1)];
-        const slot_t o = c.uoff[u];
-        if (kLocalOnly || o != kNoSlot) src[k] = t.emb + (size_t)o * W;
-        else src[k] = a.in_val + (size_t)a.ret_i[u] * W;
+        if (kLocalOnly) {
+          src[k] = t.emb + (size_t)c.uoff[u] * W;
+        } else {
+          const uint32_t r = a.src_row[u];
+          src[k] = (r & kReturnedRow) ? a.in_val + (size_t)(r & ~kReturnedRow) * W : t.emb + (size_t)r * W;
+        }
       }
       V v[kPoolAhead];
 #pragma unroll
@@ -424,7 +431,11 @@ __global__ __launch_bounds__(kBlock) void copy_segments(const CopyDesc *__restri
   if ((((uintptr_t)cd.src | (uintptr_t)cd.dst | cd.bytes) & 15) == 0) {
     const uint4 *s = (const uint4 *)cd.src;
     uint4 *o = (uint4 *)cd.dst;
-    for (size_t i = tid; i < cd.bytes / 16; i += stride) o[i] = s[i];
+    // past the caches both ways: what an exchange moves is read once more at most, and the table rows the push left
+    // in the caches are what the gather at the end of the step wants to find there
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    for (size_t i = tid; i < cd.bytes / 16; i += stride)
+      __builtin_nontemporal_store(__builtin_nontemporal_load((const u32x4 *)s + i), (u32x4 *)o + i);
   } else {
     const uint32_t *s = (const uint32_t *)cd.src;
     uint32_t *o = (uint32_t *)cd.dst;
@@ -508,7 +519,7 @@ void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerS
   hipLaunchKernelGGL(scan_positions, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
   if (q_max) {
 #define CALL(V, L) \
-  hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q_max, kPackAhead * (kBlock / L)), nshards), dim3(kBlock), 0, s, shards_dev)
+  hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q_max, kPackAhead * (kBlock / L)), nshards), dim3(kBlock), 0, s, shards_dev, nsrc)
     HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   }
@@ -526,7 +537,8 @@ void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, co
 void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
                     uint32_t *stats, uint32_t *host_stats) {
   if (!n_unique || !a.got) return;
-  hipLaunchKernelGGL(count_remote, dim3(kCountBlocks), dim3(kBlock), 0, s, t, cur, a.got, stats, host_stats);
+  hipLaunchKernelGGL(count_remote, dim3(kCountBlocks), dim3(kBlock), 0, s, t, cur, a.got, a.ret_i, a.src_row, stats,
+                     host_stats);
   const bool vec4 = t.width % 4 == 0;
   const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
 #define CALL(V, L) \

@@ -154,7 +154,7 @@ class Shard {
   // send side
   DeviceBuf q_idx, q_ver, g_idx, g_cnt, g_val;
   // receive side (owner role)
-  DeviceBuf rq_idx, rq_ver, rg_idx, rg_cnt, rg_val, outdated, out_pos, q_slot, ret_ver, ret_val, ret_seg_dev;
+  DeviceBuf rq_idx, rq_ver, rg_idx, rg_cnt, rg_val, outdated, ret_slot, q_slot, src_row, ret_ver, ret_val, ret_seg_dev;
   std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
   // requester side of the return
   DeviceBuf got, ret_i, in_ver, in_val;

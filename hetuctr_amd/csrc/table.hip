@@ -451,7 +451,7 @@ void Shard::fill_owner_args(OwnerShard &o) {
   const int R = cfg.nrank;
   const uint32_t Q = (uint32_t)rq_seg[R];
   outdated.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
-  out_pos.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
+  ret_slot.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
   q_slot.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(slot_t));
   ret_ver.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(version_t));
   ret_val.reserve((size_t)std::max<uint32_t>(Q, 1) * cfg.width * sizeof(embed_t));
@@ -475,7 +475,7 @@ void Shard::fill_owner_args(OwnerShard &o) {
   o.query_tiles = (uint32_t)query_tiles(Q); // one tile even without queries: the segment table is written
   o.outdated = outdated.as<uint32_t>();
   o.tile_cnt = query_sums.as<uint32_t>();
-  o.out_pos = out_pos.as<uint32_t>();
+  o.ret_slot = ret_slot.as<slot_t>();
   o.q_slot = q_slot.as<slot_t>();
   o.ret_ver = ret_ver.as<version_t>();
   o.ret_val = ret_val.as<embed_t>();
@@ -501,6 +501,7 @@ void Shard::write_back(float *dst, uint32_t bag) {
   PullArgs a;
   a.got = nullptr;
   a.ret_i = nullptr;
+  a.src_row = nullptr;
   a.in_ver = nullptr;
   a.in_val = nullptr;
   a.dst = dst;
@@ -518,6 +519,8 @@ void Shard::write_back(float *dst, uint32_t bag) {
                           nullptr);
     a.got = got.as<uint32_t>();
     a.ret_i = ret_i.as<uint32_t>();
+    src_row.reserve((size_t)std::max<uint32_t>(cur.U, 1) * 4);
+    a.src_row = src_row.as<uint32_t>();
     a.in_ver = in_ver.as<version_t>();
     a.in_val = in_val.as<embed_t>();
     launch_refresh(s, tv, cur.view(), cur.U, a, stats.as<uint32_t>(), mirror->stats);

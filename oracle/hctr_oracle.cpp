@@ -30,6 +30,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <numeric>
@@ -136,6 +137,29 @@ void init_values(embed_t *out, size_t len, int type, float a, float b, unsigned 
   }
 }
 
+// A zero-filled array whose pages the system hands out when they are first touched (calloc): a table of tens of
+// millions of rows that starts from zeros costs memory and time only for the rows the test's batches reach.
+template <typename T> struct ZeroArray {
+  T *p = nullptr;
+  size_t n = 0;
+  ZeroArray() {}
+  ZeroArray(const ZeroArray &) = delete;
+  ZeroArray &operator=(const ZeroArray &) = delete;
+  ZeroArray(ZeroArray &&o) noexcept : p(o.p), n(o.n) { o.p = nullptr; o.n = 0; }
+  ~ZeroArray() { free(p); }
+  void reset(size_t count) {
+    free(p);
+    p = (T *)calloc(count ? count : 1, sizeof(T));
+    n = p ? count : 0;
+  }
+  T *data() { return p; }
+  const T *data() const { return p; }
+  size_t size() const { return n; }
+  T &operator[](size_t i) { return p[i]; }
+  const T &operator[](size_t i) const { return p[i]; }
+  T *begin() { return p; }
+};
+
 // ---------------------------------------------------------------------------------------------
 // Per-batch record (csrc/core/preprocess_struct.h:7-24)
 // ---------------------------------------------------------------------------------------------
@@ -152,7 +176,7 @@ struct Rank {
   size_t S = 0, C = 0; // stored rows, cached rows (offsets < C are cached)
   std::vector<index_t> store_ids;   // id at each offset
   std::vector<index_t> slot;        // id -> offset or -1 (stands for the hash map find)
-  std::vector<embed_t> emb, pend;
+  ZeroArray<embed_t> emb, pend;
   std::vector<version_t> ver, upd;
   Batch cur, prev;
   std::vector<index_t> need, prefix; // push plan of prev
@@ -199,12 +223,13 @@ bool init_rank(Group &g, Rank &rk, const index_t *storage, size_t S, int init_ty
     if (g.root[storage[i]] == rk.rank) rk.store_ids[c++] = storage[i];
   rk.slot.assign(g.IDMax, kInvalidIndex);
   for (size_t o = 0; o < S; o++) rk.slot[rk.store_ids[o]] = (index_t)o; // insert (key[i] -> i) (:84-87)
-  rk.emb.resize(S * g.W);
-  rk.pend.assign(rk.C * g.W, 0.f);                                       // :102-103
+  rk.emb.reset(S * g.W);
+  rk.pend.reset(rk.C * g.W);                                             // :102-103
+  if (rk.emb.size() != S * g.W || rk.pend.size() != rk.C * g.W) { g.err = "out of memory"; return false; }
   rk.upd.assign(rk.C, 0);                                                // :104-105
   rk.ver.resize(S);
   for (size_t o = 0; o < S; o++) rk.ver[o] = o < rk.C ? kInvalidVersion : 0; // :108-112
-  init_values(rk.emb.data(), S * g.W, init_type, a, b, seed);            // :156, value depends on offset
+  if (init_type != 0) init_values(rk.emb.data(), S * g.W, init_type, a, b, seed); // :156, value depends on offset
   return true;
 }
 
@@ -564,7 +589,7 @@ long long orc_fetch(void *h, int rank, int which, void *out, size_t cap) {
     for (size_t i = 0; i < n && i < cap; i++) o[i] = (long long)v[i];
     return (long long)n;
   };
-  auto putf = [&](const std::vector<embed_t> &v) -> long long {
+  auto putf = [&](const ZeroArray<embed_t> &v) -> long long {
     memcpy(out, v.data(), std::min(cap, v.size()) * sizeof(embed_t));
     return (long long)v.size();
   };

@@ -119,3 +119,50 @@ def test_large_configs_by_properties(name):
     ver = t.fetch(capi.VERSION)
     assert int(ver.sum()) == 2 * n                               # two batches were pushed, one count per key
     t.close()
+
+
+@pytest.mark.parametrize("feeders,bounds,steps", [((0,), (0, 0), 3), (tuple(range(8)), (2, 3), 5)])
+def test_cfg3_eight_shards_full_size_bit_exact(feeders, bounds, steps):
+    """The 8-shard configuration at its full size (33.8M rows x 128 over eight shards of one loopback group) next to the
+    CPU oracle with the same eight logical ranks.  First the benchmark's own case: rank 0 feeds full batches and caches
+    the hottest tenth of its remote rows, the peers only serve, bounds 0/0.  Then every rank feeds an eighth of a
+    batch, every rank caches, and the bounds let rows go stale (pull 2, push 3), so that pending gradients, refreshed
+    rows and pushes from several sources to one row all occur at this size."""
+    from tests.gpu_util import Pair, INT_ITEMS_PRE, INT_ITEMS_POST
+    cfg = workloads.CONFIGS["cfg3"]
+    R, width = cfg["nrank"], cfg["width"]
+    ks = workloads.KeyStream(cfg, seed=0)
+    root, storage = workloads.shard_layout(ks, R, cfg["cache_frac"], cached_ranks=feeders)
+    say("cfg3 full size: %d rows x %d over %d shards, feeders %s, bounds %s, %d keys per full batch" %
+        (ks.rows, width, R, feeders, bounds, ks.n))
+    p = Pair(R, ks.rows, width, root, storage, init=("Zero", 0.0, 0.0), lr=cfg["lr"], bounds=bounds)
+    p.oracle.set_parallel(True)
+    rng = np.random.default_rng(11)
+    share = ks.n // len(feeders)
+    empty = np.zeros(0, np.int64)
+    grads = [None] * R
+    light = [it for it in INT_ITEMS_PRE if it not in (capi.KEYS, capi.IDX_MAP)] # those two are covered at small sizes
+    for step in range(steps + 1):
+        last = step == steps                       # the last step pulls without gradients (inference)
+        full = ks.batch()
+        if len(feeders) == 1:
+            keys = [full if r == feeders[0] else empty for r in range(R)]
+        else:
+            keys = [full[r * share:(r + 1) * share] if r in feeders else empty for r in range(R)]
+        p.preprocess(keys, device_keys=True)
+        p.compare_ints(light, "step %d" % step)
+        out, ref = p.push_pull([None] * R if last else grads)
+        for r in feeders:
+            assert np.array_equal(out[r], ref[r]), "step %d rank %d: %d rows differ" % (
+                step, r, int((out[r] != ref[r]).any(axis=1).sum()))
+        p.compare_ints([capi.OUTDATED, capi.GOT, capi.STATS, capi.UPDATES], "step %d" % step)
+        grads = [rng.normal(0, 1e-3, size=(k.shape[0], width)).astype(np.float32) if k.shape[0] else None for k in keys]
+        say("  step %d ok; stats of rank 0 (hit, miss, refreshed, pushed, served, received): %s" %
+            (step, p.tables[0].fetch(capi.STATS)[:6].tolist()))
+    for r in range(R):                             # versions of all rows, pending gradients of all cached rows
+        assert np.array_equal(p.tables[r].fetch(capi.VERSION), p.oracle.fetch(r, capi.VERSION)), "versions rank %d" % r
+        assert np.array_equal(p.tables[r].fetch(capi.PENDING), p.oracle.fetch(r, capi.PENDING)), "pending rank %d" % r
+    if len(feeders) > 1:
+        st = np.sum([p.tables[r].fetch(capi.STATS)[:6] for r in range(R)], axis=0)
+        assert st[0] > 0, "no cached row was fresh enough to be used: the bounds were meant to allow it"
+    p.close()
