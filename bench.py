@@ -28,10 +28,15 @@ def parse():
     ap.add_argument("--config", default="cfg2")
     ap.add_argument("--batches", type=int, default=4, help="distinct key batches cycled through")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and samples (debugging only)")
+    ap.add_argument("--samples", type=int, default=0,
+                    help="samples per batch instead of the config's (the reference's script defaults to 2048, "
+                         "tests/benchmark.py:74); the table keeps its size")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=10,
                     help="full-size steps of the CPU baseline leg (about 12 core-seconds at the default)")
     ap.add_argument("--no-stage-timing", action="store_true")
+    ap.add_argument("--no-variants", action="store_true",
+                    help="skip the extra passes (literal call protocol, permuted ids): for profiles of the headline alone")
     ap.add_argument("--host-keys", action="store_true",
                     help="hand the ids over as pageable host buffers (adds their transfer to the step)")
     ap.add_argument("--pooled", action="store_true",
@@ -386,7 +391,9 @@ def main():
         return
     if a.partition:
         return main_partition(a)
-    cfg = workloads.CONFIGS[a.config]
+    cfg = dict(workloads.CONFIGS[a.config])
+    if a.samples:
+        cfg["samples"] = a.samples
     if cfg.get("nrank", 1) > 1:
         return main_sharded(a, cfg)
     width, lr = cfg["width"], cfg["lr"]
@@ -540,13 +547,13 @@ def main():
     # the reference's literal call protocol: preprocess returns when all its work is done (hetu_gpu_table.cu:64), so
     # nothing of the batch's index runs beside the push
     literal = None
-    if not a.host_keys:
+    if not a.host_keys and not a.no_variants:
         table.defer_index(False)
         literal = variant(key_ptr, timing=False)
         table.defer_index(True)
     # the same workload with the hot rows of every field scattered over the field instead of lying side by side
     permuted = None
-    if a.config == "cfg2" and a.scale == 1.0 and not a.host_keys:
+    if a.config == "cfg2" and a.scale == 1.0 and not a.host_keys and not a.no_variants and not a.samples:
         pcfg = workloads.CONFIGS["cfg2_permuted"]
         pks = workloads.KeyStream(pcfg, seed=0, scale=a.scale)
         pkeys = [torch.from_numpy(pks.batch()).cuda() for _ in range(len(dkeys))]

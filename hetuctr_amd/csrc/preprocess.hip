@@ -17,7 +17,7 @@ constexpr int kTile = kBlock * kItems; // 2048: scan_blocks(n) sizes the scratch
 // of the batch's run counters, and the per-tile counts of the first sort pass' digit: a block works on one sort tile, so the sort
 // needs no counting launch of its own for that pass.  This is the one kernel that reads the caller's buffer: the
 // call may return when it is through.
-template <typename K>
+template <typename K, int ITEMS>
 __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restrict__ keys, uint32_t n, uint64_t id_max,
                                                          int id_bits, int nrank, const worker_t *__restrict__ root,
                                                          K *__restrict__ comp, uint32_t *__restrict__ err,
@@ -27,17 +27,17 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
   const uint32_t nb = 1u << dbits, mask = nb - 1;
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
   if (blockIdx.x == 0 && threadIdx.x < kRunCounters && nlong) nlong[threadIdx.x] = 0; // counters of this batch
-  const uint32_t base = blockIdx.x * kSortTile;
-  uint64_t id[kSortItems];
+  const uint32_t base = blockIdx.x * (ITEMS * kSortBlock);
+  uint64_t id[ITEMS];
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
+  for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = base + k * kSortBlock + threadIdx.x;
     id[k] = i < n ? (uint64_t)load_once(&keys[i]) : 0; // the caller's ids are read here and nowhere else
   }
   __syncthreads();
   bool bad = false;
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
+  for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = base + k * kSortBlock + threadIdx.x;
     if (i < n && id[k] >= id_max) { // also catches negative ids
       bad = true;
@@ -45,11 +45,11 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
     }
   }
   if (bad) atomicOr(err, 1u);
-  uint64_t owner[kSortItems];
+  uint64_t owner[ITEMS];
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) owner[k] = nrank > 1 ? root[id[k]] : 0;
+  for (int k = 0; k < ITEMS; k++) owner[k] = nrank > 1 ? root[id[k]] : 0;
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
+  for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = base + k * kSortBlock + threadIdx.x;
     const K c = (K)((owner[k] << id_bits) | id[k]);
     if (i < n) comp[i] = c;
@@ -297,12 +297,17 @@ void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, co
   if (!n) return;
   const unsigned nblocks = (unsigned)sort_tiles(n);
   const int dbits = sort_first_digit_bits(kl.total_bits);
-  if (kl.wide)
-    hipLaunchKernelGGL(make_keys<uint64_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
-                       t.root, (uint64_t *)comp_keys, err, nlong, dbits, sort_counts);
-  else
-    hipLaunchKernelGGL(make_keys<uint32_t>, dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max, kl.id_bits, t.nrank,
-                       t.root, (uint32_t *)comp_keys, err, nlong, dbits, sort_counts);
+#define CALL(I)                                                                                                       \
+  do {                                                                                                                \
+    if (kl.wide)                                                                                                      \
+      hipLaunchKernelGGL((make_keys<uint64_t, I>), dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max,          \
+                         kl.id_bits, t.nrank, t.root, (uint64_t *)comp_keys, err, nlong, dbits, sort_counts);         \
+    else                                                                                                              \
+      hipLaunchKernelGGL((make_keys<uint32_t, I>), dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max,          \
+                         kl.id_bits, t.nrank, t.root, (uint32_t *)comp_keys, err, nlong, dbits, sort_counts);         \
+  } while (0)
+  HCTR_SORT_ITEMS_DISPATCH(n, CALL);
+#undef CALL
   HCTR_HIP(hipGetLastError());
 }
 

@@ -9,17 +9,42 @@ namespace hctr {
 #define HCTR_SORT_BLOCK 512
 #endif
 constexpr int kSortBlock = HCTR_SORT_BLOCK;     // threads per block
-#ifndef HCTR_SORT_ITEMS
-#define HCTR_SORT_ITEMS 8
-#endif
-constexpr int kSortItems = HCTR_SORT_ITEMS;     // keys per thread
-constexpr int kSortTile = kSortBlock * kSortItems;
 constexpr int kSortMaxDigitBits = 10;           // up to 1024 bins
 constexpr int kSortMaxBins = 1 << kSortMaxDigitBits;
-inline size_t sort_tiles(size_t n) { return (n + kSortTile - 1) / kSortTile; }
+// Keys per thread, hence keys per tile (one block sorts one tile per pass), chosen by the size of the input: a small
+// input is cut into small tiles so that enough blocks share it (its passes are latency, not traffic); a huge one into
+// large tiles, because every tile costs a row of digit counts that is written, scanned and read again in every pass.
+#ifndef HCTR_SORT_ITEMS_LARGE
+#define HCTR_SORT_ITEMS_LARGE 16
+#endif
+#ifndef HCTR_SORT_ITEMS_SMALL
+#define HCTR_SORT_ITEMS_SMALL 2
+#endif
+constexpr int kSortItemsSmall = HCTR_SORT_ITEMS_SMALL, kSortItemsDefault = 8, kSortItemsLarge = HCTR_SORT_ITEMS_LARGE;
+inline int sort_items(size_t n) {
+  return n <= ((size_t)1 << 17) ? kSortItemsSmall : (n >= ((size_t)1 << 23) ? kSortItemsLarge : kSortItemsDefault);
+}
+inline size_t sort_tile(size_t n) { return (size_t)kSortBlock * sort_items(n); }
+inline size_t sort_tiles(size_t n) { return (n + sort_tile(n) - 1) / sort_tile(n); }
 // words of scratch a sort of n keys needs: per tile and bin the count of the digit in the earlier tiles, then the
-// total of every bin
+// total of every bin.  Not monotonic in n (the tile grows with it): size the scratch for the n that is sorted.
 inline size_t sort_scratch_words(size_t n) { return (sort_tiles(n) + 1) * (size_t)kSortMaxBins; }
+// the most words any input of up to n_max keys needs
+inline size_t sort_scratch_words_upto(size_t n_max) {
+  size_t w = sort_scratch_words(n_max);
+  if (n_max > ((size_t)1 << 17)) w = w > sort_scratch_words((size_t)1 << 17) ? w : sort_scratch_words((size_t)1 << 17);
+  if (n_max > ((size_t)1 << 23) - 1) w = w > sort_scratch_words(((size_t)1 << 23) - 1) ? w : sort_scratch_words(((size_t)1 << 23) - 1);
+  return w;
+}
+// expands CALL(ITEMS) for the tile shape of an input of n keys
+#define HCTR_SORT_ITEMS_DISPATCH(n, CALL)                      \
+  do {                                                         \
+    switch (::hctr::sort_items(n)) {                           \
+      case ::hctr::kSortItemsSmall: CALL(::hctr::kSortItemsSmall); break;     \
+      case ::hctr::kSortItemsLarge: CALL(::hctr::kSortItemsLarge); break;     \
+      default: CALL(::hctr::kSortItemsDefault); break;         \
+    }                                                          \
+  } while (0)
 
 struct SortScratch {
   uint32_t *words = nullptr;   // sort_scratch_words(n) of them
@@ -57,8 +82,8 @@ __device__ __forceinline__ void count_digit(uint32_t *h, uint32_t d, bool in) {
 // buffers of n elements; the sorted keys end in *keys_sorted (one of tmp_k0/tmp_k1) and the sorted
 // positions in vals_out.  n == 0 is a no-op.  Three launches per pass of up to kSortMaxDigitBits bits.
 // first_counts_done: scratch.words already holds the per-tile counts of the first pass' digit
-// (sort_first_digit_bits(bits) low bits, rows of 1 << that many words, tiles of kSortTile keys), written by the
-// kernel that made the keys (see count_digit).
+// (sort_first_digit_bits(bits) low bits, rows of 1 << that many words, tiles of sort_tile(n) keys), written by the
+// kernel that made the keys (see count_digit); its tiles are those of sort_tile(n).
 // step_from / step_to: only the launches [step_from, step_to) of the sort are enqueued by this call, launch 3 * p + k
 // being the count (k = 0), the column scan (1) or the scatter (2) of pass p; a caller that enqueues the sort in
 // pieces passes the same other arguments every time.

@@ -17,31 +17,30 @@ namespace {
 
 constexpr int kWaves = kSortBlock / kWave;
 constexpr uint32_t kXcds = 8;              // accelerator dies of the device, each with its own L2
-constexpr int kSub = kSortTile / kWaves; // keys per wave
-constexpr int kRounds = kSub / kWave;    // 64-key groups per wave
-static_assert(kRounds * kWave * kWaves == kSortTile, "tile shape");
+// A tile of ITEMS * kSortBlock keys: wave w takes the w-th run of ITEMS * 64 consecutive keys, 64 keys per round.
 static_assert(kSortMaxBins <= 2 * kSortBlock, "a thread owns at most two bins");
 static_assert(kSortBlock <= 1024 && kSortBlock % kWave == 0, "block shape");
 
 // Digit counts of one tile: row `tile` of counts[tile][bin].  A run of equal digits in consecutive lanes (what a
 // partly sorted input and a hot key make of most waves) adds once, from its first lane, so that the LDS atomics
 // of one instruction rarely meet on one word.
-template <typename K>
+template <typename K, int ITEMS>
 __global__ __launch_bounds__(kSortBlock) void digit_histogram(const K *__restrict__ keys, uint32_t n, int shift,
                                                               int dbits, uint32_t *__restrict__ counts) {
   __shared__ uint32_t h[kSortMaxBins];
   const uint32_t nb = 1u << dbits, mask = nb - 1;
-  K key[kSortItems];
+  constexpr uint32_t kTile = ITEMS * kSortBlock;
+  K key[ITEMS];
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
-    const uint32_t idx = blockIdx.x * kSortTile + k * kSortBlock + threadIdx.x;
+  for (int k = 0; k < ITEMS; k++) {
+    const uint32_t idx = blockIdx.x * kTile + k * kSortBlock + threadIdx.x;
     key[k] = idx < n ? keys[idx] : (K)0;
   }
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
-    const uint32_t idx = blockIdx.x * kSortTile + k * kSortBlock + threadIdx.x;
+  for (int k = 0; k < ITEMS; k++) {
+    const uint32_t idx = blockIdx.x * kTile + k * kSortBlock + threadIdx.x;
     count_digit(h, (uint32_t)(key[k] >> shift) & mask, idx < n);
   }
   __syncthreads();
@@ -94,7 +93,7 @@ __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ 
   }
 }
 
-template <typename K, bool kFirst>
+template <typename K, bool kFirst, int ITEMS>
 __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
                                                       K *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
                                                       uint32_t n, int shift, int dbits, uint32_t tiles,
@@ -110,9 +109,12 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
 #else
   const uint32_t tile = blockIdx.x;
 #endif
+  constexpr int kRounds = ITEMS;                   // 64-key groups per wave
+  constexpr int kSub = ITEMS * kWave;              // keys per wave
+  constexpr uint32_t kSortTile = ITEMS * kSortBlock;
   // one LDS area, used twice: first the wave-private digit counters, then the tile sorted by digit
   constexpr int kCntWords = kWaves * kSortMaxBins;
-  constexpr int kTileWords = kSortTile * (int)(sizeof(K) / 4 + 1);
+  constexpr int kTileWords = (int)kSortTile * (int)(sizeof(K) / 4 + 1);
   __shared__ __align__(8) uint32_t area[kCntWords > kTileWords ? kCntWords : kTileWords];
   __shared__ uint32_t base[kSortMaxBins];      // global position of the bin's first key of this tile
   __shared__ uint32_t bin_start[kSortMaxBins]; // position of the bin inside the tile sorted by digit
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
   // neighbouring threads now hold neighbouring keys of a bin: the global stores of a bin are contiguous
   const uint32_t tile_n = min((uint32_t)kSortTile, n - tile * kSortTile);
 #pragma unroll
-  for (int k = 0; k < kSortItems; k++) {
+  for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = k * kSortBlock + threadIdx.x;
     if (i < tile_n) {
       const K kk = skey[i];
@@ -278,18 +280,27 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
     uint32_t *vout = (p == passes - 1) ? vals_out : vtmp[p & 1];
     const uint32_t nb = 1u << dbits;
     auto wanted = [&](int kind) { return 3 * p + kind >= step_from && 3 * p + kind < step_to; };
-    if (wanted(0) && (p > 0 || !first_counts_done))
-      hipLaunchKernelGGL(digit_histogram<K>, dim3(tiles), dim3(kSortBlock), 0, stream, kin, n, shift, dbits, counts);
+    if (wanted(0) && (p > 0 || !first_counts_done)) {
+#define CALL(I) \
+  hipLaunchKernelGGL((digit_histogram<K, I>), dim3(tiles), dim3(kSortBlock), 0, stream, kin, n, shift, dbits, counts)
+      HCTR_SORT_ITEMS_DISPATCH(n, CALL);
+#undef CALL
+    }
     if (wanted(1))
       hipLaunchKernelGGL(scan_tiles, dim3((nb + kScanCols - 1) / kScanCols), dim3(kScanBlock), 0, stream, counts, tiles,
                          nb, bin_total);
     if (wanted(2)) {
-      if (p == 0)
-        hipLaunchKernelGGL((scatter<K, true>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift,
-                           dbits, tiles, counts, bin_total);
-      else
-        hipLaunchKernelGGL((scatter<K, false>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,
-                           shift, dbits, tiles, counts, bin_total);
+#define CALL(I)                                                                                                     \
+  do {                                                                                                              \
+    if (p == 0)                                                                                                     \
+      hipLaunchKernelGGL((scatter<K, true, I>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,  \
+                         shift, dbits, tiles, counts, bin_total);                                                   \
+    else                                                                                                            \
+      hipLaunchKernelGGL((scatter<K, false, I>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, \
+                         shift, dbits, tiles, counts, bin_total);                                                   \
+  } while (0)
+      HCTR_SORT_ITEMS_DISPATCH(n, CALL);
+#undef CALL
     }
     HCTR_HIP(hipGetLastError());
     kin = kout;

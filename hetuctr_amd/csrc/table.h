@@ -173,7 +173,7 @@ class Shard {
 constexpr size_t kNoAllocMaxKeys = 262144;
 size_t index_scratch_bytes(uint32_t n, bool wide);
 constexpr size_t kNoAllocScratchBytes = 2 * (kNoAllocMaxKeys * 8) + 2 * (kNoAllocMaxKeys * 4) +
-                                        (kNoAllocMaxKeys / kSortTile + 2) * kSortMaxBins * 4 + 4096;
+                                        (kNoAllocMaxKeys / (kSortBlock * kSortItemsSmall) + 2) * kSortMaxBins * 4 + 4096;
 
 // All shards of one loopback group live in one process on one device and share one stream.  The group
 // carries the collective calls: every shard's thread deposits its arguments, the last one to arrive runs the
