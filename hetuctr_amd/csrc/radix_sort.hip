@@ -50,7 +50,10 @@ __global__ __launch_bounds__(kSortBlock) void digit_histogram(const K *__restric
 // counts[tile][bin] -> in place, the count of the bin in the earlier tiles; bin_total[bin].  A block scans kScanCols
 // neighbouring bins: thread (part, col) adds up its part of the tiles for one bin.  Up to kScanKeep rows per thread
 // stay in registers between the sum and the rewrite (one trip to memory); longer parts are read twice.
-constexpr int kScanBlock = 512, kScanCols = 16, kScanParts = kScanBlock / kScanCols, kScanKeep = 16;
+#ifndef HCTR_SCAN_COLS
+#define HCTR_SCAN_COLS 16
+#endif
+constexpr int kScanBlock = 512, kScanCols = HCTR_SCAN_COLS, kScanParts = kScanBlock / kScanCols, kScanKeep = 16;
 __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ counts, uint32_t tiles, uint32_t nb,
                                                          uint32_t *__restrict__ bin_total) {
   __shared__ uint32_t part_sum[kScanParts][kScanCols];
