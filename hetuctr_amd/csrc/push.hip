@@ -8,6 +8,10 @@
 // order differs from it in the last bits by an amount that grows with the number of duplicates.  Here
 // every run of equal keys is summed by ONE chain of additions per column, in exactly that order: sums are
 // bit-identical to the reference's order (compiled without fused multiply-add contraction), for any skew.
+// "Bit-identical" is against that non-contracted restatement on the CPU: the reference itself is built by nvcc,
+// whose default may fuse `sum *= -lr; dest += sum` (generate_query.cu:37-39) into one multiply-add, so against a
+// CUDA build the last rounding of an updated value can differ by one ulp.  The contract against the reference is
+// its own tolerance, 1e-5 relative.
 //
 // One launch, three ranges of blocks, one per class of run length (the long chains are dispatched first and the
 // other blocks fill the machine behind them):

@@ -61,7 +61,7 @@ int hctr_preprocess(hctr_table *t, const int64_t *keys, size_t n);
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same result as hctr_preprocess, and like the
  * reference's call it returns when all its work is done; it calls no hipMalloc / hipFree and no allocating routine:
  *   - the index scratch (sort ping-pong buffers, per-tile digit counts, scan sums) lives in a static device array of
- *     6.3 MiB that every GPU the library runs on holds until the process ends;
+ *     7.0 MiB that every GPU the library runs on holds until the process ends;
  *   - n is at most 262144 keys (HCTR_NOALLOC_MAX_KEYS), larger batches are refused;
  *   - keys must be DEVICE memory (a transfer from pageable host memory is staged by the runtime);
  *   - the table has one shard, and its two batch buffers already hold n keys: they are sized by ordinary
