@@ -282,9 +282,14 @@ def main_sharded(a, cfg):
     gptr = [grad.data_ptr() if r in dkeys else 0 for r in range(R)]
     dptr = [dsts[r].data_ptr() if r in dkeys else 0 for r in range(R)]
 
+    # the argument arrays of the two calls, one set per batch, built outside the loop
+    calls = [capi.GroupStep(tables, [dkeys[r][b].data_ptr() if r in dkeys else 0 for r in range(R)], counts, gptr, dptr)
+             for b in range(nb)]
+
     def step(i):
-        capi.group_preprocess(tables, [dkeys[r][i % nb].data_ptr() if r in dkeys else 0 for r in range(R)], counts)
-        capi.group_push_pull(tables, gptr, dptr)
+        c = calls[i % nb]
+        c.preprocess()
+        c.push_pull()
 
     w0 = max(a.warmup, 2) + nb
     for i in range(w0):
@@ -299,6 +304,17 @@ def main_sharded(a, cfg):
         pp_ms += q
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    # how long each of the two calls holds the host (a pass of its own: the clock reads cost time)
+    call_s = [0.0, 0.0]
+    for i in range(a.steps):
+        c = calls[(w0 + i) % nb]
+        t1 = time.perf_counter()
+        c.preprocess()
+        t2 = time.perf_counter()
+        c.push_pull()
+        t3 = time.perf_counter()
+        call_s[0] += t2 - t1
+        call_s[1] += t3 - t2
     stages = None
     if not a.no_stage_timing:
         tables[0].stage_timing(True)
@@ -338,6 +354,7 @@ def main_sharded(a, cfg):
         "cache_per_step_all_ranks": {"remote_unique_keys_hit": hit, "missed_not_cached": miss, "refreshed": refresh,
                                      "rows_pushed_to_owners": pushed, "rows_returned_by_owners": served},
         "device_ms_per_step": {"preprocess": pre_ms / a.steps, "push_pull": pp_ms / a.steps},
+        "host_ms_per_call": {"preprocess": 1e3 * call_s[0] / a.steps, "push_pull": 1e3 * call_s[1] / a.steps},
         "step_hbm": {"algorithmic_bytes": int(bytes_step), "achieved_GBps": gbs, "frac": gbs / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": "whole step (all shards' kernels)", "achieved": gbs, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None, "avg_ms": ms_step,

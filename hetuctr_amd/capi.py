@@ -220,6 +220,29 @@ def group_push_pull(tables, grad_ptrs, dst_ptrs):
     _check(lib().hctr_group_push_pull(hs, len(tables), _ptrs(grad_ptrs), _ptrs(dst_ptrs)))
 
 
+class GroupStep:
+    """The two lock-step calls of a loopback group with their argument arrays built once: a caller that steps the same
+    buffers again and again (a benchmark loop, a training loop with fixed staging buffers) pays two foreign calls per
+    step and no array construction."""
+
+    def __init__(self, tables, key_ptrs, ns, grad_ptrs, dst_ptrs):
+        self._lib = lib()
+        self._n = len(tables)
+        self._hs = (C.c_void_p * self._n)(*[t._h for t in tables])
+        self._keys = _ptrs(key_ptrs)
+        self._sizes = (C.c_size_t * self._n)(*ns)
+        self._grads = _ptrs(grad_ptrs)
+        self._dsts = _ptrs(dst_ptrs)
+
+    def preprocess(self):
+        if self._lib.hctr_group_preprocess(self._hs, self._n, self._keys, self._sizes):
+            _check(1)
+
+    def push_pull(self):
+        if self._lib.hctr_group_push_pull(self._hs, self._n, self._grads, self._dsts):
+            _check(1)
+
+
 def group_push_pull_pooled(tables, grad_ptrs, dst_ptrs, bag):
     hs = (C.c_void_p * len(tables))(*[t._h for t in tables])
     _check(lib().hctr_group_push_pull_pooled(hs, len(tables), _ptrs(grad_ptrs), _ptrs(dst_ptrs), bag))

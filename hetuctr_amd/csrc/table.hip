@@ -996,37 +996,38 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     return;
   }
   if (defer_index && !stage_timing) {
-    // Several shards: the ids are read and the push plan of the previous batches is made on the main stream, and the
-    // call returns when that is done (the plan sizes the push buffers).  The index of the current batches runs on the
-    // second stream; the next push_pull starts the pushes at once and waits for the index before it builds the
-    // queries, which are the first thing that needs it.
-    if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
-    for (Shard *m : members) {
-      m->swap_batches();
-      m->ingest_keys(keys[m->cfg.rank], n[m->cfg.rank], &m->mirror->key_err);
-    }
-    HCTR_HIP(hipEventRecord(ev_keys, stream));
-    // a previous batch that no push_pull has seen yet (two preprocess calls in a row) is planned here
+    // Several shards: as with one, the ids are read by a kernel on the second stream and the call returns when that
+    // kernel is through; the index of the current batches follows on that stream (no event between the two streams:
+    // waiting for one costs the host 15-20 us), next to the pushes that the next push_pull queues first.  push_pull
+    // waits for the index before it builds the queries, which are the first thing that needs it.  The push plan of the
+    // previous batches was made at the end of the step before.
     std::vector<Shard *> late;
+    for (Shard *m : members) m->swap_batches();
+    // a previous batch that no push_pull has seen yet (two preprocess calls in a row) is planned here, on the main
+    // stream, and waited for (the plan sizes the push buffers)
     for (Shard *m : members)
       if (!m->prev.planned) {
         m->plan_batch(m->prev);
         late.push_back(m);
       }
-    if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
+    {
+      StreamSwitch on(*this, index_stream);
+      if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
+      for (Shard *m : members) m->ingest_keys(keys[m->cfg.rank], n[m->cfg.rank], &m->mirror->key_err);
+      if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
+      HCTR_HIP(hipEventRecord(ev_keys, stream));
+    }
     // Only the first launches of the index go out here (they keep the GPU busy until the pushes arrive); the rest
     // follows from push_pull once the push kernels are in their queue.
-    HCTR_HIP(hipStreamWaitEvent(index_stream, ev_keys, 0));
     enqueue_index_all(1);
     index_rest_pending = true;
-    if (!late.empty() || time_calls) {
-      sync_stream();
-    } else { // the ids have been read: the caller may reuse its buffers
-      hipError_t e;
+    {
+      hipError_t e; // the ids have been read: the caller may reuse its buffers
       while ((e = hipEventQuery(ev_keys)) == hipErrorNotReady) {
       }
       HCTR_HIP(e);
     }
+    if (!late.empty()) sync_stream();
     for (Shard *m : late) m->finish_plan(m->prev);
     float ms = 0.f;
     if (time_calls) HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
@@ -1116,22 +1117,30 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
   for (Shard *m : members) m->generate_gradient(grads[m->cfg.rank], bag);
   if (time_calls) HCTR_HIP(hipEventRecord(ev_push, stream));
   if (nrank > 1) HCTR_HIP(hipEventRecord(ev_pushed, stream));
-  enqueue_index_rest(); // single shard: the push is in its queue, now the rest of the current batch's index
-  if (index_pending && nrank > 1) {
-    // the pushes are queued; the queries are built from the index of the current batches, which the host needs too
-    // (unique keys and queries per owner size the exchange)
-    index_pending = false;
-    wait_for(index_stream);
-    for (Shard *m : members) m->finish_index();
-    exchange_shapes();
-  }
+  enqueue_index_rest(); // the pushes are in their queue, now the rest of the current batches' index
   if (nrank > 1) {
-    // the push plans of the current batches, for the step in which they are the previous ones: after the pushes of
-    // this step (they move the update counters the plan reads), beside everything else the step still does
-    StreamSwitch on(*this, index_stream);
-    HCTR_HIP(hipStreamWaitEvent(stream, ev_pushed, 0));
-    for (Shard *m : members) m->plan_batch(m->cur);
-    HCTR_HIP(hipEventRecord(ev_plan, stream));
+    const bool wait_index = index_pending;
+    if (wait_index) HCTR_HIP(hipEventRecord(ev_index, index_stream));
+    {
+      // the push plans of the current batches, for the step in which they are the previous ones: after the pushes of
+      // this step (they move the update counters the plan reads), beside everything else the step still does; queued
+      // before the host looks at the index, so that nothing but the queries stands between that look and the exchange
+      StreamSwitch on(*this, index_stream);
+      HCTR_HIP(hipStreamWaitEvent(stream, ev_pushed, 0));
+      for (Shard *m : members) m->plan_batch(m->cur);
+      HCTR_HIP(hipEventRecord(ev_plan, stream));
+    }
+    if (wait_index) {
+      // the queries are built from the index of the current batches, which the host needs too (unique keys and queries
+      // per owner size the exchange)
+      index_pending = false;
+      hipError_t e;
+      while ((e = hipEventQuery(ev_index)) == hipErrorNotReady) {
+      }
+      HCTR_HIP(e);
+      for (Shard *m : members) m->finish_index();
+      exchange_shapes();
+    }
   }
   for (Shard *m : members) m->generate_query();
   const bool join_index = index_pending;
