@@ -76,8 +76,9 @@ def cpu_baseline(cfg, ks, batches, width, lr, steps):
     dst = np.empty((n, width), np.float32)
     o.preprocess_raw([batches[0]])
     o.push_pull_into([None], [dst])                       # warm-up: first pull, nothing to push yet
-    o.preprocess_raw([batches[1 % len(batches)]])
-    o.push_pull_into([grad], [dst])
+    for b in range(1, len(batches) + 2):                  # ... then every batch once: the rows they reach are paged in
+        o.preprocess_raw([batches[b % len(batches)]])
+        o.push_pull_into([grad], [dst])
     t0 = time.perf_counter()
     for s in range(steps):
         o.preprocess_raw([batches[(s + 2) % len(batches)]])

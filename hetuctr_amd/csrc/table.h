@@ -88,7 +88,10 @@ class Group;
 
 // launches of the sort that a deferred preprocess of a single shard enqueues itself: the column scan and the scatter
 // of the first pass and the count of the second (the first count comes from the key kernel)
-constexpr int kEarlySortSteps = 4;
+#ifndef HCTR_EARLY_SORT_STEPS
+#define HCTR_EARLY_SORT_STEPS 4
+#endif
+constexpr int kEarlySortSteps = HCTR_EARLY_SORT_STEPS;
 
 // stages whose device time can be measured separately (HIP events on the group's stream)
 enum Stage { S_KEYS = 0, S_SORT, S_UNIQUE, S_PLAN, S_PUSH, S_QUERY, S_EXCHANGE, S_OWNER, S_REFRESH, S_GATHER, S_COUNT };
