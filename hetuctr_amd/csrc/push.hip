@@ -133,11 +133,11 @@ __device__ __forceinline__ void move_counters(const TableView &t, int id_bits, c
   }
 }
 
-// Applies the finished sum of unique rank u (already multiplied by -lr) to column(s) `col`.
-// `counters`: this lane also moves the version / update counters.  Update types as in generate_query.cu:18-25.
+// Applies the finished sum of unique rank u (already multiplied by -lr) to column(s) `col`.  Update types as in
+// generate_query.cu:18-25.  The counters of the row move in the last blocks of the launch.
 template <int VEC, typename K>
 __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
-                                          uint32_t u, typename Vec<VEC>::T s, uint32_t col, bool counters) {
+                                          uint32_t u, typename Vec<VEC>::T s, uint32_t col) {
   typedef typename Vec<VEC>::T V;
   const slot_t o = p.uoff[u];
   const uint32_t W = t.width;
@@ -146,7 +146,6 @@ __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const
     V cur = *e;
     Vec<VEC>::add(cur, s);
     *e = cur;
-    if (counters) t.ver[o] += (version_t)(p.run_start[u + 1] - p.run_start[u]);
     return;
   }
   const bool need = a.need[u] != 0;
@@ -170,7 +169,6 @@ __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const
     }
     *g = pg;
   }
-  if (counters) move_counters<K>(t, id_bits, p, a, u, o, type, q);
 }
 
 // ---- short role ----------------------------------------------------------------------------------------
@@ -303,7 +301,6 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
           }
           *(V *)(t.pend + (size_t)off[i] * W + col) = g;
         }
-        if (c0 == 0 && gl == 0) move_counters<K>(t, id_bits, p, a, u0 + i, off[i], type[i], q[i]);
       }
     }
   }
@@ -367,7 +364,7 @@ __device__ __forceinline__ void medium_role(const TableView &t, int id_bits, con
         Vec<VEC>::add(e, scaled);
         *(V *)(t.emb + (size_t)off * W + col) = e; // versions: bump_versions
       } else {
-        apply_row<VEC, K>(t, id_bits, p, a, u, scaled, col, c0 == 0 && gl == 0);
+        apply_row<VEC, K>(t, id_bits, p, a, u, scaled, col);
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -665,7 +662,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
         if (col_ok) {
           const float scaled = acc * neg_lr;
           if (direct) t.emb[(size_t)m.w * W + mycol] = e + scaled;
-          else apply_row<1, K>(t, id_bits, p, a, m.x, scaled, mycol, slice == 0 && threadIdx.x == 0);
+          else apply_row<1, K>(t, id_bits, p, a, m.x, scaled, mycol);
         }
       }
     }
@@ -708,16 +705,24 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
     const uint32_t b = blockIdx.x - kLongBlocks - kMedBlocks;
     if (b < short_blocks) {
       short_role<VEC, LPR, K, kSingle, kPooled>(t, id_bits, p, a, b, U);
-    } else if (kSingle) {
-      // Single shard: every key is owned, so the only counter is the row version, which grows by the number of
-      // duplicates (generate_query.cu:68-69).  One thread per unique key, in the last blocks of the grid.
+    } else {
+      // The counters of every unique key, one thread per key, in the last blocks of the grid: they depend on the
+      // batch's index and plan only, not on the sums.
       const uint32_t u = (b - short_blocks) * kPushBlock + threadIdx.x;
-      // nontemporal: a counter line is touched once per step; left in the cache it is written back in the middle of
-      // the gather that follows
       if (u < U) {
-        version_t *vp = &t.ver[p.uoff[u]];
-        const version_t v = __builtin_nontemporal_load(vp) + (version_t)(p.run_start[u + 1] - p.run_start[u]);
-        __builtin_nontemporal_store(v, vp);
+        if (kSingle) {
+          // Single shard: every key is owned, so the only counter is the row version, which grows by the number of
+          // duplicates (generate_query.cu:68-69).  Nontemporal: a counter line is touched once per step; left in the
+          // cache it is written back in the middle of the gather that follows.
+          version_t *vp = &t.ver[p.uoff[u]];
+          const version_t v = __builtin_nontemporal_load(vp) + (version_t)(p.run_start[u + 1] - p.run_start[u]);
+          __builtin_nontemporal_store(v, vp);
+        } else {
+          const slot_t o = p.uoff[u];
+          const bool need = a.need[u] != 0;
+          const int type = o == kNoSlot ? 0 : ((uint32_t)o >= t.n_cached ? 1 : (need ? 2 : 3));
+          move_counters<K>(t, id_bits, p, a, u, o, type, a.prefix[u]);
+        }
       }
     }
   }
@@ -726,7 +731,7 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
 template <int VEC, int LPR, typename K, bool kSingle, bool kPooled>
 void launch_push_t(hipStream_t st, const TableView &t, int id_bits, const BatchView &p, uint32_t U, const PushArgs &a) {
   constexpr int kGroups = kPushBlock / LPR;
-  const unsigned ver_blocks = kSingle ? div_up(U, kPushBlock) : 0; // version counters of a single shard
+  const unsigned ver_blocks = div_up(U, kPushBlock); // the counters of every unique key
   const unsigned rest = kMedBlocks + div_up(U, kGroups * kRunsPerGroup) + ver_blocks;
   hipLaunchKernelGGL((push_fused<VEC, LPR, K, kSingle, kPooled>), dim3(kLongBlocks + rest), dim3(kPushBlock), 0, st, t, id_bits, p,
                      a, U);
