@@ -14,13 +14,16 @@ constexpr int kSortMaxBins = 1 << kSortMaxDigitBits;
 // Keys per thread, hence keys per tile (one block sorts one tile per pass), chosen by the size of the input: a small
 // input is cut into small tiles so that enough blocks share it (its passes are latency, not traffic); a huge one into
 // large tiles, because every tile costs a row of digit counts that is written, scanned and read again in every pass.
+#ifndef HCTR_SORT_ITEMS_DEFAULT
+#define HCTR_SORT_ITEMS_DEFAULT 8
+#endif
 #ifndef HCTR_SORT_ITEMS_LARGE
 #define HCTR_SORT_ITEMS_LARGE 16
 #endif
 #ifndef HCTR_SORT_ITEMS_SMALL
 #define HCTR_SORT_ITEMS_SMALL 2
 #endif
-constexpr int kSortItemsSmall = HCTR_SORT_ITEMS_SMALL, kSortItemsDefault = 8, kSortItemsLarge = HCTR_SORT_ITEMS_LARGE;
+constexpr int kSortItemsSmall = HCTR_SORT_ITEMS_SMALL, kSortItemsDefault = HCTR_SORT_ITEMS_DEFAULT, kSortItemsLarge = HCTR_SORT_ITEMS_LARGE;
 inline int sort_items(size_t n) {
   return n <= ((size_t)1 << 17) ? kSortItemsSmall : (n >= ((size_t)1 << 23) ? kSortItemsLarge : kSortItemsDefault);
 }
