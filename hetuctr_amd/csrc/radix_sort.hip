@@ -179,7 +179,6 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
     // lanes of this group with the same digit: one ballot per digit bit; a lane keeps the lanes that agree with it
     const uint64_t vm = __ballot(valid);
     uint32_t mlo = (uint32_t)vm, mhi = (uint32_t)(vm >> 32);
-#pragma unroll 10
     for (int b = 0; b < dbits; b++) {
       const uint32_t y = (uint32_t)__builtin_amdgcn_sbfe((int)d, b, 1); // all ones if the bit is set
       const uint64_t bal = __ballot(y != 0);
