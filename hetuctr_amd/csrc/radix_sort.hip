@@ -96,7 +96,8 @@ __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ 
   }
 }
 
-template <typename K, bool kFirst, int ITEMS>
+// DBITS: the digit width if known at compile time (the match loop is then straight-line code), else 0
+template <typename K, bool kFirst, int ITEMS, int DBITS>
 __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
                                                       K *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
                                                       uint32_t n, int shift, int dbits, uint32_t tiles,
@@ -179,11 +180,17 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
     // lanes of this group with the same digit: one ballot per digit bit; a lane keeps the lanes that agree with it
     const uint64_t vm = __ballot(valid);
     uint32_t mlo = (uint32_t)vm, mhi = (uint32_t)(vm >> 32);
-    for (int b = 0; b < dbits; b++) {
+    auto match_bit = [&](int b) {
       const uint32_t y = (uint32_t)__builtin_amdgcn_sbfe((int)d, b, 1); // all ones if the bit is set
       const uint64_t bal = __ballot(y != 0);
       mlo &= ~((uint32_t)bal ^ y);
       mhi &= ~((uint32_t)(bal >> 32) ^ y);
+    };
+    if (DBITS) {
+#pragma unroll
+      for (int b = 0; b < DBITS; b++) match_bit(b);
+    } else {
+      for (int b = 0; b < dbits; b++) match_bit(b);
     }
     const uint64_t m = ((uint64_t)mhi << 32) | mlo;
     // m: valid lanes of this group with the same digit (meaningless on invalid lanes)
@@ -292,17 +299,27 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
       hipLaunchKernelGGL(scan_tiles, dim3((nb + kScanCols - 1) / kScanCols), dim3(kScanBlock), 0, stream, counts, tiles,
                          nb, bin_total);
     if (wanted(2)) {
-#define CALL(I)                                                                                                     \
-  do {                                                                                                              \
-    if (p == 0)                                                                                                     \
-      hipLaunchKernelGGL((scatter<K, true, I>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n,  \
-                         shift, dbits, tiles, counts, bin_total);                                                   \
-    else                                                                                                            \
-      hipLaunchKernelGGL((scatter<K, false, I>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, \
-                         shift, dbits, tiles, counts, bin_total);                                                   \
+#define CALL3(I, F, D)                                                                                              \
+  hipLaunchKernelGGL((scatter<K, F, I, D>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift, \
+                     dbits, tiles, counts, bin_total)
+#define CALL2(I, F)                   \
+  do {                                \
+    switch (dbits) {                  \
+      case 8: CALL3(I, F, 8); break;  \
+      case 9: CALL3(I, F, 9); break;  \
+      case 10: CALL3(I, F, 10); break; \
+      default: CALL3(I, F, 0); break; \
+    }                                 \
+  } while (0)
+#define CALL(I)                \
+  do {                         \
+    if (p == 0) CALL2(I, true); \
+    else CALL2(I, false);      \
   } while (0)
       HCTR_SORT_ITEMS_DISPATCH(n, CALL);
 #undef CALL
+#undef CALL2
+#undef CALL3
     }
     HCTR_HIP(hipGetLastError());
     kin = kout;
