@@ -54,3 +54,36 @@ def test_random_configuration(seed):
         p.compare_state(1e-5, "case %d step %d" % (seed, step))
         prev_n = sizes
     p.close()
+
+
+@pytest.mark.parametrize("seed", list(range(16)))
+def test_random_call_sequences(seed):
+    """The two calls in any order a caller may use them: preprocess twice in a row (the skipped batch is pushed later or
+    never), push_pull again without a preprocess in between (the same previous batch is pushed once more by the same
+    plan), inference steps in between -- every call mirrored in the oracle, everything compared after every call."""
+    rs, nrank, width, length, bounds, root, storage, init, lr = make_case(100 + seed)
+    print("sequence case", seed, "nrank", nrank, "width", width, "length", length, "bounds", bounds, flush=True)
+    p = Pair(nrank, length, width, root, storage, init=init, lr=lr, bounds=bounds, seed=seed)
+    draw = zipf_sampler(length, 1.3, rs)
+    cur_n, prev_n = [0] * nrank, [0] * nrank
+    p.preprocess([np.zeros(0, np.int64)] * nrank)           # Pair.push_pull sizes its outputs from the last preprocess
+    for step in range(10):
+        op = int(rs.choice([0, 0, 1, 1, 1, 2]))            # 0: preprocess, 1: push_pull with gradients, 2: inference pull
+        where = "case %d call %d op %d" % (seed, step, op)
+        if op == 0:
+            sizes = [int(rs.choice([0, 5, 300, 2500, 20000])) for _ in range(nrank)]
+            keys = [draw(k) if k else np.zeros(0, np.int64) for k in sizes]
+            p.preprocess(keys, device_keys=bool(rs.integers(0, 2)))
+            p.compare_ints(INT_ITEMS_PRE, where)
+            prev_n, cur_n = cur_n, sizes
+        else:
+            grads = [None if op == 2 else rs.normal(0, 0.05, size=(prev_n[r], width)).astype(np.float32)
+                     for r in range(nrank)]
+            out, ref = p.push_pull(grads)
+            p.compare_ints(INT_ITEMS_POST, where)
+            for r in range(nrank):
+                assert_close(out[r], ref[r], 1e-5, "dst %s rank %d" % (where, r))
+            p.compare_state(1e-5, where)
+            if op == 2:
+                prev_n = [0] * nrank                         # an inference step drops the previous batch (hetu_gpu_table.cu:14-21)
+    p.close()
