@@ -591,7 +591,8 @@ void launch_plain_copy(hipStream_t s, const void *src, void *dst, size_t bytes) 
 void launch_copies(hipStream_t s, const CopyDesc *descs_device, uint32_t n, size_t max_bytes) {
   if (!n || !max_bytes) return;
   const unsigned bx = (unsigned)std::min<size_t>(1024, (max_bytes / 16 + kBlock - 1) / kBlock + 1);
-  hipLaunchKernelGGL(copy_segments, dim3(bx, n), dim3(kBlock), 0, s, descs_device);
+  for (uint32_t first = 0; first < n; first += 65535u) // the second grid dimension ends at 65535
+    hipLaunchKernelGGL(copy_segments, dim3(bx, std::min(n - first, 65535u)), dim3(kBlock), 0, s, descs_device + first);
   HCTR_HIP(hipGetLastError());
 }
 

@@ -255,3 +255,31 @@ def test_group_errors():
     with pytest.raises(RuntimeError, match="already exists"):
         capi.Table(0, 2, 0, "10.0.0.1", 999, 2, 4, 0, 0, root, np.array([0]), ("Zero", 0, 0), 0.1)
     t0.close()
+
+
+@pytest.mark.parametrize("nrank", [33, 200])
+def test_many_shards(nrank):
+    """More shards than any benchmark uses (the owner-side kernels walk up to 256 sources per target row, the exchanges
+    describe nrank * nrank segment pairs): three steps with caches and staleness against the oracle."""
+    rng = np.random.default_rng(nrank)
+    length, width = 5000, 12
+    root = rng.integers(0, nrank, size=length).astype(np.uint8)
+    storage = []
+    for r in range(nrank):
+        own, other = np.flatnonzero(root == r), np.flatnonzero(root != r)
+        storage.append(np.concatenate([own, rng.choice(other, other.shape[0] // 4, replace=False)]).astype(np.int64))
+    p = Pair(nrank, length, width, root, storage, init=("Uniform", -0.1, 0.1), lr=0.1, bounds=(1, 2))
+    draw = zipf_sampler(length, 1.2, rng)
+    prev = [0] * nrank
+    for step in range(3):
+        sizes = [int(rng.choice([0, 40, 400])) for _ in range(nrank)]
+        keys = [draw(k) if k else np.zeros(0, np.int64) for k in sizes]
+        p.preprocess(keys)
+        p.compare_ints(INT_ITEMS_PRE, "step %d" % step)
+        out, ref = p.push_pull([rng.normal(0, 0.1, size=(prev[r], width)).astype(np.float32) for r in range(nrank)])
+        p.compare_ints(INT_ITEMS_POST, "step %d" % step)
+        for r in range(nrank):
+            assert_close(out[r], ref[r], 1e-5, "dst step %d rank %d" % (step, r))
+        p.compare_state(1e-5, "step %d" % step)
+        prev = sizes
+    p.close()
