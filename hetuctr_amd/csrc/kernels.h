@@ -196,17 +196,19 @@ void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, co
 // requester: refresh cached rows that came back, then gather every key's row into dst
 struct PullArgs {
   const uint32_t *got;       // [U] or nullptr: nothing came back (nrank == 1)
-  const uint32_t *ret_i;     // [U] index into the returned rows
+  uint32_t *ret_i;           // [U] index into the returned rows (written by launch_refresh)
   uint32_t *src_row;         // [U] where the gather reads a key's row (written by launch_refresh): offset or returned row
   const version_t *in_ver;
   const embed_t *in_val;
   embed_t *dst;              // [n][width]
   bool stream_stores;        // write dst with nontemporal stores (see Shard::write_back)
 };
+// Index of every returned row per unique key (a.ret_i), where the gather reads each key's row (a.src_row), the counts of
+// the step and the refresh of the cached rows that came back.  tile_sums: scratch of scan_blocks(n_unique) words;
 // stats: five device words that read zero before the first call (the launch leaves them zero again); host_stats: four
 // words the device can write (hit / miss / refreshed counts of the step, error bits)
 void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
-                    uint32_t *stats, uint32_t *host_stats);
+                    uint32_t *tile_sums, uint32_t *stats, uint32_t *host_stats);
 void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a);
 // sum-pooled lookups: dst[b] = the rows of positions b * bag .. b * bag + bag - 1 added up in that order
 // (cur.idx_map must be filled: launch_idx_map)

@@ -264,34 +264,67 @@ __global__ void build_return_descs(ReturnPeers p, int nrank, uint32_t width, Cop
   o[1].bytes = (size_t)n * width * sizeof(embed_t);
 }
 
-// Counts of the step's remote unique keys: [0] cached and fresh enough, [1] not stored here, [2] cached and
-// refreshed; [3] bit 3: an owned row came back as outdated (it never may).  Atomics on one address are served one
-// after the other, so every thread counts its strided share in registers and a block adds its totals once.  The block
-// that finishes last hands the totals to the host (pinned memory) and puts the device counters back to zero for the
-// next step: no clearing launch before, no copy after.
-constexpr int kCountBlocks = 128;
-// The same pass leaves, per unique key, where the gather finds its row: the resident offset, or (top bit set) the
-// index among the returned rows; the gather then reaches a row in as many dependent loads as on a single shard.
+// What comes back per unique key of the step, in two launches over tiles of kRTile keys:
+//  got_tile_sums   returned rows per tile
+//  remote_emit     ret_i[u] = index of u's row among the returned rows (exclusive scan of the flags; a tile adds up the
+//                  sums of the tiles before it itself); src_row[u] = where the gather finds the row: the resident offset,
+//                  or (top bit set) that index; and the counts of the step: [0] cached and fresh enough, [1] not stored
+//                  here, [2] cached and refreshed, [3] bit 3: an owned row came back as outdated (it never may).
+// Atomics on one address are served one after the other, so every thread counts its keys in registers and a block
+// adds its totals once.  The block that finishes last hands the totals to the host (pinned memory) and puts the device
+// counters back to zero for the next step: no clearing launch before, no copy after.
 constexpr uint32_t kReturnedRow = 0x80000000u;
-__global__ __launch_bounds__(kBlock) void count_remote(TableView t, BatchView c, const uint32_t *__restrict__ got,
-                                                       const uint32_t *__restrict__ ret_i, uint32_t *__restrict__ src_row,
-                                                       uint32_t *__restrict__ stats, uint32_t *__restrict__ host_stats) {
+constexpr int kRItems = 8, kRTile = kBlock * kRItems; // 2048 keys: the tile scan_blocks() sizes the scratch for
+__global__ __launch_bounds__(kBlock) void got_tile_sums(const uint32_t *__restrict__ got, uint32_t U,
+                                                        uint32_t *__restrict__ tile_sums) {
+  __shared__ uint32_t sm[kBlock / kWave + 1];
+  const uint32_t j0 = blockIdx.x * kRTile + threadIdx.x * kRItems;
+  uint32_t c = 0;
+#pragma unroll
+  for (int k = 0; k < kRItems; k++) c += (j0 + k < U) ? got[j0 + k] : 0u;
+  uint32_t total;
+  block_exclusive_scan<kBlock>(c, sm, total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+__global__ __launch_bounds__(kBlock) void remote_emit(TableView t, BatchView c, const uint32_t *__restrict__ got,
+                                                      const uint32_t *__restrict__ tile_sums, uint32_t U,
+                                                      uint32_t *__restrict__ ret_i, uint32_t *__restrict__ src_row,
+                                                      uint32_t *__restrict__ stats, uint32_t *__restrict__ host_stats) {
+  __shared__ uint32_t sm[kBlock / kWave + 1];
   __shared__ uint32_t tot[4];
   __shared__ bool last;
   if (threadIdx.x < 4) tot[threadIdx.x] = 0;
-  __syncthreads();
-  const uint32_t U = *c.d_U;
+  uint32_t s = 0;
+  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlock) s += tile_sums[i];
+  uint32_t prefix;
+  block_exclusive_scan<kBlock>(s, sm, prefix); // its total: returned rows in the tiles before this one
+  const uint32_t j0 = blockIdx.x * kRTile + threadIdx.x * kRItems;
+  uint32_t g[kRItems], mine = 0;
+  slot_t o[kRItems];
+#pragma unroll
+  for (int k = 0; k < kRItems; k++) {
+    const bool in = j0 + k < U;
+    g[k] = in ? got[j0 + k] : 0u;
+    o[k] = in ? c.uoff[j0 + k] : 0;
+    mine += g[k];
+  }
+  uint32_t total;
+  uint32_t run = prefix + block_exclusive_scan<kBlock>(mine, sm, total);
   uint32_t n0 = 0, n1 = 0, n2 = 0, bad = 0;
-  for (uint32_t u = blockIdx.x * kBlock + threadIdx.x; u < U; u += kCountBlocks * kBlock) {
-    const slot_t o = c.uoff[u];
-    src_row[u] = o == kNoSlot ? (kReturnedRow | ret_i[u]) : (uint32_t)o;
-    if (o == kNoSlot) n1++;
-    else if ((uint32_t)o < t.n_cached) {
-      if (got[u]) n2++;
-      else n0++;
-    } else if (got[u]) {
-      bad = 8u;
+#pragma unroll
+  for (int k = 0; k < kRItems; k++) {
+    if (j0 + k < U) {
+      ret_i[j0 + k] = run;
+      src_row[j0 + k] = o[k] == kNoSlot ? (kReturnedRow | run) : (uint32_t)o[k];
+      if (o[k] == kNoSlot) n1++;
+      else if ((uint32_t)o[k] < t.n_cached) {
+        if (g[k]) n2++;
+        else n0++;
+      } else if (g[k]) {
+        bad = 8u;
+      }
     }
+    run += g[k];
   }
   for (int d = 32; d; d >>= 1) {
     n0 += __shfl_down(n0, d);
@@ -535,10 +568,12 @@ void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, co
 }
 
 void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
-                    uint32_t *stats, uint32_t *host_stats) {
+                    uint32_t *tile_sums, uint32_t *stats, uint32_t *host_stats) {
   if (!n_unique || !a.got) return;
-  hipLaunchKernelGGL(count_remote, dim3(kCountBlocks), dim3(kBlock), 0, s, t, cur, a.got, a.ret_i, a.src_row, stats,
-                     host_stats);
+  const unsigned tiles = div_up(n_unique, kRTile);
+  hipLaunchKernelGGL(got_tile_sums, dim3(tiles), dim3(kBlock), 0, s, a.got, n_unique, tile_sums);
+  hipLaunchKernelGGL(remote_emit, dim3(tiles), dim3(kBlock), 0, s, t, cur, a.got, tile_sums, n_unique, a.ret_i, a.src_row,
+                     stats, host_stats);
   const bool vec4 = t.width % 4 == 0;
   const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
 #define CALL(V, L) \

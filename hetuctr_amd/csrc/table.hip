@@ -515,15 +515,13 @@ void Shard::write_back(float *dst, uint32_t bag) {
     ret_i.reserve((size_t)std::max<uint32_t>(cur.U, 1) * 4);
     reserve_batch_scratch(cur.U);
     StageScope st(*group, S_REFRESH);
-    launch_exclusive_scan(s, got.as<uint32_t>(), ret_i.as<uint32_t>(), cur.U, nullptr, block_sums.as<uint32_t>(),
-                          nullptr);
     a.got = got.as<uint32_t>();
     a.ret_i = ret_i.as<uint32_t>();
     src_row.reserve((size_t)std::max<uint32_t>(cur.U, 1) * 4);
     a.src_row = src_row.as<uint32_t>();
     a.in_ver = in_ver.as<version_t>();
     a.in_val = in_val.as<embed_t>();
-    launch_refresh(s, tv, cur.view(), cur.U, a, stats.as<uint32_t>(), mirror->stats);
+    launch_refresh(s, tv, cur.view(), cur.U, a, sp.block_sums, stats.as<uint32_t>(), mirror->stats);
   }
   if (dst != nullptr) {
     StageScope st(*group, S_GATHER);
