@@ -154,8 +154,9 @@ void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const B
                  const PushArgs &a);
 
 // ---- query / owner side / pull -------------------------------------------------------------------------
-void launch_lookup_version(hipStream_t s, const TableView &t, const BatchView &cur, version_t *q_ver);
-void launch_unique_ids(hipStream_t s, const KeyLayout &kl, const BatchView &cur, index_t *q_idx);
+// id and local version of every unique key of the current batch (n_unique: the host's count of them)
+void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t n_unique,
+                          index_t *q_idx, version_t *q_ver);
 // Owner side of a step: applying the received pushes (per target row in source order) and serving the received
 // queries (outdated flags, positions of the rows to return, rows packed, first returned row of every requester).
 // One entry per shard of the group; one set of launches serves them all.

@@ -15,18 +15,16 @@ template <int VEC> struct RowVec;
 template <> struct RowVec<4> { typedef floatx4 T; };
 template <> struct RowVec<1> { typedef float T; };
 
-__global__ __launch_bounds__(kBlock) void lookup_version(TableView t, BatchView c, version_t *__restrict__ q_ver) {
+// The queries of a step (csrc/core/generate_query.cu:91-106): per unique key its id and the version of the local copy
+// (invalid if the key is not resident here).
+template <typename K>
+__global__ __launch_bounds__(kBlock) void build_queries(TableView t, int id_bits, BatchView c, index_t *__restrict__ q_idx,
+                                                        version_t *__restrict__ q_ver) {
   const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
   if (u >= *c.d_U) return;
   const slot_t o = c.uoff[u];
-  q_ver[u] = o != kNoSlot ? t.ver[o] : kInvalidVersion;
-}
-
-template <typename K>
-__global__ __launch_bounds__(kBlock) void unique_ids(int id_bits, BatchView c, index_t *__restrict__ q_idx) {
-  const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
-  if (u >= *c.d_U) return;
   q_idx[u] = (index_t)(((const K *)c.ukey)[u] & (K)(((uint64_t)1 << id_bits) - 1));
+  q_ver[u] = o != kNoSlot ? t.ver[o] : kInvalidVersion;
 }
 
 // ---- owner side: every kernel below serves ALL shards of a loopback group in one launch (blockIdx.y = shard), the
@@ -511,16 +509,12 @@ inline int lanes_for(uint32_t width, int vec) {
 
 } // namespace
 
-void launch_lookup_version(hipStream_t s, const TableView &t, const BatchView &cur, version_t *q_ver) {
-  if (!cur.n) return;
-  hipLaunchKernelGGL(lookup_version, dim3(div_up(cur.n, kBlock)), dim3(kBlock), 0, s, t, cur, q_ver);
-  HCTR_HIP(hipGetLastError());
-}
-
-void launch_unique_ids(hipStream_t s, const KeyLayout &kl, const BatchView &cur, index_t *q_idx) {
-  if (!cur.n) return;
-  if (kl.wide) hipLaunchKernelGGL(unique_ids<uint64_t>, dim3(div_up(cur.n, kBlock)), dim3(kBlock), 0, s, kl.id_bits, cur, q_idx);
-  else hipLaunchKernelGGL(unique_ids<uint32_t>, dim3(div_up(cur.n, kBlock)), dim3(kBlock), 0, s, kl.id_bits, cur, q_idx);
+void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t n_unique,
+                          index_t *q_idx, version_t *q_ver) {
+  if (!n_unique) return;
+  const dim3 grid(div_up(n_unique, kBlock));
+  if (kl.wide) hipLaunchKernelGGL(build_queries<uint64_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, q_idx, q_ver);
+  else hipLaunchKernelGGL(build_queries<uint32_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, q_idx, q_ver);
   HCTR_HIP(hipGetLastError());
 }
 

@@ -439,8 +439,7 @@ void Shard::generate_query() {
   q_idx.reserve((size_t)std::max<uint32_t>(cur.U, 1) * sizeof(index_t));
   q_ver.reserve((size_t)std::max<uint32_t>(cur.U, 1) * sizeof(version_t));
   StageScope st(*group, S_QUERY);
-  launch_lookup_version(s, tv, cur.view(), q_ver.as<version_t>());
-  launch_unique_ids(s, kl, cur.view(), q_idx.as<index_t>());
+  launch_build_queries(s, tv, kl, cur.view(), cur.U, q_idx.as<index_t>(), q_ver.as<version_t>());
 }
 
 // What the owner-side kernels need of this shard for the step (csrc/core/handle_query.cu:7-116): the received pushes
