@@ -894,12 +894,7 @@ void Group::exchange_return() {
 // csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
 // Waits for the stream by polling: the calls are short and a blocking wait adds tens of microseconds of
 // wake-up latency to each of them.
-void Group::sync_stream() {
-  hipError_t e;
-  while ((e = hipStreamQuery(stream)) == hipErrorNotReady) {
-  }
-  HCTR_HIP(e);
-}
+void Group::sync_stream() { HCTR_HIP(hipStreamSynchronize(stream)); }
 
 namespace {
 void wait_for(hipStream_t s) {
