@@ -897,12 +897,7 @@ void Group::exchange_return() {
 void Group::sync_stream() { HCTR_HIP(hipStreamSynchronize(stream)); }
 
 namespace {
-void wait_for(hipStream_t s) {
-  hipError_t e;
-  while ((e = hipStreamQuery(s)) == hipErrorNotReady) {
-  }
-  HCTR_HIP(e);
-}
+void wait_for(hipStream_t s) { HCTR_HIP(hipStreamSynchronize(s)); }
 } // namespace
 
 // Enqueues index stages of the ingested batch (single shard) on the stream the stages currently use.
@@ -972,10 +967,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     HCTR_HIP(hipEventRecord(ev_keys, stream));
     enqueue_index(m, 1);
     index_rest_pending = true;
-    hipError_t e;
-    while ((e = hipEventQuery(ev_keys)) == hipErrorNotReady) {
-    }
-    HCTR_HIP(e);
+    HCTR_HIP(hipEventSynchronize(ev_keys));
     if (time_calls) {
       float ms = 0.f;
       HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
@@ -1013,12 +1005,7 @@ void Group::preprocess_all(const int64_t *const *keys, const size_t *n) {
     // follows from push_pull once the push kernels are in their queue.
     enqueue_index_all(1);
     index_rest_pending = true;
-    {
-      hipError_t e; // the ids have been read: the caller may reuse its buffers
-      while ((e = hipEventQuery(ev_keys)) == hipErrorNotReady) {
-      }
-      HCTR_HIP(e);
-    }
+    HCTR_HIP(hipEventSynchronize(ev_keys)); // the ids have been read: the caller may reuse its buffers
     if (!late.empty()) sync_stream();
     for (Shard *m : late) m->finish_plan(m->prev);
     float ms = 0.f;
@@ -1126,10 +1113,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
       // the queries are built from the index of the current batches, which the host needs too (unique keys and queries
       // per owner size the exchange)
       index_pending = false;
-      hipError_t e;
-      while ((e = hipEventQuery(ev_index)) == hipErrorNotReady) {
-      }
-      HCTR_HIP(e);
+      HCTR_HIP(hipEventSynchronize(ev_index));
       for (Shard *m : members) m->finish_index();
       exchange_shapes();
     }
