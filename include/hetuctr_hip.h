@@ -140,8 +140,10 @@ int hctr_stream(hctr_table *t, void **stream_out);
  * switches the measurement on for the calls that follow. */
 int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
 
-/* hctr_preprocess returns as soon as the caller's ids have been read (the buffer may be reused) and, with several
- * shards, the push plan of the previous batch is made.  The sort / unique stages of that batch keep running on a
+/* hctr_preprocess returns as soon as the caller's ids have been read (the buffer may be reused).  With several shards
+ * the push plan of the previous batch was made at the end of the step before (only a batch that no hctr_push_pull has
+ * seen, e.g. after two hctr_preprocess calls in a row, is planned, and waited for, in this call).  The sort / unique
+ * stages of the new batch keep running on a
  * second stream, next to the gradient push that the following hctr_push_pull starts, and are waited for before the
  * rows are gathered (several shards: before the queries are built).  preprocess_ms above is then the time up to
  * that return, push_pull_ms covers the rest.  Anything that needs the batch's index earlier (a second hctr_preprocess,
