@@ -1,6 +1,6 @@
 // Stable LSD radix sort for gfx950, 64-lane wavefronts.
 //
-// One pass = three launches, nothing waits on another block inside a kernel and no global atomics are used
+// One pass = three launches (two for a small input, see kSelfScanTiles), nothing waits on another block inside a kernel and no global atomics are used
 // (device-scope atomics are two orders of magnitude slower than plain stores on this part):
 //   digit_histogram   per-tile digit counts -> counts[tile][bin], rows written whole
 //   scan_tiles        per bin: exclusive scan of its column over the tiles + the bin's total
@@ -53,6 +53,9 @@ __global__ __launch_bounds__(kSortBlock) void digit_histogram(const K *__restric
 #ifndef HCTR_SCAN_COLS
 #define HCTR_SCAN_COLS 16
 #endif
+#ifndef HCTR_SELF_SCAN_TILES
+#define HCTR_SELF_SCAN_TILES 64
+#endif
 constexpr int kScanBlock = 512, kScanCols = HCTR_SCAN_COLS, kScanParts = kScanBlock / kScanCols, kScanKeep = 16;
 __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ counts, uint32_t tiles, uint32_t nb,
                                                          uint32_t *__restrict__ bin_total) {
@@ -96,8 +99,14 @@ __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ 
   }
 }
 
+// An input of at most this many tiles is sorted without the scan launches: every scatter block adds up the columns of
+// the raw counts itself (a few rows from L2 cost less than a launch on a chain of dependent kernels).
+constexpr uint32_t kSelfScanTiles = HCTR_SELF_SCAN_TILES;
+constexpr int kSelfScanAhead = 32;         // rows of counts requested together
+
 // DBITS: the digit width if known at compile time (the match loop is then straight-line code), else 0
-template <typename K, bool kFirst, int ITEMS, int DBITS>
+// kSelfScan: tile_prefix holds the raw counts of digit_histogram, bin_total is not read
+template <typename K, bool kFirst, int ITEMS, int DBITS, bool kSelfScan>
 __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
                                                       K *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
                                                       uint32_t n, int shift, int dbits, uint32_t tiles,
@@ -149,11 +158,29 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
   // earlier tiles
   {
     uint32_t all[2] = {0, 0}, mine[2] = {0, 0};
+    if (kSelfScan) {
+      for (int q = 0; q < 2; q++) {
+        if (blo + q < bhi) {
+          const uint32_t *col = tile_prefix + blo + q;
+          for (uint32_t t0 = 0; t0 < tiles; t0 += kSelfScanAhead) {
+            uint32_t v[kSelfScanAhead];
 #pragma unroll
-    for (int q = 0; q < 2; q++) {
-      if (blo + q < bhi) {
-        all[q] = bin_total[blo + q];
-        mine[q] = tile_prefix[(size_t)tile * nb + blo + q];
+            for (int u = 0; u < kSelfScanAhead; u++) v[u] = t0 + u < tiles ? col[(size_t)(t0 + u) * nb] : 0u;
+#pragma unroll
+            for (int u = 0; u < kSelfScanAhead; u++) {
+              all[q] += v[u];
+              mine[q] += t0 + u < tile ? v[u] : 0u;
+            }
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 2; q++) {
+        if (blo + q < bhi) {
+          all[q] = bin_total[blo + q];
+          mine[q] = tile_prefix[(size_t)tile * nb + blo + q];
+        }
       }
     }
     uint32_t total;
@@ -277,6 +304,7 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
   uint32_t *counts = scratch.words;
   uint32_t *bin_total = scratch.words + (size_t)tiles * kSortMaxBins;
   const int passes = (bits + kSortMaxDigitBits - 1) / kSortMaxDigitBits;
+  const bool self_scan = sort_items(n) == kSortItemsSmall && tiles <= kSelfScanTiles;
   int shift = 0;
   const K *kin = keys_in;
   const uint32_t *vin = nullptr;
@@ -295,13 +323,18 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
       HCTR_SORT_ITEMS_DISPATCH(n, CALL);
 #undef CALL
     }
-    if (wanted(1))
+    if (wanted(1) && !self_scan)
       hipLaunchKernelGGL(scan_tiles, dim3((nb + kScanCols - 1) / kScanCols), dim3(kScanBlock), 0, stream, counts, tiles,
                          nb, bin_total);
     if (wanted(2)) {
-#define CALL3(I, F, D)                                                                                              \
-  hipLaunchKernelGGL((scatter<K, F, I, D>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, shift, \
-                     dbits, tiles, counts, bin_total)
+#define CALL4(I, F, D, S)                                                                                     \
+  hipLaunchKernelGGL((scatter<K, F, I, D, S>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, \
+                     shift, dbits, tiles, counts, bin_total)
+#define CALL3(I, F, D)                                                      \
+  do {                                                                      \
+    if (self_scan && I == kSortItemsSmall) CALL4(I, F, D, (I == kSortItemsSmall)); \
+    else CALL4(I, F, D, false);                                             \
+  } while (0)
 #define CALL2(I, F)                   \
   do {                                \
     switch (dbits) {                  \
@@ -320,6 +353,7 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
 #undef CALL
 #undef CALL2
 #undef CALL3
+#undef CALL4
     }
     HCTR_HIP(hipGetLastError());
     kin = kout;

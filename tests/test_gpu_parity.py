@@ -286,6 +286,31 @@ def test_repeated_and_changing_batch_sizes():
     p.close()
 
 
+@pytest.mark.parametrize("nrank", [1, 2])
+def test_batch_sizes_where_the_sort_changes_shape(nrank):
+    # 1024-key tiles up to 2^17 keys (up to 64 of them without scan launches), 4096-key tiles above: the sizes on both
+    # sides of every switch, one after the other on one table (the scratch of one size is reused by the next)
+    say("sort shapes, shards", nrank)
+    rng = np.random.default_rng(35 + nrank)
+    length, width = 3_000_000, 4                           # 22-bit ids (+ 1 bit of rank): three digit widths in a sort
+    root = rng.integers(0, nrank, size=length).astype(np.uint8)
+    storage = [np.flatnonzero(root == r).astype(np.int64) for r in range(nrank)]
+    p = Pair(nrank, length, width, root, storage, init=("Zero", 0.0, 0.0), lr=0.5)
+    sizes = [1024, 1025, 65536, 65537, 65536 + 1024, 131072, 131073, 1023, 140_000, 64 * 1024 - 1]
+    prev_n = [0] * nrank
+    for step, n in enumerate(sizes):
+        ns = [n if r == 0 else max(n // 3, 1) for r in range(nrank)]
+        keys = [rng.integers(0, length, size=k).astype(np.int64) for k in ns]
+        p.preprocess(keys, device_keys=True)
+        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.SIZES], "n %d" % n)
+        out, ref = p.push_pull([rng.normal(0, 1e-2, size=(k, width)).astype(np.float32) for k in prev_n])
+        for r in range(nrank):
+            assert_close(out[r], ref[r], 1e-5, "dst n %d rank %d" % (n, r))
+        prev_n = ns
+    p.compare_state(1e-5, "end")
+    p.close()
+
+
 def test_key_error_is_raised_by_preprocess_and_the_table_goes_on():
     say("bad key, early return")
     length, width, n = 1000, 8, 500
