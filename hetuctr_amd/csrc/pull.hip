@@ -362,7 +362,7 @@ __global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, Pull
   const uint32_t gl = threadIdx.x % LPR, W = t.width;
   const slot_t o = c.uoff[u];
   const bool got = a.got[u] != 0;
-  if (!got || o == kNoSlot || (uint32_t)o >= t.n_cached) return; // (an owned row that came back is reported by count_remote)
+  if (!got || o == kNoSlot || (uint32_t)o >= t.n_cached) return; // (an owned row that came back is reported by remote_emit)
   const uint32_t k = a.ret_i[u];
   if (gl == 0) t.ver[o] = a.in_ver[k];
   for (uint32_t col = gl * VEC; col < W; col += LPR * VEC)
