@@ -149,6 +149,10 @@ struct PushArgs {
   version_t *g_cnt;
   embed_t *g_val;
 };
+// pos[u] = prefix[u] + delta[owner of unique key u] for the n_unique unique keys of `prev`: the place of a pushed row in
+// a receive area shared by all owners, from its place in the shard's own plan (delta: nrank words in device memory)
+void launch_place_rows(hipStream_t s, const KeyLayout &kl, const BatchView &prev, uint32_t n_unique,
+                       const uint32_t *prefix, const uint32_t *delta, uint32_t *pos);
 // n_unique: number of unique keys of `prev` (host copy)
 void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &prev, uint32_t n_unique,
                  const PushArgs &a);

@@ -728,6 +728,14 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
   }
 }
 
+template <typename K>
+__global__ __launch_bounds__(256) void place_rows(const K *__restrict__ ukey, uint32_t U, int id_bits,
+                                                  const uint32_t *__restrict__ prefix,
+                                                  const uint32_t *__restrict__ delta, uint32_t *__restrict__ pos) {
+  const uint32_t u = blockIdx.x * 256 + threadIdx.x;
+  if (u < U) pos[u] = prefix[u] + delta[(uint32_t)(ukey[u] >> id_bits)];
+}
+
 template <int VEC, int LPR, typename K, bool kSingle, bool kPooled>
 void launch_push_t(hipStream_t st, const TableView &t, int id_bits, const BatchView &p, uint32_t U, const PushArgs &a) {
   constexpr int kGroups = kPushBlock / LPR;
@@ -763,6 +771,18 @@ void launch_push_k(hipStream_t ps, const TableView &t, int id_bits, const BatchV
 }
 
 } // namespace
+
+void launch_place_rows(hipStream_t s, const KeyLayout &kl, const BatchView &prev, uint32_t n_unique,
+                       const uint32_t *prefix, const uint32_t *delta, uint32_t *pos) {
+  if (!n_unique) return;
+  if (kl.wide)
+    hipLaunchKernelGGL(place_rows<uint64_t>, dim3(div_up(n_unique, 256)), dim3(256), 0, s, (const uint64_t *)prev.ukey,
+                       n_unique, kl.id_bits, prefix, delta, pos);
+  else
+    hipLaunchKernelGGL(place_rows<uint32_t>, dim3(div_up(n_unique, 256)), dim3(256), 0, s, (const uint32_t *)prev.ukey,
+                       n_unique, kl.id_bits, prefix, delta, pos);
+  HCTR_HIP(hipGetLastError());
+}
 
 void launch_push(hipStream_t ps, const TableView &t, const KeyLayout &kl, const BatchView &prev, uint32_t n_unique,
                  const PushArgs &a) {

@@ -129,7 +129,9 @@ class Shard {
   void finish_plan(Batch &b); // takes the counts over into b once they are there
   void finish_index();
   void check_key_error();                   // raises if the ingested batch held a key outside [0, length)
-  void generate_gradient(const float *grad, uint32_t bag = 1);
+  // the push of a step in two halves, so that a group can place every shard's pushed rows before any push kernel runs
+  void begin_push(const float *grad, uint32_t bag = 1);  // which batch is pushed (none on an inference step), checks
+  void generate_gradient(const uint32_t *delta);         // the push kernel; delta: see Group::place_pushes
   void generate_query();
   void fill_owner_args(OwnerShard &o);      // handleGradient + handleQuery: what the group's owner-side launches need
   void finish_handle_query();               // after the step: return counts and error flags from the pinned block
@@ -155,10 +157,14 @@ class Shard {
   DevStat *dst_ = nullptr; // == dstat.p
   uint32_t *err_ptr() const { return &dst_->err; }
   // send side
-  DeviceBuf q_idx, q_ver, g_idx, g_cnt, g_val;
+  DeviceBuf q_idx, q_ver;
+  const float *push_grad_ = nullptr; // arguments of the push between begin_push and generate_gradient
+  uint32_t push_bag_ = 1;
   // receive side (owner role)
-  DeviceBuf rq_idx, rq_ver, rg_idx, rg_cnt, rg_val, outdated, ret_slot, q_slot, src_row, ret_ver, ret_val, ret_seg_dev;
+  DeviceBuf rq_idx, rq_ver, outdated, ret_slot, q_slot, src_row, ret_ver, ret_val, ret_seg_dev;
   std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
+  uint64_t rg_base = 0;      // first row of this shard's piece of the group's receive area for pushed rows
+  DeviceBuf push_pos;        // place of every unique key's pushed row in that area (plan position + distance)
   // requester side of the return
   DeviceBuf got, ret_i, in_ver, in_val;
   HostMirror *mirror = nullptr;
@@ -205,6 +211,12 @@ class Group {
   OwnerShard *owner_host = nullptr;
   DeviceBuf owner_dev;
   void owner_side();
+  // Where every shard's pushed rows go: one receive area for the whole group (ids, counts, rows), cut into one piece
+  // per owner and, inside it, per source; sized from the plans before any push kernel runs.  Every sender gets, per
+  // owner, the distance between a row's place in its own plan and its place in the area (nrank words per sender).
+  void place_pushes();
+  DeviceBuf rg_idx_all, rg_cnt_all, rg_val_all, push_delta_dev;
+  uint32_t *push_delta_host = nullptr;   // pinned staging of the distances
   bool time_calls = false;               // bracket the two calls with events (hctr_last_times switches it on)
   std::vector<Shard *> members;
   DeviceBuf desc_dev[2];                 // copy descriptors of the query exchange [0] and of the return exchange [1]

@@ -393,7 +393,7 @@ void Shard::check_key_error() {
 }
 
 // csrc/core/generate_query.cu:85-89; inference rule of csrc/core/hetu_gpu_table.cu:14-21
-void Shard::generate_gradient(const float *grad, uint32_t bag) {
+void Shard::begin_push(const float *grad, uint32_t bag) {
   hipStream_t s = group->stream;
   if (grad == nullptr) {
     prev.n = 0;
@@ -404,31 +404,37 @@ void Shard::generate_gradient(const float *grad, uint32_t bag) {
   }
   prev_active = prev.n > 0;
   last_stats[3] = 0;
+  push_grad_ = grad;
+  push_bag_ = bag;
   if (!prev_active) return;
   uint64_t pushes = 0;
   for (int i = 0; i < cfg.nrank; i++) pushes += prev.push_cnt[i];
   last_stats[3] = (long long)pushes;
-  const size_t W = cfg.width;
   HCTR_CHECK(prev.n % bag == 0, "pooled push: the previous batch is not a whole number of bags");
+}
+
+void Shard::generate_gradient(const uint32_t *delta) {
+  if (!prev_active) return;
+  hipStream_t s = group->stream;
   PushArgs a;
-  a.grad = grad;
-  a.bag = BagDiv(bag);
+  a.grad = push_grad_;
+  a.bag = BagDiv(push_bag_);
   a.need = nullptr;
   a.prefix = nullptr;
   a.g_idx = nullptr;
   a.g_cnt = nullptr;
   a.g_val = nullptr;
-  if (cfg.nrank > 1) {
-    g_idx.reserve(std::max<uint64_t>(pushes, 1) * sizeof(index_t));
-    g_cnt.reserve(std::max<uint64_t>(pushes, 1) * sizeof(version_t));
-    g_val.reserve(std::max<uint64_t>(pushes, 1) * W * sizeof(embed_t));
-    a.need = prev.need.as<uint32_t>();
-    a.prefix = prev.prefix.as<uint32_t>();
-    a.g_idx = g_idx.as<index_t>();
-    a.g_cnt = g_cnt.as<version_t>();
-    a.g_val = g_val.as<embed_t>();
-  }
   StageScope st(*group, S_PUSH);
+  if (cfg.nrank > 1) {
+    // the pushed rows go straight into the group's receive area: plan position -> position there
+    push_pos.reserve((size_t)std::max<uint32_t>(prev.U, 1) * 4);
+    launch_place_rows(s, kl, prev.view(), prev.U, prev.prefix.as<uint32_t>(), delta, push_pos.as<uint32_t>());
+    a.need = prev.need.as<uint32_t>();
+    a.prefix = push_pos.as<uint32_t>();
+    a.g_idx = group->rg_idx_all.as<index_t>();
+    a.g_cnt = group->rg_cnt_all.as<version_t>();
+    a.g_val = group->rg_val_all.as<embed_t>();
+  }
   launch_push(s, tv, kl, prev.view(), prev.U, a);
 }
 
@@ -457,9 +463,9 @@ void Shard::fill_owner_args(OwnerShard &o) {
   query_sums.reserve((query_tiles(Q) + 2) * 4);
   last_stats[5] = (long long)rg_seg[R];
   o.t = tv;
-  o.rg_idx = rg_idx.as<index_t>();
-  o.rg_cnt = rg_cnt.as<version_t>();
-  o.rg_val = rg_val.as<embed_t>();
+  o.rg_idx = group->rg_idx_all.as<index_t>() + rg_base;
+  o.rg_cnt = group->rg_cnt_all.as<version_t>() + rg_base;
+  o.rg_val = group->rg_val_all.as<embed_t>() + rg_base * cfg.width;
   o.longest = 0;
   for (int i = 0; i <= R; i++) {
     o.rg_seg[i] = (uint32_t)rg_seg[i];
@@ -685,6 +691,7 @@ Group::~Group() {
   if (ev_pushed) (void)hipEventDestroy(ev_pushed);
   if (ev_plan) (void)hipEventDestroy(ev_plan);
   if (owner_host) (void)hipHostFree(owner_host);
+  if (push_delta_host) (void)hipHostFree(push_delta_host);
 }
 
 void Group::join(Shard *s) {
@@ -797,46 +804,73 @@ void Group::run_copies(std::vector<CopyDesc> &descs) {
   descs.clear();
 }
 
-// csrc/core/all2all.cu:18-87: every receive buffer is the senders' buckets for this shard, in source order
+// The pushes of a step never pass through a send buffer: a pushed row is written by the push kernel into the receive
+// area of its owner (csrc/core/all2all.cu:48-87 moves it there in the reference).  How many rows every shard pushes to
+// every owner is known from the plans before any push kernel starts, so the area is sized and cut here: one piece per
+// owner, inside it one per source, both in rank order.  In one process the area is one allocation; between GPUs every
+// owner would hold its piece and hand its address to the others.
+void Group::place_pushes() {
+  const int R = nrank;
+  if (R == 1) return;
+  if (!push_delta_host) {
+    HCTR_HIP(hipHostMalloc((void **)&push_delta_host, (size_t)R * R * sizeof(uint32_t), hipHostMallocDefault));
+    push_delta_dev.reserve((size_t)R * R * sizeof(uint32_t));
+  }
+  uint64_t total = 0;
+  for (int d = 0; d < R; d++) {
+    Shard &dst = *members[d];
+    dst.rg_base = total;
+    uint64_t G = 0;
+    for (int s = 0; s < R; s++) {
+      dst.rg_seg[s] = G;
+      if (members[s]->prev_active) G += members[s]->prev.push_cnt[d];
+    }
+    dst.rg_seg[R] = G;
+    total += G;
+  }
+  HCTR_CHECK(total < 0xfffffff0ull, "more than 2^32 rows are pushed in one step");
+  if (!total) return;
+  const size_t W = members[0]->cfg.width;
+  rg_idx_all.reserve(total * sizeof(index_t));
+  rg_cnt_all.reserve(total * sizeof(version_t));
+  rg_val_all.reserve(total * W * sizeof(embed_t));
+  for (int s = 0; s < R; s++) {
+    Shard &src = *members[s];
+    uint64_t glo = 0; // rows of this source for the owners before d
+    for (int d = 0; d < R; d++) {
+      const Shard &dst = *members[d];
+      // (place in the area) - (place in the source's plan), modulo 2^32 like the sum the kernel forms
+      push_delta_host[(size_t)s * R + d] = (uint32_t)(dst.rg_base + dst.rg_seg[s] - glo);
+      if (src.prev_active) glo += src.prev.push_cnt[d];
+    }
+  }
+  HCTR_HIP(hipMemcpyAsync(push_delta_dev.p, push_delta_host, (size_t)R * R * sizeof(uint32_t), hipMemcpyHostToDevice, stream));
+}
+
+// csrc/core/all2all.cu:18-46: every receive buffer is the senders' buckets for this shard, in source order (the
+// queries; the pushed rows are in place already, see place_pushes)
 void Group::exchange_query() {
   const int R = nrank;
   std::vector<CopyDesc> descs;
   for (int d = 0; d < R; d++) {
     Shard &dst = *members[d];
-    const size_t W = dst.cfg.width;
-    uint64_t Q = 0, G = 0;
+    uint64_t Q = 0;
     for (int s = 0; s < R; s++) {
-      Shard &src = *members[s];
       dst.rq_seg[s] = Q;
-      dst.rg_seg[s] = G;
-      Q += src.cur.send_cnt[d];
-      if (src.prev_active) G += src.prev.push_cnt[d];
+      Q += members[s]->cur.send_cnt[d];
     }
     dst.rq_seg[R] = Q;
-    dst.rg_seg[R] = G;
-    HCTR_CHECK(Q < 0xfffffff0ull && G < 0xfffffff0ull, "more than 2^32 rows arrive at one shard");
+    HCTR_CHECK(Q < 0xfffffff0ull, "more than 2^32 queries arrive at one shard");
     dst.rq_idx.reserve(std::max<uint64_t>(Q, 1) * sizeof(index_t));
     dst.rq_ver.reserve(std::max<uint64_t>(Q, 1) * sizeof(version_t));
-    dst.rg_idx.reserve(std::max<uint64_t>(G, 1) * sizeof(index_t));
-    dst.rg_cnt.reserve(std::max<uint64_t>(G, 1) * sizeof(version_t));
-    dst.rg_val.reserve(std::max<uint64_t>(G, 1) * W * sizeof(embed_t));
     for (int s = 0; s < R; s++) {
       Shard &src = *members[s];
-      uint64_t qlo = 0, glo = 0;
-      for (int i = 0; i < d; i++) {
-        qlo += src.cur.send_cnt[i];
-        glo += src.prev.push_cnt[i];
-      }
+      uint64_t qlo = 0;
+      for (int i = 0; i < d; i++) qlo += src.cur.send_cnt[i];
       const uint64_t qn = src.cur.send_cnt[d];
       if (qn) {
         descs.push_back({src.q_idx.as<index_t>() + qlo, dst.rq_idx.as<index_t>() + dst.rq_seg[s], qn * sizeof(index_t)});
         descs.push_back({src.q_ver.as<version_t>() + qlo, dst.rq_ver.as<version_t>() + dst.rq_seg[s], qn * sizeof(version_t)});
-      }
-      const uint64_t gn = src.prev_active ? src.prev.push_cnt[d] : 0;
-      if (gn) {
-        descs.push_back({src.g_idx.as<index_t>() + glo, dst.rg_idx.as<index_t>() + dst.rg_seg[s], gn * sizeof(index_t)});
-        descs.push_back({src.g_cnt.as<version_t>() + glo, dst.rg_cnt.as<version_t>() + dst.rg_seg[s], gn * sizeof(version_t)});
-        descs.push_back({src.g_val.as<embed_t>() + glo * W, dst.rg_val.as<embed_t>() + dst.rg_seg[s] * W, gn * W * sizeof(embed_t)});
       }
     }
   }
@@ -1093,7 +1127,10 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
   if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
-  for (Shard *m : members) m->generate_gradient(grads[m->cfg.rank], bag);
+  for (Shard *m : members) m->begin_push(grads[m->cfg.rank], bag);
+  place_pushes();
+  for (Shard *m : members)
+    m->generate_gradient(nrank > 1 ? push_delta_dev.as<uint32_t>() + (size_t)nrank * m->cfg.rank : nullptr);
   if (time_calls) HCTR_HIP(hipEventRecord(ev_push, stream));
   if (nrank > 1) HCTR_HIP(hipEventRecord(ev_pushed, stream));
   enqueue_index_rest(); // the pushes are in their queue, now the rest of the current batches' index
