@@ -181,23 +181,22 @@ struct OwnerShard {
   uint32_t *outdated, *tile_cnt;
   slot_t *q_slot;            // slot of every received query (kNoSlot: not owned here)
   slot_t *ret_slot;          // slots of the rows to return, in return order
-  version_t *ret_ver;
-  embed_t *ret_val;
+  // The returned rows are written straight into the requesters' buffers.  in_ver / in_val: THIS shard's buffers as a
+  // requester (an owner finds its requester s in entry s of the array of shards); ret_delta[s]: what an owner adds to
+  // the place of a row in its own return order to get the row's place in requester s' buffers, where the rows of all
+  // owners stand in owner order.
+  version_t *in_ver;
+  embed_t *in_val;
+  uint32_t *ret_delta;       // [nsrc]
   uint32_t *err;             // the shard's error word
   uint32_t *seg_dev;         // [0..nsrc] first returned row of every requester's segment, device copy
   uint32_t *seg_host;        // the same in memory the host reads; [257] = error flags
 };
 size_t query_tiles(uint32_t q);                       // tile_cnt needs this many words + 1
 uint32_t owner_push_rows_per_block(uint32_t width);   // rows of the longest source one block of the push kernel takes
-// shards_dev: the array in device memory; shards_host: the same values on the host (launch geometry)
+// shards_dev: the array in device memory; shards_host: the same values on the host (launch geometry).  nshards == nsrc:
+// every shard of the group is in the array, in rank order (an owner looks its requesters up there).
 void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerShard *shards_host, int nshards, int nsrc);
-// return exchange on the loopback: descs[2 * (s * nrank + d)] (versions) and the one after it (rows) for requester s
-// and owner d, from the owners' segment tables on the device; the pointer arrays (nrank entries each) must be
-// readable by the device
-struct CopyDesc;
-void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, const version_t *const *ret_ver,
-                               const embed_t *const *ret_val, version_t *const *in_ver, embed_t *const *in_val,
-                               int nrank, uint32_t width, CopyDesc *descs);
 // requester: refresh cached rows that came back, then gather every key's row into dst
 struct PullArgs {
   const uint32_t *got;       // [U] or nullptr: nothing came back (nrank == 1)

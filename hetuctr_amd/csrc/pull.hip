@@ -205,26 +205,59 @@ __global__ __launch_bounds__(kBlock) void scan_positions(const OwnerShard *__res
   if (last_block && threadIdx.x == 0) S.seg_host[257] = *S.err;
 }
 
-// kPackAhead rows to return per group of LPR lanes; which rows, scan_positions has listed
+// Where the rows an owner returns stand in the requesters' buffers: a requester's rows arrive in owner order
+// (csrc/core/all2all.cu:89-130), and how many rows an owner returns to a requester is only known on the device.
+// Thread (owner d, requester s): ret_delta of d for s = rows the owners before d return to s, minus the start of s'
+// segment in d's own return order.
+__global__ void place_returns(const OwnerShard *__restrict__ shards, int nrank) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (uint32_t)nrank * nrank) return;
+  const int d = i / nrank, s = i % nrank;
+  uint32_t before = 0;
+  for (int e = 0; e < d; e++) before += shards[e].seg_dev[s + 1] - shards[e].seg_dev[s];
+  shards[d].ret_delta[s] = before - shards[d].seg_dev[s];
+}
+
+// kPackAhead rows to return per group of LPR lanes; which rows, scan_positions has listed.  A row goes straight into
+// the buffers of the shard that asked for it (in one process a plain device address, between GPUs peer memory).
 constexpr int kPackAhead = 2;
 template <int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict__ shards, int nseg) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
+  __shared__ uint32_t sseg[258], sdelta[257];
   const OwnerShard &S = shards[blockIdx.y];
-  const uint32_t total = S.seg_dev[nseg]; // rows this shard returns
+  for (int i = threadIdx.x; i <= nseg; i += kBlock) sseg[i] = S.seg_dev[i];
+  for (int i = threadIdx.x; i < nseg; i += kBlock) sdelta[i] = S.ret_delta[i];
+  __syncthreads();
+  const uint32_t total = sseg[nseg]; // rows this shard returns
   const uint32_t k0 = blockIdx.x * (kGroups * kPackAhead) + threadIdx.x / LPR;
   if (k0 >= total) return;
   const embed_t *__restrict__ emb = S.t.emb;
-  embed_t *__restrict__ ret_val = S.ret_val;
   const uint32_t gl = threadIdx.x % LPR, W = S.t.width;
   slot_t o[kPackAhead];
 #pragma unroll
   for (int a = 0; a < kPackAhead; a++) o[a] = k0 + a * kGroups < total ? S.ret_slot[k0 + a * kGroups] : kNoSlot;
+  // the requester of every row: the segment of the return order it lies in (segments may be empty)
+  embed_t *dst_val[kPackAhead];
+  version_t *dst_ver[kPackAhead];
+#pragma unroll
+  for (int a = 0; a < kPackAhead; a++) {
+    const uint32_t k = min(k0 + a * kGroups, total - 1);
+    uint32_t lo = 0, hi = nseg - 1;
+    while (lo < hi) { // the first segment that ends behind k
+      const uint32_t mid = (lo + hi) / 2;
+      if (sseg[mid + 1] <= k) lo = mid + 1;
+      else hi = mid;
+    }
+    const uint32_t row = k + sdelta[lo];
+    dst_val[a] = shards[lo].in_val + (size_t)row * W;
+    dst_ver[a] = shards[lo].in_ver + row;
+  }
   if (gl == 0) {
 #pragma unroll
     for (int a = 0; a < kPackAhead; a++)
-      if (o[a] != kNoSlot) S.ret_ver[k0 + a * kGroups] = S.t.ver[o[a]];
+      if (o[a] != kNoSlot) *dst_ver[a] = S.t.ver[o[a]];
   }
   for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
     V v[kPackAhead];
@@ -233,33 +266,8 @@ __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict
       if (o[a] != kNoSlot) v[a] = *(const V *)(emb + (size_t)o[a] * W + col);
 #pragma unroll
     for (int a = 0; a < kPackAhead; a++)
-      if (o[a] != kNoSlot) *(V *)(ret_val + (size_t)(k0 + a * kGroups) * W + col) = v[a];
+      if (o[a] != kNoSlot) *(V *)(dst_val[a] + col) = v[a];
   }
-}
-
-// The copies of the return exchange (csrc/core/all2all.cu:89-130) described on the device: how many rows an owner
-// returns to a requester is only known there.  Thread (requester s, owner d) writes the two descriptors (versions,
-// rows) of that pair; the rows of requester s arrive in owner order.
-struct ReturnPeers {
-  const uint32_t *const *ret_seg;   // [nrank] per owner: first returned row of every requester's segment, [nrank] = total
-  const version_t *const *ret_ver;  // [nrank] per owner
-  const embed_t *const *ret_val;    // [nrank] per owner
-  version_t *const *in_ver;         // [nrank] per requester
-  embed_t *const *in_val;           // [nrank] per requester
-};
-__global__ void build_return_descs(ReturnPeers p, int nrank, uint32_t width, CopyDesc *__restrict__ descs) {
-  const int s = blockIdx.x, d = threadIdx.x;
-  if (d >= nrank) return;
-  uint32_t before = 0;
-  for (int e = 0; e < d; e++) before += p.ret_seg[e][s + 1] - p.ret_seg[e][s];
-  const uint32_t lo = p.ret_seg[d][s], n = p.ret_seg[d][s + 1] - lo;
-  CopyDesc *o = descs + 2 * ((size_t)s * nrank + d);
-  o[0].src = p.ret_ver[d] + lo;
-  o[0].dst = p.in_ver[s] + before;
-  o[0].bytes = (size_t)n * sizeof(version_t);
-  o[1].src = p.ret_val[d] + (size_t)lo * width;
-  o[1].dst = p.in_val[s] + (size_t)before * width;
-  o[1].bytes = (size_t)n * width * sizeof(embed_t);
 }
 
 // What comes back per unique key of the step, in two launches over tiles of kRTile keys:
@@ -545,19 +553,12 @@ void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerS
   hipLaunchKernelGGL(decide_count, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev);
   hipLaunchKernelGGL(scan_positions, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
   if (q_max) {
+    hipLaunchKernelGGL(place_returns, dim3(div_up((uint32_t)(nsrc * nsrc), kBlock)), dim3(kBlock), 0, s, shards_dev, nsrc);
 #define CALL(V, L) \
   hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q_max, kPackAhead * (kBlock / L)), nshards), dim3(kBlock), 0, s, shards_dev, nsrc)
     HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   }
-  HCTR_HIP(hipGetLastError());
-}
-
-void launch_build_return_descs(hipStream_t s, const uint32_t *const *ret_seg, const version_t *const *ret_ver,
-                               const embed_t *const *ret_val, version_t *const *in_ver, embed_t *const *in_val,
-                               int nrank, uint32_t width, CopyDesc *descs) {
-  ReturnPeers p{ret_seg, ret_ver, ret_val, in_ver, in_val};
-  hipLaunchKernelGGL(build_return_descs, dim3(nrank), dim3(std::max(64, (nrank + 63) / 64 * 64)), 0, s, p, nrank, width, descs);
   HCTR_HIP(hipGetLastError());
 }
 

@@ -161,7 +161,7 @@ class Shard {
   const float *push_grad_ = nullptr; // arguments of the push between begin_push and generate_gradient
   uint32_t push_bag_ = 1;
   // receive side (owner role)
-  DeviceBuf rq_idx, rq_ver, outdated, ret_slot, q_slot, src_row, ret_ver, ret_val, ret_seg_dev;
+  DeviceBuf rq_idx, rq_ver, outdated, ret_slot, q_slot, src_row, ret_seg_dev;
   std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
   uint64_t rg_base = 0;      // first row of this shard's piece of the group's receive area for pushed rows
   DeviceBuf push_pos;        // place of every unique key's pushed row in that area (plan position + distance)
@@ -209,7 +209,7 @@ class Group {
   void flush_index();                    // waits for a pending index and takes its results over
   // owner-side arguments of every shard: pinned staging and the device copy the kernels read
   OwnerShard *owner_host = nullptr;
-  DeviceBuf owner_dev;
+  DeviceBuf owner_dev, ret_delta_dev;    // ret_delta_dev: nrank words per owner, see OwnerShard::ret_delta
   void owner_side();
   // Where every shard's pushed rows go: one receive area for the whole group (ids, counts, rows), cut into one piece
   // per owner and, inside it, per source; sized from the plans before any push kernel runs.  Every sender gets, per
@@ -221,7 +221,6 @@ class Group {
   std::vector<Shard *> members;
   DeviceBuf desc_dev[2];                 // copy descriptors of the query exchange [0] and of the return exchange [1]
   CopyDesc *desc_host[2] = {nullptr, nullptr};
-  void **peer_tab = nullptr;             // pinned: per-shard buffer addresses the return exchange reads on the device
   CopyDesc *reserve_descs(size_t n, int which);
   size_t desc_cap[2] = {0, 0};
   double wait_seconds = 120.0;

@@ -458,8 +458,11 @@ void Shard::fill_owner_args(OwnerShard &o) {
   outdated.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
   ret_slot.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
   q_slot.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(slot_t));
-  ret_ver.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(version_t));
-  ret_val.reserve((size_t)std::max<uint32_t>(Q, 1) * cfg.width * sizeof(embed_t));
+  // requester role: what comes back lands here (a row per unique key at most), written by the owners
+  const size_t rows_ub = std::max<uint32_t>(cur.U, 1);
+  got.reserve(rows_ub * 4);
+  in_ver.reserve(rows_ub * sizeof(version_t));
+  in_val.reserve(rows_ub * cfg.width * sizeof(embed_t));
   query_sums.reserve((query_tiles(Q) + 2) * 4);
   last_stats[5] = (long long)rg_seg[R];
   o.t = tv;
@@ -482,8 +485,9 @@ void Shard::fill_owner_args(OwnerShard &o) {
   o.tile_cnt = query_sums.as<uint32_t>();
   o.ret_slot = ret_slot.as<slot_t>();
   o.q_slot = q_slot.as<slot_t>();
-  o.ret_ver = ret_ver.as<version_t>();
-  o.ret_val = ret_val.as<embed_t>();
+  o.in_ver = in_ver.as<version_t>();
+  o.in_val = in_val.as<embed_t>();
+  o.ret_delta = group->ret_delta_dev.as<uint32_t>() + (size_t)cfg.rank * R;
   o.err = err_ptr();
   o.seg_dev = ret_seg_dev.as<uint32_t>();
   o.seg_host = mirror->ret_seg;
@@ -678,7 +682,6 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
 Group::~Group() {
   for (CopyDesc *d : desc_host)
     if (d) (void)hipHostFree(d);
-  if (peer_tab) (void)hipHostFree(peer_tab);
   if (ev0) (void)hipEventDestroy(ev0);
   if (ev1) (void)hipEventDestroy(ev1);
   for (auto &m : marks) { (void)hipEventDestroy(m.a); (void)hipEventDestroy(m.b); }
@@ -753,6 +756,7 @@ void Group::owner_side() {
   if (!owner_host) {
     HCTR_HIP(hipHostMalloc((void **)&owner_host, (size_t)nrank * sizeof(OwnerShard), hipHostMallocDefault));
     owner_dev.reserve((size_t)nrank * sizeof(OwnerShard));
+    ret_delta_dev.reserve((size_t)nrank * nrank * sizeof(uint32_t));
   }
   for (Shard *m : members) m->fill_owner_args(owner_host[m->cfg.rank]);
   StageScope st(*this, S_OWNER);
@@ -878,51 +882,31 @@ void Group::exchange_query() {
 }
 
 // csrc/core/all2all.cu:89-130: flags go back to the requesters, then versions and rows of the flagged queries.
-// How many queries a requester sent to an owner is known on the host; how many of them come back with a row is only
-// known on the device, so the descriptors of those copies are written there (no wait in the middle of the step) and
-// the requester's buffers are sized for the most that can come back (every query it sent).
+// The versions and rows are in place already: the owners wrote them into the requesters' buffers (pack_rows).  What is
+// left are the flags, one per query, whose numbers the host knows.
 void Group::exchange_return() {
   const int R = nrank;
   std::vector<CopyDesc> descs;
-  size_t max_bytes = 0;
-  if (!peer_tab) HCTR_HIP(hipHostMalloc((void **)&peer_tab, 5 * 256 * sizeof(void *), hipHostMallocDefault));
-  const uint32_t **tab_seg = (const uint32_t **)peer_tab;
-  const version_t **tab_rver = (const version_t **)(peer_tab + 256);
-  const embed_t **tab_rval = (const embed_t **)(peer_tab + 512);
-  version_t **tab_iver = (version_t **)(peer_tab + 768);
-  embed_t **tab_ival = (embed_t **)(peer_tab + 1024);
   for (int s = 0; s < R; s++) { // requester
     Shard &req = *members[s];
-    const size_t W = req.cfg.width;
-    const size_t rows_ub = std::max<uint32_t>(req.cur.U, 1); // a row per unique key at most
-    req.got.reserve(rows_ub * 4);
-    req.in_ver.reserve(rows_ub * sizeof(version_t));
-    req.in_val.reserve(rows_ub * W * sizeof(embed_t));
     uint64_t uoff = 0;
     for (int d = 0; d < R; d++) { // owner, in rank order
       Shard &own = *members[d];
       const uint64_t qn = own.rq_seg[s + 1] - own.rq_seg[s];
       if (qn) descs.push_back({own.outdated.as<uint32_t>() + own.rq_seg[s], req.got.as<uint32_t>() + uoff, qn * 4});
-      max_bytes = std::max(max_bytes, (size_t)qn * W * sizeof(embed_t));
       uoff += qn;
     }
     HCTR_CHECK(uoff == req.cur.U, "internal: returned flags do not cover the unique keys");
-    tab_seg[s] = req.ret_seg_dev.as<uint32_t>();
-    tab_rver[s] = req.ret_ver.as<version_t>();
-    tab_rval[s] = req.ret_val.as<embed_t>();
-    tab_iver[s] = req.in_ver.as<version_t>();
-    tab_ival[s] = req.in_val.as<embed_t>();
   }
   StageScope st(*this, S_EXCHANGE);
-  const size_t n_host = descs.size(), n_dev = 2 * (size_t)R * R;
-  CopyDesc *dev = reserve_descs(n_host + n_dev, 1);
-  if (n_host) {
-    memcpy(desc_host[1], descs.data(), n_host * sizeof(CopyDesc));
-    HCTR_HIP(hipMemcpyAsync(dev, desc_host[1], n_host * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
-  }
-  launch_build_return_descs(stream, tab_seg, tab_rver, tab_rval, tab_iver, tab_ival, R, members[0]->tv.width, dev + n_host);
-  for (size_t lo = 0; lo < n_host + n_dev; lo += 32768)
-    launch_copies(stream, dev + lo, (uint32_t)std::min<size_t>(32768, n_host + n_dev - lo), max_bytes);
+  if (descs.empty()) return;
+  CopyDesc *dev = reserve_descs(descs.size(), 1);
+  memcpy(desc_host[1], descs.data(), descs.size() * sizeof(CopyDesc));
+  HCTR_HIP(hipMemcpyAsync(dev, desc_host[1], descs.size() * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
+  size_t max_bytes = 0;
+  for (const CopyDesc &c : descs) max_bytes = std::max(max_bytes, (size_t)c.bytes);
+  for (size_t lo = 0; lo < descs.size(); lo += 32768)
+    launch_copies(stream, dev + lo, (uint32_t)std::min<size_t>(32768, descs.size() - lo), max_bytes);
 }
 
 // csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
