@@ -188,6 +188,11 @@ struct OwnerShard {
   version_t *in_ver;
   embed_t *in_val;
   uint32_t *ret_delta;       // [nsrc]
+  // The flag of every received query goes straight to its requester as well: got = THIS shard's flags as a requester
+  // (one per unique key, owners in rank order); got_delta[s]: what an owner adds to the place of a query in its receive
+  // buffer to get the place of the flag in requester s' array (known on the host).
+  uint32_t *got;
+  uint32_t got_delta[257];
   uint32_t *err;             // the shard's error word
   uint32_t *seg_dev;         // [0..nsrc] first returned row of every requester's segment, device copy
   uint32_t *seg_host;        // the same in memory the host reads; [257] = error flags

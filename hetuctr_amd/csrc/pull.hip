@@ -142,25 +142,36 @@ __global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__r
 // device memory, where the return exchange reads it, and to the host.
 // pack_rows: version and row of every flagged query packed at its position (:24-40), from the list of their slots
 // that scan_positions leaves.
-__global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restrict__ shards) {
+__global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restrict__ shards, int nseg) {
   const OwnerShard &S = shards[blockIdx.y];
   if (blockIdx.x >= S.query_tiles) return;
   const TableView &t = S.t;
   __shared__ uint32_t wcnt[kBlock / kWave];
+  __shared__ uint32_t sseg[258];
+  for (int i = threadIdx.x; i <= nseg; i += kBlock) sseg[i] = S.rq_seg[i];
+  __syncthreads();
   const uint32_t k = blockIdx.x * kBlock + threadIdx.x;
   uint32_t flag = 0;
   if (k < S.q) {
     const slot_t o = owned_slot(t.slot, (uint64_t)S.rq_idx[k], t.id_max, t.n_cached);
     S.q_slot[k] = o;
+    // the requester: the segment of the receive buffer the query lies in (segments may be empty)
+    uint32_t lo = 0, hi = nseg - 1;
+    while (lo < hi) { // the first segment that ends behind k
+      const uint32_t mid = (lo + hi) / 2;
+      if (sseg[mid + 1] <= k) lo = mid + 1;
+      else hi = mid;
+    }
     if (o == kNoSlot) {
       atomicOr(S.err, 4u);
     } else {
       const version_t local = S.rq_ver[k], global = t.ver[o];
-      const bool from_self = k >= S.rq_seg[t.rank] && k < S.rq_seg[t.rank + 1];
+      const bool from_self = lo == (uint32_t)t.rank;
       const bool out = local == kInvalidVersion || local + t.pull_bound < global;
       flag = (out && !from_self) ? 1u : 0u;
     }
     S.outdated[k] = flag;
+    shards[lo].got[k + S.got_delta[lo]] = flag; // the requester reads it from its own array
   }
   const uint64_t m = __ballot(flag != 0);
   if (lane_id() == 0) wcnt[threadIdx.x / kWave] = __popcll(m);
@@ -550,7 +561,7 @@ void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerS
     HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   }
-  hipLaunchKernelGGL(decide_count, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev);
+  hipLaunchKernelGGL(decide_count, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
   hipLaunchKernelGGL(scan_positions, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
   if (q_max) {
     hipLaunchKernelGGL(place_returns, dim3(div_up((uint32_t)(nsrc * nsrc), kBlock)), dim3(kBlock), 0, s, shards_dev, nsrc);

@@ -255,7 +255,6 @@ class Group {
  private:
   void exchange_shapes();
   void exchange_query();
-  void exchange_return();
   void run_copies(std::vector<CopyDesc> &descs);
   template <typename F> void collective(int rank, int op, F &&run_all);
   std::mutex mu_;

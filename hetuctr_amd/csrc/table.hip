@@ -488,6 +488,14 @@ void Shard::fill_owner_args(OwnerShard &o) {
   o.in_ver = in_ver.as<version_t>();
   o.in_val = in_val.as<embed_t>();
   o.ret_delta = group->ret_delta_dev.as<uint32_t>() + (size_t)cfg.rank * R;
+  o.got = got.as<uint32_t>();
+  // csrc/core/all2all.cu:89-130: the flags of requester s' queries stand in its array in owner order; this owner's
+  // begin behind the queries s sent to the owners before it
+  for (int s = 0; s < R; s++) {
+    uint64_t before = 0;
+    for (int e = 0; e < cfg.rank; e++) before += group->members[s]->cur.send_cnt[e];
+    o.got_delta[s] = (uint32_t)(before - rq_seg[s]);
+  }
   o.err = err_ptr();
   o.seg_dev = ret_seg_dev.as<uint32_t>();
   o.seg_host = mirror->ret_seg;
@@ -881,34 +889,6 @@ void Group::exchange_query() {
   run_copies(descs);
 }
 
-// csrc/core/all2all.cu:89-130: flags go back to the requesters, then versions and rows of the flagged queries.
-// The versions and rows are in place already: the owners wrote them into the requesters' buffers (pack_rows).  What is
-// left are the flags, one per query, whose numbers the host knows.
-void Group::exchange_return() {
-  const int R = nrank;
-  std::vector<CopyDesc> descs;
-  for (int s = 0; s < R; s++) { // requester
-    Shard &req = *members[s];
-    uint64_t uoff = 0;
-    for (int d = 0; d < R; d++) { // owner, in rank order
-      Shard &own = *members[d];
-      const uint64_t qn = own.rq_seg[s + 1] - own.rq_seg[s];
-      if (qn) descs.push_back({own.outdated.as<uint32_t>() + own.rq_seg[s], req.got.as<uint32_t>() + uoff, qn * 4});
-      uoff += qn;
-    }
-    HCTR_CHECK(uoff == req.cur.U, "internal: returned flags do not cover the unique keys");
-  }
-  StageScope st(*this, S_EXCHANGE);
-  if (descs.empty()) return;
-  CopyDesc *dev = reserve_descs(descs.size(), 1);
-  memcpy(desc_host[1], descs.data(), descs.size() * sizeof(CopyDesc));
-  HCTR_HIP(hipMemcpyAsync(dev, desc_host[1], descs.size() * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
-  size_t max_bytes = 0;
-  for (const CopyDesc &c : descs) max_bytes = std::max(max_bytes, (size_t)c.bytes);
-  for (size_t lo = 0; lo < descs.size(); lo += 32768)
-    launch_copies(stream, dev + lo, (uint32_t)std::min<size_t>(32768, descs.size() - lo), max_bytes);
-}
-
 // csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
 // Waits for the stream by polling: the calls are short and a blocking wait adds tens of microseconds of
 // wake-up latency to each of them.
@@ -1151,7 +1131,6 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
     exchange_query();
     owner_side();
     // the reference waits here for the return counts (hetu_gpu_table.cu:33); they stay on the device
-    exchange_return();
   }
   for (Shard *m : members) m->write_back(dsts[m->cfg.rank], bag);
   if (time_calls) HCTR_HIP(hipEventRecord(ev1, stream));
