@@ -158,9 +158,10 @@ void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const B
                  const PushArgs &a);
 
 // ---- query / owner side / pull -------------------------------------------------------------------------
-// id and local version of every unique key of the current batch (n_unique: the host's count of them)
+// id and local version of every unique key of the current batch (n_unique: the host's count of them), written to place
+// (unique rank + delta[owner of the key]) of q_idx / q_ver (delta: nrank words in device memory)
 void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t n_unique,
-                          index_t *q_idx, version_t *q_ver);
+                          const uint32_t *delta, index_t *q_idx, version_t *q_ver);
 // Owner side of a step: applying the received pushes (per target row in source order) and serving the received
 // queries (outdated flags, positions of the rows to return, rows packed, first returned row of every requester).
 // One entry per shard of the group; one set of launches serves them all.
@@ -228,9 +229,6 @@ void launch_init_values(hipStream_t s, embed_t *out, size_t len, int type, float
 void launch_fill_i64(hipStream_t s, version_t *p, size_t n, version_t v);
 void launch_fill_i32(hipStream_t s, int32_t *p, size_t n, int32_t v);
 void launch_build_directory(hipStream_t s, const index_t *store_ids, uint32_t n_stored, slot_t *slot);
-// segmented copies of an exchange: n descriptors {src, dst, bytes}
-struct CopyDesc { const void *src; void *dst; size_t bytes; };
-void launch_copies(hipStream_t s, const CopyDesc *descs_device, uint32_t n, size_t max_bytes);
 void launch_plain_copy(hipStream_t s, const void *src, void *dst, size_t bytes); // bytes % 16 == 0
 // keys_out[r * fields + f] = log[rows[r] * fields + f]; a row number outside [0, n_samples) sets bit 0 of *err
 void launch_sample_rows(hipStream_t s, const index_t *log, uint64_t n_samples, uint32_t fields, const index_t *rows,

@@ -16,15 +16,19 @@ template <> struct RowVec<4> { typedef floatx4 T; };
 template <> struct RowVec<1> { typedef float T; };
 
 // The queries of a step (csrc/core/generate_query.cu:91-106): per unique key its id and the version of the local copy
-// (invalid if the key is not resident here).
+// (invalid if the key is not resident here), written where the key's owner reads its queries: place u + delta[owner]
+// of a receive area all owners share.
 template <typename K>
-__global__ __launch_bounds__(kBlock) void build_queries(TableView t, int id_bits, BatchView c, index_t *__restrict__ q_idx,
+__global__ __launch_bounds__(kBlock) void build_queries(TableView t, int id_bits, BatchView c,
+                                                        const uint32_t *__restrict__ delta, index_t *__restrict__ q_idx,
                                                         version_t *__restrict__ q_ver) {
   const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
   if (u >= *c.d_U) return;
   const slot_t o = c.uoff[u];
-  q_idx[u] = (index_t)(((const K *)c.ukey)[u] & (K)(((uint64_t)1 << id_bits) - 1));
-  q_ver[u] = o != kNoSlot ? t.ver[o] : kInvalidVersion;
+  const K key = ((const K *)c.ukey)[u];
+  const uint32_t pos = u + delta[(uint32_t)(key >> id_bits)];
+  q_idx[pos] = (index_t)(key & (K)(((uint64_t)1 << id_bits) - 1));
+  q_ver[pos] = o != kNoSlot ? t.ver[o] : kInvalidVersion;
 }
 
 // ---- owner side: every kernel below serves ALL shards of a loopback group in one launch (blockIdx.y = shard), the
@@ -474,25 +478,6 @@ __global__ __launch_bounds__(kBlock) void gather_pooled(TableView t, BatchView c
   }
 }
 
-__global__ __launch_bounds__(kBlock) void copy_segments(const CopyDesc *__restrict__ d) {
-  const CopyDesc cd = d[blockIdx.y];
-  const size_t stride = (size_t)gridDim.x * kBlock;
-  const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
-  if ((((uintptr_t)cd.src | (uintptr_t)cd.dst | cd.bytes) & 15) == 0) {
-    const uint4 *s = (const uint4 *)cd.src;
-    uint4 *o = (uint4 *)cd.dst;
-    // past the caches both ways: what an exchange moves is read once more at most, and the table rows the push left
-    // in the caches are what the gather at the end of the step wants to find there
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    for (size_t i = tid; i < cd.bytes / 16; i += stride)
-      __builtin_nontemporal_store(__builtin_nontemporal_load((const u32x4 *)s + i), (u32x4 *)o + i);
-  } else {
-    const uint32_t *s = (const uint32_t *)cd.src;
-    uint32_t *o = (uint32_t *)cd.dst;
-    for (size_t i = tid; i < cd.bytes / 4; i += stride) o[i] = s[i];
-  }
-}
-
 // plain 16-byte-lane copy of known size: the yardstick the HBM byte counters are scaled with
 __global__ __launch_bounds__(kBlock) void plain_copy(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
   const size_t stride = (size_t)gridDim.x * kBlock;
@@ -529,11 +514,11 @@ inline int lanes_for(uint32_t width, int vec) {
 } // namespace
 
 void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t n_unique,
-                          index_t *q_idx, version_t *q_ver) {
+                          const uint32_t *delta, index_t *q_idx, version_t *q_ver) {
   if (!n_unique) return;
   const dim3 grid(div_up(n_unique, kBlock));
-  if (kl.wide) hipLaunchKernelGGL(build_queries<uint64_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, q_idx, q_ver);
-  else hipLaunchKernelGGL(build_queries<uint32_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, q_idx, q_ver);
+  if (kl.wide) hipLaunchKernelGGL(build_queries<uint64_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, delta, q_idx, q_ver);
+  else hipLaunchKernelGGL(build_queries<uint32_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, delta, q_idx, q_ver);
   HCTR_HIP(hipGetLastError());
 }
 
@@ -626,14 +611,6 @@ void launch_gather_pooled(hipStream_t s, const TableView &t, const BatchView &cu
 
 void launch_plain_copy(hipStream_t s, const void *src, void *dst, size_t bytes) {
   hipLaunchKernelGGL(plain_copy, dim3(256 * 16), dim3(kBlock), 0, s, (const uint4 *)src, (uint4 *)dst, bytes / 16);
-  HCTR_HIP(hipGetLastError());
-}
-
-void launch_copies(hipStream_t s, const CopyDesc *descs_device, uint32_t n, size_t max_bytes) {
-  if (!n || !max_bytes) return;
-  const unsigned bx = (unsigned)std::min<size_t>(1024, (max_bytes / 16 + kBlock - 1) / kBlock + 1);
-  for (uint32_t first = 0; first < n; first += 65535u) // the second grid dimension ends at 65535
-    hipLaunchKernelGGL(copy_segments, dim3(bx, std::min(n - first, 65535u)), dim3(kBlock), 0, s, descs_device + first);
   HCTR_HIP(hipGetLastError());
 }
 

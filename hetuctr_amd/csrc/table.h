@@ -132,7 +132,7 @@ class Shard {
   // the push of a step in two halves, so that a group can place every shard's pushed rows before any push kernel runs
   void begin_push(const float *grad, uint32_t bag = 1);  // which batch is pushed (none on an inference step), checks
   void generate_gradient(const uint32_t *delta);         // the push kernel; delta: see Group::place_pushes
-  void generate_query();
+  void generate_query(const uint32_t *delta); // delta: see Group::place_queries
   void fill_owner_args(OwnerShard &o);      // handleGradient + handleQuery: what the group's owner-side launches need
   void finish_handle_query();               // after the step: return counts and error flags from the pinned block
   void write_back(float *dst, uint32_t bag = 1);
@@ -157,13 +157,13 @@ class Shard {
   DevStat *dst_ = nullptr; // == dstat.p
   uint32_t *err_ptr() const { return &dst_->err; }
   // send side
-  DeviceBuf q_idx, q_ver;
   const float *push_grad_ = nullptr; // arguments of the push between begin_push and generate_gradient
   uint32_t push_bag_ = 1;
   // receive side (owner role)
-  DeviceBuf rq_idx, rq_ver, outdated, ret_slot, q_slot, src_row, ret_seg_dev;
+  DeviceBuf outdated, ret_slot, q_slot, src_row, ret_seg_dev;
   std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
   uint64_t rg_base = 0;      // first row of this shard's piece of the group's receive area for pushed rows
+  uint64_t rq_base = 0;      // first query of its piece of the receive area for queries
   DeviceBuf push_pos;        // place of every unique key's pushed row in that area (plan position + distance)
   // requester side of the return
   DeviceBuf got, ret_i, in_ver, in_val;
@@ -217,12 +217,12 @@ class Group {
   void place_pushes();
   DeviceBuf rg_idx_all, rg_cnt_all, rg_val_all, push_delta_dev;
   uint32_t *push_delta_host = nullptr;   // pinned staging of the distances
+  // the same for the queries of a step: one receive area (ids, versions), nrank distances per requester
+  void place_queries();
+  DeviceBuf rq_idx_all, rq_ver_all, query_delta_dev;
+  uint32_t *query_delta_host = nullptr;
   bool time_calls = false;               // bracket the two calls with events (hctr_last_times switches it on)
   std::vector<Shard *> members;
-  DeviceBuf desc_dev[2];                 // copy descriptors of the query exchange [0] and of the return exchange [1]
-  CopyDesc *desc_host[2] = {nullptr, nullptr};
-  CopyDesc *reserve_descs(size_t n, int which);
-  size_t desc_cap[2] = {0, 0};
   double wait_seconds = 120.0;
   void sync_stream();
 
@@ -255,7 +255,6 @@ class Group {
  private:
   void exchange_shapes();
   void exchange_query();
-  void run_copies(std::vector<CopyDesc> &descs);
   template <typename F> void collective(int rank, int op, F &&run_all);
   std::mutex mu_;
   std::condition_variable cv_;

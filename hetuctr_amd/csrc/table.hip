@@ -439,13 +439,13 @@ void Shard::generate_gradient(const uint32_t *delta) {
 }
 
 // csrc/core/generate_query.cu:91-106
-void Shard::generate_query() {
+void Shard::generate_query(const uint32_t *delta) {
   if (cfg.nrank == 1) return; // a shard never finds its own rows outdated (handle_query.cu:47-54)
   hipStream_t s = group->stream;
-  q_idx.reserve((size_t)std::max<uint32_t>(cur.U, 1) * sizeof(index_t));
-  q_ver.reserve((size_t)std::max<uint32_t>(cur.U, 1) * sizeof(version_t));
   StageScope st(*group, S_QUERY);
-  launch_build_queries(s, tv, kl, cur.view(), cur.U, q_idx.as<index_t>(), q_ver.as<version_t>());
+  // every query is written where its owner reads it: the group's receive area (see Group::place_queries)
+  launch_build_queries(s, tv, kl, cur.view(), cur.U, delta, group->rq_idx_all.as<index_t>(),
+                       group->rq_ver_all.as<version_t>());
 }
 
 // What the owner-side kernels need of this shard for the step (csrc/core/handle_query.cu:7-116): the received pushes
@@ -477,8 +477,8 @@ void Shard::fill_owner_args(OwnerShard &o) {
   for (int i = 1; i < R; i++)
     if (rg_seg[i + 1] - rg_seg[i] > rg_seg[o.longest + 1] - rg_seg[o.longest]) o.longest = i;
   o.push_blocks = div_up(rg_seg[o.longest + 1] - rg_seg[o.longest], owner_push_rows_per_block(tv.width));
-  o.rq_idx = rq_idx.as<index_t>();
-  o.rq_ver = rq_ver.as<version_t>();
+  o.rq_idx = group->rq_idx_all.as<index_t>() + rq_base;
+  o.rq_ver = group->rq_ver_all.as<version_t>() + rq_base;
   o.q = Q;
   o.query_tiles = (uint32_t)query_tiles(Q); // one tile even without queries: the segment table is written
   o.outdated = outdated.as<uint32_t>();
@@ -688,8 +688,6 @@ Group::Group(int nr, int dev, std::string k) : nrank(nr), device_id(dev), key(st
 }
 
 Group::~Group() {
-  for (CopyDesc *d : desc_host)
-    if (d) (void)hipHostFree(d);
   if (ev0) (void)hipEventDestroy(ev0);
   if (ev1) (void)hipEventDestroy(ev1);
   for (auto &m : marks) { (void)hipEventDestroy(m.a); (void)hipEventDestroy(m.b); }
@@ -703,6 +701,7 @@ Group::~Group() {
   if (ev_plan) (void)hipEventDestroy(ev_plan);
   if (owner_host) (void)hipHostFree(owner_host);
   if (push_delta_host) (void)hipHostFree(push_delta_host);
+  if (query_delta_host) (void)hipHostFree(query_delta_host);
 }
 
 void Group::join(Shard *s) {
@@ -788,34 +787,6 @@ void Group::set_stage_timing(bool on) {
   }
 }
 
-// Descriptors travel host -> pinned staging -> device with an asynchronous copy.  The two exchanges of a step have a
-// staging area and a device array each: nothing waits between them any more, so the second must not overwrite what the
-// first one's copy has not read yet.  A step ends with a wait, which is what makes reuse in the next step safe.
-CopyDesc *Group::reserve_descs(size_t n, int which) {
-  if (n > desc_cap[which]) {
-    HCTR_HIP(hipStreamSynchronize(stream)); // the old arrays may still be read by a copy or a launch in flight
-    if (desc_host[which]) HCTR_HIP(hipHostFree(desc_host[which]));
-    desc_host[which] = nullptr;
-    desc_cap[which] = n * 2;
-    HCTR_HIP(hipHostMalloc((void **)&desc_host[which], desc_cap[which] * sizeof(CopyDesc), hipHostMallocDefault));
-  }
-  desc_dev[which].reserve(desc_cap[which] * sizeof(CopyDesc));
-  return desc_dev[which].as<CopyDesc>();
-}
-
-void Group::run_copies(std::vector<CopyDesc> &descs) {
-  if (descs.empty()) return;
-  StageScope st(*this, S_EXCHANGE);
-  CopyDesc *dev = reserve_descs(descs.size(), 0);
-  memcpy(desc_host[0], descs.data(), descs.size() * sizeof(CopyDesc));
-  HCTR_HIP(hipMemcpyAsync(dev, desc_host[0], descs.size() * sizeof(CopyDesc), hipMemcpyHostToDevice, stream));
-  size_t max_bytes = 0;
-  for (auto &d : descs) max_bytes = std::max(max_bytes, d.bytes);
-  for (size_t lo = 0; lo < descs.size(); lo += 32768)
-    launch_copies(stream, dev + lo, (uint32_t)std::min<size_t>(32768, descs.size() - lo), max_bytes);
-  descs.clear();
-}
-
 // The pushes of a step never pass through a send buffer: a pushed row is written by the push kernel into the receive
 // area of its owner (csrc/core/all2all.cu:48-87 moves it there in the reference).  How many rows every shard pushes to
 // every owner is known from the plans before any push kernel starts, so the area is sized and cut here: one piece per
@@ -859,34 +830,43 @@ void Group::place_pushes() {
   HCTR_HIP(hipMemcpyAsync(push_delta_dev.p, push_delta_host, (size_t)R * R * sizeof(uint32_t), hipMemcpyHostToDevice, stream));
 }
 
-// csrc/core/all2all.cu:18-46: every receive buffer is the senders' buckets for this shard, in source order (the
-// queries; the pushed rows are in place already, see place_pushes)
-void Group::exchange_query() {
+// csrc/core/all2all.cu:18-46: every owner's receive buffer is the requesters' buckets for it, in source order.  The
+// queries do not pass through a send buffer either: how many unique keys every shard asks every owner for is known on the
+// host once the index is done, so the group's receive area is cut (one piece per owner, inside it one per source) and
+// every shard's query kernel writes into it; a unique key of rank u lands u + (distance for its owner) into the area.
+void Group::place_queries() {
   const int R = nrank;
-  std::vector<CopyDesc> descs;
+  if (R == 1) return;
+  if (!query_delta_host) {
+    HCTR_HIP(hipHostMalloc((void **)&query_delta_host, (size_t)R * R * sizeof(uint32_t), hipHostMallocDefault));
+    query_delta_dev.reserve((size_t)R * R * sizeof(uint32_t));
+  }
+  uint64_t total = 0;
   for (int d = 0; d < R; d++) {
     Shard &dst = *members[d];
+    dst.rq_base = total;
     uint64_t Q = 0;
     for (int s = 0; s < R; s++) {
       dst.rq_seg[s] = Q;
       Q += members[s]->cur.send_cnt[d];
     }
     dst.rq_seg[R] = Q;
-    HCTR_CHECK(Q < 0xfffffff0ull, "more than 2^32 queries arrive at one shard");
-    dst.rq_idx.reserve(std::max<uint64_t>(Q, 1) * sizeof(index_t));
-    dst.rq_ver.reserve(std::max<uint64_t>(Q, 1) * sizeof(version_t));
-    for (int s = 0; s < R; s++) {
-      Shard &src = *members[s];
-      uint64_t qlo = 0;
-      for (int i = 0; i < d; i++) qlo += src.cur.send_cnt[i];
-      const uint64_t qn = src.cur.send_cnt[d];
-      if (qn) {
-        descs.push_back({src.q_idx.as<index_t>() + qlo, dst.rq_idx.as<index_t>() + dst.rq_seg[s], qn * sizeof(index_t)});
-        descs.push_back({src.q_ver.as<version_t>() + qlo, dst.rq_ver.as<version_t>() + dst.rq_seg[s], qn * sizeof(version_t)});
-      }
-    }
+    total += Q;
   }
-  run_copies(descs);
+  HCTR_CHECK(total < 0xfffffff0ull, "more than 2^32 queries in one step");
+  rq_idx_all.reserve(std::max<uint64_t>(total, 1) * sizeof(index_t));
+  rq_ver_all.reserve(std::max<uint64_t>(total, 1) * sizeof(version_t));
+  if (!total) return;
+  for (int s = 0; s < R; s++) {
+    uint64_t ulo = 0; // unique keys of this shard that belong to the owners before d
+    for (int d = 0; d < R; d++) {
+      const Shard &dst = *members[d];
+      query_delta_host[(size_t)s * R + d] = (uint32_t)(dst.rq_base + dst.rq_seg[s] - ulo);
+      ulo += members[s]->cur.send_cnt[d];
+    }
+    HCTR_CHECK(ulo == members[s]->cur.U, "internal: the queries per owner do not add up to the unique keys");
+  }
+  HCTR_HIP(hipMemcpyAsync(query_delta_dev.p, query_delta_host, (size_t)R * R * sizeof(uint32_t), hipMemcpyHostToDevice, stream));
 }
 
 // csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
@@ -1119,7 +1099,8 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
       exchange_shapes();
     }
   }
-  for (Shard *m : members) m->generate_query();
+  place_queries();
+  for (Shard *m : members) m->generate_query(nrank > 1 ? query_delta_dev.as<uint32_t>() + (size_t)nrank * m->cfg.rank : nullptr);
   const bool join_index = index_pending;
   if (join_index) {
     // the push kernel is in the main stream's queue; the gather below also needs the index of the current batch,
@@ -1128,7 +1109,6 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
     HCTR_HIP(hipStreamWaitEvent(stream, ev_index, 0));
   }
   if (nrank > 1) {
-    exchange_query();
     owner_side();
     // the reference waits here for the return counts (hetu_gpu_table.cu:33); they stay on the device
   }
