@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict
       if (o[a] != kNoSlot) v[a] = *(const V *)(emb + (size_t)o[a] * W + col);
 #pragma unroll
     for (int a = 0; a < kPackAhead; a++)
-      if (o[a] != kNoSlot) *(V *)(dst_val[a] + col) = v[a];
+      if (o[a] != kNoSlot) __builtin_nontemporal_store(v[a], (V *)(dst_val[a] + col)); // read next by another shard's kernels
   }
 }
 

@@ -103,12 +103,19 @@ template <> struct Vec<4> {
   static __device__ __forceinline__ T zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
   static __device__ __forceinline__ void add(T &a, const T &b) { a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w; }
   static __device__ __forceinline__ T scale(const T &a, float s) { return make_float4(a.x * s, a.y * s, a.z * s, a.w * s); }
+  // a store past the caches: for rows another shard's kernel reads next
+  static __device__ __forceinline__ void store_away(T *p, const T &a) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    f4 v = {a.x, a.y, a.z, a.w};
+    __builtin_nontemporal_store(v, (f4 *)p);
+  }
 };
 template <> struct Vec<1> {
   typedef float T;
   static __device__ __forceinline__ T zero() { return 0.f; }
   static __device__ __forceinline__ void add(T &a, const T &b) { a += b; }
   static __device__ __forceinline__ T scale(const T &a, float s) { return a * s; }
+  static __device__ __forceinline__ void store_away(T *p, const T &a) { __builtin_nontemporal_store(a, p); }
 };
 
 // The version / update counters of unique rank u and its entry among the pushed rows (gradient_index_kernel,
@@ -157,14 +164,14 @@ __device__ __forceinline__ void apply_row(const TableView &t, int id_bits, const
     Vec<VEC>::add(cur, s);
     *e = cur;
   } else {
-    *(V *)(a.g_val + (size_t)q * W + col) = s;
+    Vec<VEC>::store_away((V *)(a.g_val + (size_t)q * W + col), s);
   }
   if (type >= 2) {
     V *g = (V *)(t.pend + (size_t)o * W + col);
     V pg = *g;
     Vec<VEC>::add(pg, s);
     if (type == 2) {
-      *(V *)(a.g_val + (size_t)q * W + col) = pg;
+      Vec<VEC>::store_away((V *)(a.g_val + (size_t)q * W + col), pg);
       pg = Vec<VEC>::zero();
     }
     *g = pg;
@@ -290,13 +297,13 @@ __device__ __forceinline__ void short_role(const TableView &t, int id_bits, cons
           Vec<VEC>::add(r, scaled);
           *(V *)(t.emb + (size_t)off[i] * W + col) = r;
         } else {
-          *(V *)(a.g_val + (size_t)q[i] * W + col) = scaled;
+          Vec<VEC>::store_away((V *)(a.g_val + (size_t)q[i] * W + col), scaled);
         }
         if (type[i] >= 2) {
           V g = pg[i];
           Vec<VEC>::add(g, scaled);
           if (type[i] == 2) {
-            *(V *)(a.g_val + (size_t)q[i] * W + col) = g;
+            Vec<VEC>::store_away((V *)(a.g_val + (size_t)q[i] * W + col), g);
             g = Vec<VEC>::zero();
           }
           *(V *)(t.pend + (size_t)off[i] * W + col) = g;
