@@ -160,12 +160,13 @@ def partitioned_layout(ks, nrank, cache_frac, log_samples, batch_samples, rounds
 
 def sharded_extra_bytes(width, touched_cached, pushed, received, queried, returned, refreshed):
     """Bytes a step moves on top of algorithmic_bytes when rows are sharded and cached (same accounting): the
-    pending-gradient store and update counter of touched cached rows, the push buffer and its loopback copy,
-    applying received gradient rows, the query (id, version, directory slot, flag, both ways), packing and
-    returning rows, refreshing cached rows."""
+    pending-gradient store and update counter of touched cached rows, every pushed row written once (into its owner's
+    receive area: id, count, row), applying received gradient rows, the query (id, version, directory slot, flag, both
+    ways), every returned row read from the owner's table and written once (into the requester's buffer, with its
+    version), refreshing cached rows.  No term for a transport: on one GPU the shards write into each other's buffers."""
     row = 4 * width
-    return (touched_cached * (2 * row + 16) + pushed * (row + 2 * row + 32) + received * (2 * row + 32) +
-            queried * 2 * (8 + 8 + 16 + 8) + returned * (2 * row + 2 * row + 8) + refreshed * (3 * row + 8))
+    return (touched_cached * (2 * row + 16) + pushed * (row + 16) + received * (2 * row + 32) +
+            queried * 2 * (8 + 8 + 16 + 8) + returned * (2 * row + 8) + refreshed * (3 * row + 8))
 
 
 def algorithmic_bytes(n_keys, n_unique, width, bag=1):
