@@ -235,7 +235,10 @@ __global__ void place_returns(const OwnerShard *__restrict__ shards, int nrank) 
 
 // kPackAhead rows to return per group of LPR lanes; which rows, scan_positions has listed.  A row goes straight into
 // the buffers of the shard that asked for it (in one process a plain device address, between GPUs peer memory).
-constexpr int kPackAhead = 2;
+#ifndef HCTR_PACK_AHEAD
+#define HCTR_PACK_AHEAD 2
+#endif
+constexpr int kPackAhead = HCTR_PACK_AHEAD;
 template <int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict__ shards, int nseg) {
   typedef typename RowVec<VEC>::T V;
