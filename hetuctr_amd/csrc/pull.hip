@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__r
 // decide_count: the outdated flag of every query (pull rule, self-exempt, :47-54) and the number of flags per tile.
 // scan_positions: a tile's flags scanned behind the tiles before it -> position of every flagged query among the
 // returned rows (:56-57, :74-75), and the first returned row of every requester's segment (:59-61) written both to
-// device memory, where the return exchange reads it, and to the host.
+// device memory, where place_returns reads it, and to the host.
 // pack_rows: version and row of every flagged query packed at its position (:24-40), from the list of their slots
 // that scan_positions leaves.
 __global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restrict__ shards, int nseg) {

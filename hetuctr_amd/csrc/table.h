@@ -254,7 +254,6 @@ class Group {
 
  private:
   void exchange_shapes();
-  void exchange_query();
   template <typename F> void collective(int rank, int op, F &&run_all);
   std::mutex mu_;
   std::condition_variable cv_;

@@ -1,5 +1,5 @@
 // Host orchestration of the hot path: shard construction, the fixed stage order of preprocess and push_pull,
-// the loopback exchanges between the shards of a group, introspection.
+// the placement of what the shards of a loopback group hand to each other, introspection.
 // Reference: csrc/core/hetu_gpu_table.cu:9-65 (stage order), csrc/core/table_initialize.cu:66-211 (state),
 // csrc/core/all2all.cu:6-130 (what travels between which buffers, in which order).
 #include "table.h"
@@ -450,7 +450,7 @@ void Shard::generate_query(const uint32_t *delta) {
 
 // What the owner-side kernels need of this shard for the step (csrc/core/handle_query.cu:7-116): the received pushes
 // and queries, the buffers of the rows that go back.  The number of rows that go back to every requester stays on the
-// device, where the return exchange reads it; the host copy (statistics, error flags) is written by the same kernel
+// device, where the owners' kernels read it; the host copy (statistics, error flags) is written by the same kernel
 // into pinned memory and read when the step is over.
 void Shard::fill_owner_args(OwnerShard &o) {
   const int R = cfg.nrank;
@@ -1084,7 +1084,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
     {
       // the push plans of the current batches, for the step in which they are the previous ones: after the pushes of
       // this step (they move the update counters the plan reads), beside everything else the step still does; queued
-      // before the host looks at the index, so that nothing but the queries stands between that look and the exchange
+      // before the host looks at the index, so that nothing but the queries stands between that look and the owner side
       StreamSwitch on(*this, index_stream);
       HCTR_HIP(hipStreamWaitEvent(stream, ev_pushed, 0));
       for (Shard *m : members) m->plan_batch(m->cur);
@@ -1092,7 +1092,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
     }
     if (wait_index) {
       // the queries are built from the index of the current batches, which the host needs too (unique keys and queries
-      // per owner size the exchange)
+      // per owner place the queries)
       index_pending = false;
       HCTR_HIP(hipEventSynchronize(ev_index));
       for (Shard *m : members) m->finish_index();
