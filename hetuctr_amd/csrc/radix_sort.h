@@ -12,8 +12,10 @@ constexpr int kSortBlock = HCTR_SORT_BLOCK;     // threads per block
 constexpr int kSortMaxDigitBits = 10;           // up to 1024 bins
 constexpr int kSortMaxBins = 1 << kSortMaxDigitBits;
 // Keys per thread, hence keys per tile (one block sorts one tile per pass), chosen by the size of the input: a small
-// input is cut into small tiles so that enough blocks share it (its passes are latency, not traffic); a huge one into
-// large tiles, because every tile costs a row of digit counts that is written, scanned and read again in every pass.
+// input is cut into small tiles so that enough blocks share it (its passes are latency, not traffic); a large one into
+// large tiles, because every tile costs a row of digit counts that is written, scanned and read again in every pass,
+// and because fewer, longer-lived blocks take less from a kernel that runs beside the sort on another stream (at
+// 1.7 M keys the sort alone is 4 us slower with 8192-key tiles than with 4096-key ones, the step beside it 5 us faster).
 #ifndef HCTR_SORT_ITEMS_DEFAULT
 #define HCTR_SORT_ITEMS_DEFAULT 8
 #endif
@@ -24,8 +26,9 @@ constexpr int kSortMaxBins = 1 << kSortMaxDigitBits;
 #define HCTR_SORT_ITEMS_SMALL 2
 #endif
 constexpr int kSortItemsSmall = HCTR_SORT_ITEMS_SMALL, kSortItemsDefault = HCTR_SORT_ITEMS_DEFAULT, kSortItemsLarge = HCTR_SORT_ITEMS_LARGE;
+constexpr size_t kSortSmallUpTo = (size_t)1 << 17, kSortLargeFrom = (size_t)1 << 20;
 inline int sort_items(size_t n) {
-  return n <= ((size_t)1 << 17) ? kSortItemsSmall : (n >= ((size_t)1 << 23) ? kSortItemsLarge : kSortItemsDefault);
+  return n <= kSortSmallUpTo ? kSortItemsSmall : (n >= kSortLargeFrom ? kSortItemsLarge : kSortItemsDefault);
 }
 inline size_t sort_tile(size_t n) { return (size_t)kSortBlock * sort_items(n); }
 inline size_t sort_tiles(size_t n) { return (n + sort_tile(n) - 1) / sort_tile(n); }
@@ -35,8 +38,8 @@ inline size_t sort_scratch_words(size_t n) { return (sort_tiles(n) + 1) * (size_
 // the most words any input of up to n_max keys needs
 inline size_t sort_scratch_words_upto(size_t n_max) {
   size_t w = sort_scratch_words(n_max);
-  if (n_max > ((size_t)1 << 17)) w = w > sort_scratch_words((size_t)1 << 17) ? w : sort_scratch_words((size_t)1 << 17);
-  if (n_max > ((size_t)1 << 23) - 1) w = w > sort_scratch_words(((size_t)1 << 23) - 1) ? w : sort_scratch_words(((size_t)1 << 23) - 1);
+  if (n_max > kSortSmallUpTo) w = w > sort_scratch_words(kSortSmallUpTo) ? w : sort_scratch_words(kSortSmallUpTo);
+  if (n_max > kSortLargeFrom - 1) w = w > sort_scratch_words(kSortLargeFrom - 1) ? w : sort_scratch_words(kSortLargeFrom - 1);
   return w;
 }
 // expands CALL(ITEMS) for the tile shape of an input of n keys
