@@ -61,7 +61,10 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
 
 // The unique pass works on tiles of kUTile sorted positions; position j of a tile is handled by thread (j % kUBlock)
 // in round (j / kUBlock): every load and store below is coalesced across the wave.
-constexpr int kUBlock = 512, kUItems = 8, kUTile = kUBlock * kUItems;
+#ifndef HCTR_UNIQUE_ITEMS
+#define HCTR_UNIQUE_ITEMS 8
+#endif
+constexpr int kUBlock = 512, kUItems = HCTR_UNIQUE_ITEMS, kUTile = kUBlock * kUItems;
 inline unsigned unique_tiles(uint32_t n) { return div_up(n, kUTile); }
 
 // the key before sorted position j of this lane: the neighbouring lane holds it, except for lane 0
