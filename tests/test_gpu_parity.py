@@ -311,6 +311,32 @@ def test_batch_sizes_where_the_sort_changes_shape(nrank):
     p.close()
 
 
+def test_large_batches_of_ids_in_pageable_host_memory():
+    # ids handed over as numpy arrays (the reference's drivers do), megabytes at a time: sizes around powers of two and
+    # odd ones, the same array object reused and overwritten right after the call
+    say("large host batches")
+    rng = np.random.default_rng(36)
+    length, width = 500_000, 4
+    p = single(length, width, init=("Zero", 0.0, 0.0), lr=0.5)
+    buf = np.zeros(400_003, np.int64)
+    for step, n in enumerate([262_143, 262_144, 262_145, 400_003, 131_072 * 3 + 1, 300_000, 5]):
+        want = rng.integers(0, length, size=n).astype(np.int64)
+        buf[:n] = want
+        p.tables[0].preprocess(buf.ctypes.data, n)
+        buf[:n] = -1                                        # overwritten as soon as the call is back
+        p.oracle.preprocess([want])
+        p.n = [n]
+        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.KEYS], "n %d" % n)
+        out, ref = p.push_pull([None])
+        assert_close(out[0], ref[0], 1e-5, "dst n %d" % n)
+    # an id out of range in the middle of a large host batch is reported by the call
+    keys = rng.integers(0, length, size=300_000).astype(np.int64)
+    keys[123_456] = length
+    with pytest.raises(RuntimeError, match="outside"):
+        p.tables[0].preprocess(keys.ctypes.data, keys.shape[0])
+    p.close()
+
+
 def test_key_error_is_raised_by_preprocess_and_the_table_goes_on():
     say("bad key, early return")
     length, width, n = 1000, 8, 500
