@@ -32,9 +32,20 @@ inline int sort_items(size_t n) {
 }
 inline size_t sort_tile(size_t n) { return (size_t)kSortBlock * sort_items(n); }
 inline size_t sort_tiles(size_t n) { return (n + sort_tile(n) - 1) / sort_tile(n); }
-// words of scratch a sort of n keys needs: per tile and bin the count of the digit in the earlier tiles, then the
-// total of every bin.  Not monotonic in n (the tile grows with it): size the scratch for the n that is sorted.
-inline size_t sort_scratch_words(size_t n) { return (sort_tiles(n) + 1) * (size_t)kSortMaxBins; }
+// words of scratch a sort of n keys needs: per tile and bin the count of the digit in the earlier tiles (of its piece of
+// the scan), then the total of every bin (per piece).  Not monotonic in n (the tile grows with it): size the scratch for the n that is sorted.
+// An input of many tiles has its count columns scanned in up to kScanMaxChunks pieces of at least kScanChunkRows rows,
+// one block per piece and group of columns (a column of thousands of rows scanned by one block is a long serial
+// walk); every piece leaves its column totals, which the scatter adds up.
+#ifndef HCTR_SCAN_MAX_CHUNKS
+#define HCTR_SCAN_MAX_CHUNKS 16
+#endif
+constexpr uint32_t kScanMaxChunks = HCTR_SCAN_MAX_CHUNKS, kScanChunkRows = 256;
+inline uint32_t scan_chunks(size_t tiles) {
+  const size_t c = tiles / kScanChunkRows;
+  return c < 2 ? 1u : (c > kScanMaxChunks ? kScanMaxChunks : (uint32_t)c);
+}
+inline size_t sort_scratch_words(size_t n) { return (sort_tiles(n) + scan_chunks(sort_tiles(n))) * (size_t)kSortMaxBins; }
 // the most words any input of up to n_max keys needs
 inline size_t sort_scratch_words_upto(size_t n_max) {
   size_t w = sort_scratch_words(n_max);

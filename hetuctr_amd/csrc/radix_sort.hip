@@ -47,8 +47,8 @@ __global__ __launch_bounds__(kSortBlock) void digit_histogram(const K *__restric
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) counts[(size_t)blockIdx.x * nb + i] = h[i];
 }
 
-// counts[tile][bin] -> in place, the count of the bin in the earlier tiles; bin_total[bin].  A block scans kScanCols
-// neighbouring bins: thread (part, col) adds up its part of the tiles for one bin.  Up to kScanKeep rows per thread
+// counts[tile][bin] -> in place, the count of the bin in the earlier tiles of the block's piece of the rows;
+// bin_total[piece][bin].  A block scans kScanCols neighbouring bins: thread (part, col) adds up its part of the tiles for one bin.  Up to kScanKeep rows per thread
 // stay in registers between the sum and the rewrite (one trip to memory); longer parts are read twice.
 #ifndef HCTR_SCAN_COLS
 #define HCTR_SCAN_COLS 16
@@ -61,8 +61,11 @@ __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ 
                                                          uint32_t *__restrict__ bin_total) {
   __shared__ uint32_t part_sum[kScanParts][kScanCols];
   const uint32_t c = threadIdx.x % kScanCols, col = blockIdx.x * kScanCols + c, part = threadIdx.x / kScanCols;
-  const uint32_t per = (tiles + kScanParts - 1) / kScanParts;
-  const uint32_t lo = min(part * per, tiles), hi = min(lo + per, tiles);
+  // blockIdx.y: the piece of the rows this block scans (one piece: the whole column)
+  const uint32_t rows_per = (tiles + gridDim.y - 1) / gridDim.y;
+  const uint32_t clo = min(blockIdx.y * rows_per, tiles), chi = min(clo + rows_per, tiles);
+  const uint32_t per = (chi - clo + kScanParts - 1) / kScanParts;
+  const uint32_t lo = min(clo + part * per, chi), hi = min(lo + per, chi);
   const bool ok = col < nb;
   uint32_t first[kScanKeep];
 #pragma unroll
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(kScanBlock) void scan_tiles(uint32_t *__restrict__ 
   __syncthreads();
   uint32_t run = 0;
   for (uint32_t q = 0; q < part; q++) run += part_sum[q][c];
-  if (part == kScanParts - 1 && ok) bin_total[col] = run + s;
+  if (part == kScanParts - 1 && ok) bin_total[blockIdx.y * nb + col] = run + s; // the piece's total of the column
 #pragma unroll
   for (int u = 0; u < kScanKeep; u++) {
     if (ok && lo + u < hi) counts[(size_t)(lo + u) * nb + col] = run;
@@ -105,13 +108,15 @@ constexpr uint32_t kSelfScanTiles = HCTR_SELF_SCAN_TILES;
 constexpr int kSelfScanAhead = 32;         // rows of counts requested together
 
 // DBITS: the digit width if known at compile time (the match loop is then straight-line code), else 0
-// kSelfScan: tile_prefix holds the raw counts of digit_histogram, bin_total is not read
-template <typename K, bool kFirst, int ITEMS, int DBITS, bool kSelfScan>
+// kMode 0: tile_prefix / bin_total are the scanned counts and the totals of one piece
+//       1: tile_prefix holds the raw counts of digit_histogram (no scan launch), bin_total is not read
+//       2: the scan ran in `pieces` pieces: tile_prefix counts inside the tile's piece, bin_total[piece][bin] adds up
+template <typename K, bool kFirst, int ITEMS, int DBITS, int kMode>
 __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
                                                       K *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
                                                       uint32_t n, int shift, int dbits, uint32_t tiles,
                                                       const uint32_t *__restrict__ tile_prefix,
-                                                      const uint32_t *__restrict__ bin_total) {
+                                                      const uint32_t *__restrict__ bin_total, uint32_t pieces) {
 #ifndef HCTR_SORT_NO_XCD
   // Workgroups go to the 8 XCDs of the device in turn, and each XCD has an L2 of its own.  XCD x takes the x-th
   // eighth of the tiles: neighbouring tiles write neighbouring pieces of every bin, so the pieces meet in one L2 and
@@ -158,20 +163,25 @@ __global__ __launch_bounds__(kSortBlock) void scatter(const K *__restrict__ keys
   // earlier tiles
   {
     uint32_t all[2] = {0, 0}, mine[2] = {0, 0};
-    if (kSelfScan) {
+    if (kMode != 0) {
+      // a table of rows to add up per bin: all of them for the bin's total, those before `rows_mine` for this tile
+      const uint32_t *rows = kMode == 1 ? tile_prefix : bin_total;
+      const uint32_t n_rows = kMode == 1 ? tiles : pieces;
+      const uint32_t rows_mine = kMode == 1 ? tile : tile / ((tiles + pieces - 1) / pieces);
       for (int q = 0; q < 2; q++) {
         if (blo + q < bhi) {
-          const uint32_t *col = tile_prefix + blo + q;
-          for (uint32_t t0 = 0; t0 < tiles; t0 += kSelfScanAhead) {
+          const uint32_t *col = rows + blo + q;
+          for (uint32_t t0 = 0; t0 < n_rows; t0 += kSelfScanAhead) {
             uint32_t v[kSelfScanAhead];
 #pragma unroll
-            for (int u = 0; u < kSelfScanAhead; u++) v[u] = t0 + u < tiles ? col[(size_t)(t0 + u) * nb] : 0u;
+            for (int u = 0; u < kSelfScanAhead; u++) v[u] = t0 + u < n_rows ? col[(size_t)(t0 + u) * nb] : 0u;
 #pragma unroll
             for (int u = 0; u < kSelfScanAhead; u++) {
               all[q] += v[u];
-              mine[q] += t0 + u < tile ? v[u] : 0u;
+              mine[q] += t0 + u < rows_mine ? v[u] : 0u;
             }
           }
+          if (kMode == 2) mine[q] += tile_prefix[(size_t)tile * nb + blo + q];
         }
       }
     } else {
@@ -302,9 +312,10 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
   const uint32_t tiles = (uint32_t)sort_tiles(n);
   const uint32_t sgrid = (tiles + kXcds - 1) / kXcds * kXcds; // whole rounds over the XCDs
   uint32_t *counts = scratch.words;
-  uint32_t *bin_total = scratch.words + (size_t)tiles * kSortMaxBins;
+  uint32_t *bin_total = scratch.words + (size_t)tiles * kSortMaxBins; // one row per piece of the scan
   const int passes = (bits + kSortMaxDigitBits - 1) / kSortMaxDigitBits;
   const bool self_scan = sort_items(n) == kSortItemsSmall && tiles <= kSelfScanTiles;
+  const uint32_t pieces = sort_items(n) == kSortItemsLarge ? scan_chunks(tiles) : 1u;
   int shift = 0;
   const K *kin = keys_in;
   const uint32_t *vin = nullptr;
@@ -324,16 +335,17 @@ void radix_sort_positions(hipStream_t stream, const K *keys_in, uint32_t n, int 
 #undef CALL
     }
     if (wanted(1) && !self_scan)
-      hipLaunchKernelGGL(scan_tiles, dim3((nb + kScanCols - 1) / kScanCols), dim3(kScanBlock), 0, stream, counts, tiles,
-                         nb, bin_total);
+      hipLaunchKernelGGL(scan_tiles, dim3((nb + kScanCols - 1) / kScanCols, pieces), dim3(kScanBlock), 0, stream, counts,
+                         tiles, nb, bin_total);
     if (wanted(2)) {
 #define CALL4(I, F, D, S)                                                                                     \
   hipLaunchKernelGGL((scatter<K, F, I, D, S>), dim3(sgrid), dim3(kSortBlock), 0, stream, kin, vin, kout, vout, n, \
-                     shift, dbits, tiles, counts, bin_total)
-#define CALL3(I, F, D)                                                      \
-  do {                                                                      \
-    if (self_scan && I == kSortItemsSmall) CALL4(I, F, D, (I == kSortItemsSmall)); \
-    else CALL4(I, F, D, false);                                             \
+                     shift, dbits, tiles, counts, bin_total, pieces)
+#define CALL3(I, F, D)                                                                       \
+  do {                                                                                       \
+    if (self_scan && I == kSortItemsSmall) CALL4(I, F, D, (I == kSortItemsSmall ? 1 : 0));    \
+    else if (pieces > 1 && I == kSortItemsLarge) CALL4(I, F, D, (I == kSortItemsLarge ? 2 : 0)); \
+    else CALL4(I, F, D, 0);                                                                  \
   } while (0)
 #define CALL2(I, F)                   \
   do {                                \
