@@ -337,6 +337,31 @@ def test_large_batches_of_ids_in_pageable_host_memory():
     p.close()
 
 
+@pytest.mark.parametrize("nrank", [1, 3])
+def test_64_bit_sort_keys_at_every_sort_shape(nrank, monkeypatch):
+    # sort keys wider than 32 bits (owner and id of a huge id space) are forced on a small table; batch sizes from
+    # the three tile shapes of the sort, the largest one with its count columns scanned in pieces
+    monkeypatch.setenv("HETUCTR_FORCE_WIDE_KEYS", "1")
+    say("64-bit sort keys, shards", nrank)
+    rng = np.random.default_rng(37 + nrank)
+    length, width = 2_000_000, 2
+    root = rng.integers(0, nrank, size=length).astype(np.uint8)
+    storage = [np.flatnonzero(root == r).astype(np.int64) for r in range(nrank)]
+    p = Pair(nrank, length, width, root, storage, init=("Zero", 0.0, 0.0), lr=0.5)
+    prev_n = [0] * nrank
+    for n in [3000, 70_000, 200_000, 4_300_000, 1_100_000]:
+        ns = [n if r == 0 else max(n // 5, 1) for r in range(nrank)]
+        keys = [rng.integers(0, length, size=k).astype(np.int64) for k in ns]
+        p.preprocess(keys, device_keys=True)
+        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.SIZES], "n %d" % n)
+        out, ref = p.push_pull([rng.integers(-2, 3, size=(k, width)).astype(np.float32) for k in prev_n])
+        for r in range(nrank):
+            assert_close(out[r], ref[r], 1e-5, "dst n %d rank %d" % (n, r))
+        prev_n = ns
+    p.compare_state(1e-5, "end")
+    p.close()
+
+
 def test_key_error_is_raised_by_preprocess_and_the_table_goes_on():
     say("bad key, early return")
     length, width, n = 1000, 8, 500
