@@ -37,6 +37,10 @@ def parse():
     ap.add_argument("--no-stage-timing", action="store_true")
     ap.add_argument("--no-variants", action="store_true",
                     help="skip the extra passes (literal call protocol, permuted ids): for profiles of the headline alone")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the short passes over the other configurations that the default cfg2 run appends as "
+                         "`other_configs`")
+    ap.add_argument("--other-steps", type=int, default=10, help="timed steps of each `other_configs` pass")
     ap.add_argument("--host-keys", action="store_true",
                     help="hand the ids over as pageable host buffers (adds their transfer to the step)")
     ap.add_argument("--pooled", action="store_true",
@@ -239,7 +243,7 @@ def main_partition(a):
     print(json.dumps(out), flush=True)
 
 
-def main_sharded(a, cfg):
+def run_sharded(a, cfg, steps, warmup, with_cpu, stage_timing=True, name=None):
     """cfg3: the shards of an 8-way partition live on this one GPU behind the loopback.  By default only rank 0 feeds
     batches and holds the hot-row cache; the seven peers own their rows and serve rank 0's pushes and queries with
     the real owner-side kernels (in a deployment that work runs on the other GPUs, here it is inside the step
@@ -247,6 +251,7 @@ def main_sharded(a, cfg):
     refreshed; the GPU then does the work of all eight ranks in turn and `value` counts all their keys."""
     import torch
     from hetuctr_amd import capi, workloads
+    name = name or name
     R, width, lr = cfg["nrank"], cfg["width"], cfg["lr"]
     active = list(range(R)) if a.active_peers else [0]
     ks = workloads.KeyStream(cfg, seed=0, scale=a.scale)
@@ -266,7 +271,7 @@ def main_sharded(a, cfg):
     ks.release_tables()
     n = batches[0][0].shape[0]
     print("[bench] %s: %d rows x %d over %d shards, rank 0 owns %d and caches %d rows, %d keys/batch, ranks with "
-          "batches: %s" % (a.config, ks.rows, width, R, int((root == 0).sum()),
+          "batches: %s" % (name, ks.rows, width, R, int((root == 0).sum()),
                            storage[0].shape[0] - int((root == 0).sum()), n, active), file=sys.stderr, flush=True)
     torch.cuda.set_device(0)
     capi.seed(0)
@@ -292,27 +297,28 @@ def main_sharded(a, cfg):
         c.preprocess()
         c.push_pull()
 
-    w0 = max(a.warmup, 2) + nb
+    w0 = max(warmup, 2) + nb
     for i in range(w0):
         step(i)
     # the timed pass: nothing but the two calls of every step
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(a.steps):
+    for i in range(steps):
         step(w0 + i)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    # the library's own device times of the two calls (a pass of its own: reading them switches their events on)
+    # the library's own device times of the two calls (a pass of its own: their events cost host time)
     pre_ms = pp_ms = 0.0
-    tables[0].last_times()
-    for i in range(a.steps):
+    tables[0].call_timing(True)
+    for i in range(steps):
         step(w0 + i)
         p, q = tables[0].last_times()
         pre_ms += p
         pp_ms += q
+    tables[0].call_timing(False)
     # how long each of the two calls holds the host (a pass of its own: the clock reads cost time)
     call_s = [0.0, 0.0]
-    for i in range(a.steps):
+    for i in range(steps):
         c = calls[(w0 + i) % nb]
         t1 = time.perf_counter()
         c.preprocess()
@@ -322,35 +328,35 @@ def main_sharded(a, cfg):
         call_s[0] += t2 - t1
         call_s[1] += t3 - t2
     stages = None
-    if not a.no_stage_timing:
+    if stage_timing and not a.no_stage_timing:
         tables[0].stage_timing(True)
-        for i in range(a.steps):
-            step(w0 + a.steps + i)
-        stages = {k: {"ms_per_step": v[0] / a.steps, "intervals_per_step": v[1] / a.steps}
+        for i in range(steps):
+            step(w0 + steps + i)
+        stages = {k: {"ms_per_step": v[0] / steps, "intervals_per_step": v[1] / steps}
                   for k, v in tables[0].stage_times().items() if v[1]}
         tables[0].stage_timing(False)
-    k = min(a.steps, nb)                     # counters of a few more steps, outside the timed region
+    k = min(steps, nb)                     # counters of a few more steps, outside the timed region
     acc = np.zeros(6)                        # per step, summed over the ranks: hit, miss, refreshed, pushed, returned, received
     us = 0.0
     for i in range(k):
-        step(w0 + 2 * a.steps + i)
+        step(w0 + 2 * steps + i)
         for t in tables:
             acc += np.asarray(t.fetch(capi.STATS)[:6], dtype=np.float64) / k
         us += sum(float(tables[r].fetch(capi.SIZES)[1]) for r in active) / k
     hit, miss, refresh, pushed, served, received = acc
-    ms_step = 1e3 * dt / a.steps
+    ms_step = 1e3 * dt / steps
     keys_step = n * len(active)
     bytes_step = workloads.algorithmic_bytes(keys_step, us, width) + workloads.sharded_extra_bytes(
         width, hit + refresh, pushed, received, us, served, refresh)
     gbs = bytes_step / (ms_step * 1e-3) / 1e9
     out = {
-        "metric": "sparse IDs/sec per train step (pull+push)", "value": keys_step * a.steps / dt, "unit": "IDs/s",
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_step, "higher_is_better": True,
+        "metric": "sparse IDs/sec per train step (pull+push)", "value": keys_step * steps / dt, "unit": "IDs/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: %d shards of a %d-row x %d fp32 table (%s) on one GPU behind the "
                                "loopback, ranks %s feed batches of %d keys (per-field Zipf %.2f) and cache %.0f%% of "
                                "their remote rows (%s), bounds pull/push %d/%d; the other ranks only serve" %
-                               (a.config, R, ks.rows, width,
+                               (name, R, ks.rows, width,
                                 "uniform owners" if a.layout == "random" else "owners from the offline partitioner",
                                 active, n, cfg["alpha"], 100 * cfg["cache_frac"],
                                 "the hottest" if a.layout == "random" else "the partitioner's first candidates; "
@@ -359,8 +365,8 @@ def main_sharded(a, cfg):
                    "keys_per_step": keys_step, "unique_keys_per_step": us, "width": width, "rows": ks.rows},
         "cache_per_step_all_ranks": {"remote_unique_keys_hit": hit, "missed_not_cached": miss, "refreshed": refresh,
                                      "rows_pushed_to_owners": pushed, "rows_returned_by_owners": served},
-        "device_ms_per_step": {"preprocess": pre_ms / a.steps, "push_pull": pp_ms / a.steps},
-        "host_ms_per_call": {"preprocess": 1e3 * call_s[0] / a.steps, "push_pull": 1e3 * call_s[1] / a.steps},
+        "device_ms_per_step": {"preprocess": pre_ms / steps, "push_pull": pp_ms / steps},
+        "host_ms_per_call": {"preprocess": 1e3 * call_s[0] / steps, "push_pull": 1e3 * call_s[1] / steps},
         "step_hbm": {"algorithmic_bytes": int(bytes_step), "achieved_GBps": gbs, "frac": gbs / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": "whole step (all shards' kernels)", "achieved": gbs, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None, "avg_ms": ms_step,
@@ -374,19 +380,126 @@ def main_sharded(a, cfg):
     # under profiles/), valid for the default invocation only
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath) and a.scale == 1.0 and not a.active_peers and a.layout == "random" and bounds == (0, 0):
-        measured = json.load(open(tpath)).get(a.config)
+        measured = json.load(open(tpath)).get(name)
         if measured:
             out["roofline"]["traffic"] = measured.get("whole_step")
             out["kernels"] = {k: v for k, v in measured.items() if k != "whole_step"}
-    if not a.no_cpu:
-        del dkeys, grad, dsts
-        torch.cuda.empty_cache()
+    del dkeys, grad, dsts
+    torch.cuda.empty_cache()
+    if with_cpu:
         try:
             out["cpu_baseline"] = cpu_baseline_sharded(ks, R, width, lr, bounds, root, storage, batches, active,
                                                        a.cpu_steps)
         except Exception as e:  # the GPU line stands without it
             out["cpu_baseline"] = {"value": None, "error": str(e)}
-    print(json.dumps(out), flush=True)
+    return out
+
+
+def quick_single(name, cfg, steps, warmup, host_keys=False, stage_timing=True):
+    """A short pass over one single-shard configuration: `warmup` untimed steps, `steps` timed ones (nothing but the
+    two calls in the loop), then the same steps with stage events for the push and gather kernels alone.  The table
+    and every buffer are released before it returns."""
+    import torch
+    from hetuctr_amd import capi, workloads
+    width, lr = cfg["width"], cfg["lr"]
+    ks = workloads.KeyStream(cfg, seed=0)
+    batches = [ks.batch() for _ in range(3)]
+    ks.release_tables()
+    n = batches[0].shape[0]
+    capi.seed(0)
+    table = capi.Table(0, 1, 0, "127.0.0.1", 23456, ks.rows, width, 0, 0, np.zeros(ks.rows, np.uint8),
+                       np.arange(ks.rows, dtype=np.int64), cfg["init"], lr, 0)
+    dkeys = [torch.from_numpy(b).cuda() for b in batches]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    grad = torch.randn((n, width), device="cuda", generator=gen) * 1e-3
+    dst = torch.empty((n, width), device="cuda")
+    torch.cuda.synchronize()
+    ptrs = [b.ctypes.data for b in batches] if host_keys else [d.data_ptr() for d in dkeys]
+
+    def step(i):
+        table.preprocess(ptrs[i % len(ptrs)], n)
+        table.push_pull(grad.data_ptr(), dst.data_ptr())
+
+    us = []
+    for i in range(max(warmup, len(ptrs) + 1)):
+        step(i)
+        us.append(int(table.fetch(capi.SIZES)[1]))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms = 1e3 * (time.perf_counter() - t0) / steps
+    u = float(np.mean(us[-len(ptrs):]))
+    res = {"workload": "%s: %d-row x %d fp32 table, %d samples x %d fields x %d ids = %d keys per batch, %s, ids handed "
+                       "over in %s" % (name, ks.rows, width, ks.samples, ks.fields, ks.hot, n,
+                                       "uniform ids" if cfg["alpha"] is None else "per-field Zipf %.2f" % cfg["alpha"],
+                                       "pageable host memory" if host_keys else "HBM"),
+           "steps": steps, "warmup": warmup, "ms_per_step": ms, "value": n / (ms * 1e-3), "keys_per_step": n,
+           "unique_keys_per_step": u,
+           "step_hbm_frac": workloads.algorithmic_bytes(n, u, width) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    if stage_timing:
+        table.stage_timing(True)
+        for i in range(steps):
+            step(i)
+        st = table.stage_times()
+        table.stage_timing(False)
+        res["stage_ms"] = {k: v[0] / max(v[1], 1) for k, v in st.items() if v[1]}
+        for k, kern in (("segment_sum_apply", "push_fused"), ("gather", "gather")):
+            if k in res["stage_ms"]:
+                res[kern + "_frac"] = (workloads.stage_bytes(k, n, u, n, u, width) / (res["stage_ms"][k] * 1e-3) / 1e9 /
+                                       HBM_PEAK_GBS)
+    table.close()
+    del dkeys, grad, dst
+    torch.cuda.empty_cache()
+    return res
+
+
+def other_configs(a):
+    """Short passes (no CPU leg) over every other configuration the headline is not quoted on, the reference's own
+    default batch (tests/benchmark.py:74-75: 2048 samples x 26 fields) and cfg2 with the ids in pageable host memory,
+    as every script of the reference hands them over (tests/benchmark.py:63)."""
+    from hetuctr_amd import workloads
+    out = {}
+    K, W = a.other_steps, 5
+
+    def run(name, f):
+        t0 = time.perf_counter()
+        try:
+            out[name] = f()
+        except Exception as e:  # the headline stands without it
+            out[name] = {"error": "%s: %s" % (type(e).__name__, e)}
+        print("[bench] other_configs.%s done in %.1fs" % (name, time.perf_counter() - t0), file=sys.stderr, flush=True)
+
+    small = dict(workloads.CONFIGS["cfg2"])
+    small["samples"] = 2048
+    run("samples_2048", lambda: quick_single("cfg2 table, 2048-sample batches", small, 5 * K, 2 * W))
+    run("cfg2_host_ids", lambda: quick_single("cfg2", workloads.CONFIGS["cfg2"], K, W, host_keys=True, stage_timing=False))
+    run("cfg1", lambda: quick_single("cfg1", workloads.CONFIGS["cfg1"], 5 * K, 2 * W))
+
+    def cfg3():
+        r = run_sharded(a, dict(workloads.CONFIGS["cfg3"]), K, W, with_cpu=False, name="cfg3")
+        keep = ("ms_per_step", "value", "steps", "warmup", "cache_per_step_all_ranks", "device_ms_per_step",
+                "host_ms_per_call")
+        res = {k: r[k] for k in keep}
+        res["workload"] = r["config"]["workload"]
+        res["keys_per_step"] = r["config"]["keys_per_step"]
+        res["unique_keys_per_step"] = r["config"]["unique_keys_per_step"]
+        res["step_hbm_frac"] = r["step_hbm"]["frac"]
+        if r.get("stages_all_shards"):
+            res["stage_ms"] = {k: v["ms_per_step"] for k, v in r["stages_all_shards"].items()}
+        return res
+
+    run("cfg3", cfg3)
+    run("cfg4", lambda: quick_single("cfg4", workloads.CONFIGS["cfg4"], K, W))
+    run("cfg5_zipf", lambda: quick_single("cfg5_zipf", workloads.CONFIGS["cfg5_zipf"], K, W))
+    run("cfg5_uniform", lambda: quick_single("cfg5_uniform", workloads.CONFIGS["cfg5_uniform"], K, W))
+    return out
+
+
+def main_sharded(a, cfg):
+    print(json.dumps(run_sharded(a, cfg, a.steps, a.warmup, not a.no_cpu)), flush=True)
 
 
 def main():
@@ -474,16 +587,17 @@ def main():
         step(w0 + i)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    # ---- device time of the two calls (HIP events inside the library, switched on by the first query): a pass of
+    # ---- device time of the two calls (HIP events inside the library, switched on for this pass only): a pass of
     # its own, because the events cost host time in every call
     pre_ms = pp_ms = push_ms = 0.0
-    table.last_times()
+    table.call_timing(True)
     for i in range(a.steps):
         step(w0 + i)
         p, q = table.last_times()
         pre_ms += p
         pp_ms += q
         push_ms += table.last_push_ms()
+    table.call_timing(False)
     # ---- same K steps again with every stage bracketed by HIP events on the table's stream (the events cost a
     # few microseconds per stage, so the throughput above is taken without them)
     stages = {}
@@ -616,13 +730,20 @@ def main():
         "permuted_ids": permuted,
     }
     if not a.no_cpu:
-        del dst
+        dst = None
         torch.cuda.empty_cache()
         try:
             out["cpu_baseline"] = cpu_baseline(cfg, ks, batches, width, lr, a.cpu_steps)
         except MemoryError as e:  # pragma: no cover
             out["cpu_baseline"] = {"value": None, "error": str(e)}
     table.close()
+    # every other configuration in the same record: the headline keys above stay as they are
+    default_run = (a.config == "cfg2" and a.scale == 1.0 and not a.samples and not a.host_keys and not a.pooled and
+                   not a.no_variants and not a.no_others)
+    if default_run:
+        dkeys = grad = dst = None
+        torch.cuda.empty_cache()
+        out["other_configs"] = other_configs(a)
     print(json.dumps(out), flush=True)
 
 

@@ -11,7 +11,7 @@ LIB_PATH = os.environ.get("HETUCTR_LIB") or os.path.join(_HERE, "lib", "libhetuc
 INIT = {"Zero": 0, "Normal": 1, "Uniform": 2, "TruncatedNormal": 3}
 SYMBOLS = ["hctr_create", "hctr_destroy", "hctr_preprocess", "hctr_preprocess_noalloc", "hctr_push_pull", "hctr_push_pull_pooled",
            "hctr_group_preprocess", "hctr_group_push_pull", "hctr_group_push_pull_pooled", "hctr_seed", "hctr_repr", "hctr_debug", "hctr_last_error", "hctr_debug_fetch", "hctr_save", "hctr_load",
-           "hctr_stream", "hctr_last_times", "hctr_last_push_ms", "hctr_defer_index", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
+           "hctr_stream", "hctr_call_timing", "hctr_last_times", "hctr_last_push_ms", "hctr_defer_index", "hctr_stage_timing", "hctr_stage_count", "hctr_stage_name",
            "hctr_stage_times", "hctr_copy_probe", "hctr_sample_rows", "hctr_version", "hctr_part_create", "hctr_part_destroy",
            "hctr_part_sizes", "hctr_part_refine_data", "hctr_part_refine_embed", "hctr_part_get_communication",
            "hctr_part_get_priority", "hctr_part_get_result", "hctr_part_get_counts", "hctr_part_cache_lists"]
@@ -59,6 +59,7 @@ def lib():
         l.hctr_save.argtypes = [C.c_void_p, C.c_char_p]
         l.hctr_load.argtypes = [C.c_void_p, C.c_char_p]
         l.hctr_stream.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        l.hctr_call_timing.argtypes = [C.c_void_p, C.c_int]
         l.hctr_last_times.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
         l.hctr_last_push_ms.argtypes = [C.c_void_p, C.POINTER(C.c_float)]
         l.hctr_defer_index.argtypes = [C.c_void_p, C.c_int]
@@ -154,6 +155,10 @@ class Table:
         s = C.c_void_p()
         _check(lib().hctr_stream(self._h, C.byref(s)))
         return s.value
+
+    def call_timing(self, on):
+        """Switches the HIP events around the two calls on or off (last_times / last_push_ms need them on)."""
+        _check(lib().hctr_call_timing(self._h, int(on)))
 
     def last_times(self):
         a, b = C.c_float(), C.c_float()

@@ -187,10 +187,17 @@ int hctr_stream(hctr_table *t, void **stream_out) {
   });
 }
 
+int hctr_call_timing(hctr_table *t, int on) {
+  return guarded([&] {
+    HCTR_CHECK(t && t->shard, "null table");
+    t->shard->group->set_call_timing(on != 0);
+  });
+}
+
 int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms) {
   return guarded([&] {
     HCTR_CHECK(t && t->shard, "null table");
-    t->shard->group->time_calls = true; // the calls after this one are bracketed with events
+    HCTR_CHECK(t->shard->group->time_calls, "call timing is off: switch it on with hctr_call_timing(t, 1) first");
     if (preprocess_ms) *preprocess_ms = t->shard->last_pre_ms;
     if (push_pull_ms) *push_pull_ms = t->shard->last_pp_ms;
   });
@@ -199,7 +206,7 @@ int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms) {
 int hctr_last_push_ms(hctr_table *t, float *push_ms) {
   return guarded([&] {
     HCTR_CHECK(t && t->shard && push_ms, "null argument");
-    t->shard->group->time_calls = true;
+    HCTR_CHECK(t->shard->group->time_calls, "call timing is off: switch it on with hctr_call_timing(t, 1) first");
     *push_ms = t->shard->last_push_ms;
   });
 }

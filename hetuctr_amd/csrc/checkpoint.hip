@@ -13,6 +13,8 @@
 #include <cstring>
 #include <vector>
 
+#include <sys/stat.h>
+
 #include "table.h"
 
 namespace hctr {
@@ -43,6 +45,16 @@ struct File {
   }
   ~File() {
     if (f) fclose(f);
+  }
+  void close() { // a failed close loses buffered data: it is an error of the write, not something to ignore
+    FILE *g = f;
+    f = nullptr;
+    HCTR_CHECK(fclose(g) == 0, "cannot close " + path + ": " + strerror(errno));
+  }
+  uint64_t size() {
+    struct stat sb;
+    HCTR_CHECK(fstat(fileno(f), &sb) == 0, "cannot stat " + path + ": " + strerror(errno));
+    return (uint64_t)sb.st_size;
   }
   void write(const void *d, size_t n) { HCTR_CHECK(fwrite(d, 1, n, f) == n, "short write to " + path); }
   void read(void *d, size_t n) { HCTR_CHECK(fread(d, 1, n, f) == n, "short read from " + path + " (truncated file?)"); }
@@ -94,14 +106,24 @@ void Shard::save(const char *path) {
   h.pull_bound = tv.pull_bound, h.push_bound = tv.push_bound;
   const size_t S = tv.n_stored, C = tv.n_cached, W = tv.width;
   Staging st;
-  File out(path, "wb");
-  out.write(&h, sizeof h);
-  device_to_file(out, store_ids.p, S * sizeof(index_t), st, s);
-  device_to_file(out, emb.p, S * W * sizeof(embed_t), st, s);
-  device_to_file(out, ver.p, S * sizeof(version_t), st, s);
-  device_to_file(out, pend.p, C * W * sizeof(embed_t), st, s);
-  device_to_file(out, upd.p, C * sizeof(version_t), st, s);
-  HCTR_CHECK(fflush(out.f) == 0, "cannot flush " + out.path);
+  // written beside the target and renamed over it when it is complete and closed: a crash or a full disk in the
+  // middle leaves the checkpoint that was there before
+  const std::string tmp = std::string(path) + ".tmp";
+  try {
+    File out(tmp.c_str(), "wb");
+    out.write(&h, sizeof h);
+    device_to_file(out, store_ids.p, S * sizeof(index_t), st, s);
+    device_to_file(out, emb.p, S * W * sizeof(embed_t), st, s);
+    device_to_file(out, ver.p, S * sizeof(version_t), st, s);
+    device_to_file(out, pend.p, C * W * sizeof(embed_t), st, s);
+    device_to_file(out, upd.p, C * sizeof(version_t), st, s);
+    HCTR_CHECK(fflush(out.f) == 0, "cannot flush " + out.path + ": " + strerror(errno));
+    out.close();
+    HCTR_CHECK(rename(tmp.c_str(), path) == 0, "cannot rename " + tmp + " to " + path + ": " + strerror(errno));
+  } catch (...) {
+    (void)remove(tmp.c_str());
+    throw;
+  }
 }
 
 void Shard::load(const char *path) {
@@ -119,14 +141,18 @@ void Shard::load(const char *path) {
   HCTR_CHECK(h.n_stored == tv.n_stored && h.n_cached == tv.n_cached,
              "checkpoint of a shard with other resident rows (storage_arr differs)");
   const size_t S = tv.n_stored, C = tv.n_cached, W = tv.width;
+  // all or nothing: the length of the file is checked before the first array of the table is overwritten
+  const uint64_t want = sizeof(Header) + (uint64_t)S * sizeof(index_t) + (uint64_t)S * W * sizeof(embed_t) +
+                        (uint64_t)S * sizeof(version_t) + (uint64_t)C * W * sizeof(embed_t) + (uint64_t)C * sizeof(version_t);
+  const uint64_t have = in.size();
+  HCTR_CHECK(have >= want, "checkpoint is shorter than the table (truncated file?): " + in.path);
+  HCTR_CHECK(have == want, "checkpoint is longer than the table: " + in.path);
   Staging st;
   compare_with_device(in, store_ids.p, S * sizeof(index_t), st, s, "the resident ids");
   file_to_device(in, emb.p, S * W * sizeof(embed_t), st, s);
   file_to_device(in, ver.p, S * sizeof(version_t), st, s);
   file_to_device(in, pend.p, C * W * sizeof(embed_t), st, s);
   file_to_device(in, upd.p, C * sizeof(version_t), st, s);
-  char extra;
-  HCTR_CHECK(fread(&extra, 1, 1, in.f) == 0, "checkpoint is longer than the table: " + in.path);
   // the batches in flight belong to the run that wrote the file, not to this one: start from empty ones
   for (Batch *b : {&cur, &prev}) {
     b->n = 0;

@@ -165,6 +165,9 @@ class TableContainer {
     if (hctr_debug_fetch(table_, which, out.mutable_data(), n, &n)) raise_last();
     return std::move(out);
   }
+  void callTiming(bool on) {
+    if (hctr_call_timing(table_, on ? 1 : 0)) raise_last();
+  }
   py::tuple lastTimes() {
     float a = 0, b = 0;
     if (hctr_last_times(table_, &a, &b)) raise_last();
@@ -208,6 +211,7 @@ PYBIND11_MODULE(hetuCTR, m) {
       .def("__repr__", &TableContainer::debugString)
       .def("debug", &TableContainer::debugStringFull)
       .def("debug_fetch", &TableContainer::debugFetch, py::arg("which"))
+      .def("call_timing", &TableContainer::callTiming, py::arg("on"))
       .def("last_times", &TableContainer::lastTimes);
 
   m.def("seed", [](unsigned long seed) { hctr_seed(seed); });

@@ -221,7 +221,7 @@ class Group {
   void place_queries();
   DeviceBuf rq_idx_all, rq_ver_all, query_delta_dev;
   uint32_t *query_delta_host = nullptr;
-  bool time_calls = false;               // bracket the two calls with events (hctr_last_times switches it on)
+  bool time_calls = false;               // bracket the two calls with events (hctr_call_timing)
   std::vector<Shard *> members;
   double wait_seconds = 120.0;
   void sync_stream();
@@ -236,6 +236,7 @@ class Group {
   hipEvent_t take_event();
   void collect_marks();                  // after a stream sync
   void set_defer_index(bool on);         // switches the early return of preprocess; waits for a pending index first
+  void set_call_timing(bool on);         // events around the two calls; the times of earlier calls are forgotten
   void set_stage_timing(bool on);        // resets the accumulators; waits for a pending index under the group's lock
 
   void join(Shard *s);
@@ -254,6 +255,8 @@ class Group {
 
  private:
   void exchange_shapes();
+  void push_pull_steps(const float *const *grads, float *const *dsts, uint32_t bag); // the body of push_pull_all
+  bool index_joining_ = false; // push_pull has taken a pending index over and not yet read its results
   template <typename F> void collective(int rank, int op, F &&run_all);
   std::mutex mu_;
   std::condition_variable cv_;

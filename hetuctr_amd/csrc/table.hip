@@ -777,6 +777,13 @@ void Group::set_defer_index(bool on) {
   defer_index = on;
 }
 
+void Group::set_call_timing(bool on) {
+  std::lock_guard<std::mutex> lk(mu_);
+  time_calls = on;
+  for (Shard *m : members)
+    if (m) m->last_pre_ms = m->last_pp_ms = m->last_push_ms = 0.f;
+}
+
 void Group::set_stage_timing(bool on) {
   std::lock_guard<std::mutex> lk(mu_); // not while the ranks of the group are inside a collective call
   flush_index();
@@ -1070,6 +1077,33 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
   const uint32_t bag = (uint32_t)bag_size;
   HCTR_CHECK(complete(), "the loopback group named by (ip, port) is missing ranks");
   HCTR_HIP(hipSetDevice(device_id));
+  // every caller error that can be seen from the arguments is reported here, before any batch is touched or any
+  // kernel is launched: a refused call leaves the table as it found it
+  for (Shard *m : members) {
+    const int r = m->cfg.rank;
+    HCTR_CHECK(grads[r] == nullptr || m->prev.n % bag == 0, "pooled push: the previous batch is not a whole number of bags");
+    HCTR_CHECK(dsts[r] == nullptr || m->cur.n % bag == 0, "pooled pull: the batch is not a whole number of bags");
+  }
+  try {
+    push_pull_steps(grads, dsts, bag);
+  } catch (...) {
+    // Something failed after work was enqueued (a runtime error, a device-side check).  Nothing may still be running
+    // when the caller sees the error, and an index that this call started to join is handed back to the next call
+    // that needs it (flush_index takes its results over) instead of being dropped with its batch.
+    (void)hipStreamSynchronize(index_stream);
+    (void)hipStreamSynchronize(stream);
+    for (auto &mk : marks) {
+      event_pool.push_back(mk.a);
+      event_pool.push_back(mk.b);
+    }
+    marks.clear();
+    if (index_joining_) index_pending = true;
+    index_joining_ = false;
+    throw;
+  }
+}
+
+void Group::push_pull_steps(const float *const *grads, float *const *dsts, uint32_t bag) {
   if (time_calls) HCTR_HIP(hipEventRecord(ev0, stream));
   for (Shard *m : members) m->begin_push(grads[m->cfg.rank], bag);
   place_pushes();
@@ -1094,9 +1128,11 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
       // the queries are built from the index of the current batches, which the host needs too (unique keys and queries
       // per owner place the queries)
       index_pending = false;
+      index_joining_ = true;
       HCTR_HIP(hipEventSynchronize(ev_index));
       for (Shard *m : members) m->finish_index();
       exchange_shapes();
+      index_joining_ = false;
     }
   }
   place_queries();
@@ -1106,6 +1142,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
     // the push kernel is in the main stream's queue; the gather below also needs the index of the current batch,
     // still running or done on the second stream
     index_pending = false;
+    index_joining_ = true;
     HCTR_HIP(hipStreamWaitEvent(stream, ev_index, 0));
   }
   if (nrank > 1) {
@@ -1120,6 +1157,7 @@ void Group::push_pull_all(const float *const *grads, float *const *dsts, size_t 
   if (nrank > 1)
     for (Shard *m : members) m->finish_plan(m->cur);
   if (join_index) {
+    index_joining_ = false; // from here on the results are taken over, or the batch's own error is reported
     members[0]->finish_preprocess();
     exchange_shapes();
   }

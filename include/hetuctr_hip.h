@@ -54,12 +54,19 @@ int hctr_destroy(hctr_table *t);
 
 /* Replaces HetuTable::preprocess (csrc/core/hetu_gpu_table.cu:43-65): the previous batch becomes the
  * one whose gradients come next, `keys` (int64[n], HOST OR DEVICE memory) becomes the current batch.
- * Synchronous.  With nrank > 1 the call completes when every shard of the group has made it. */
+ * The call returns when the caller's ids have been read (the buffer may be reused at once) and any error in them has
+ * been reported; sorting and deduplicating them goes on behind the return and is waited for by whatever needs it
+ * next (hctr_push_pull, a second hctr_preprocess, hctr_debug_fetch).  This is the one deviation from the reference,
+ * whose call returns when all of its work is done (hetu_gpu_table.cu:64): hctr_defer_index(t, 0), or
+ * HETUCTR_DEFER_INDEX=0 in the environment, restores exactly that.  The details of the early return are with
+ * hctr_defer_index below.  With nrank > 1 the call completes when every shard of the group has made it. */
 int hctr_preprocess(hctr_table *t, const int64_t *keys, size_t n);
 
-/* hctr_preprocess for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same result as hctr_preprocess, and like the
- * reference's call it returns when all its work is done; it calls no hipMalloc / hipFree and no allocating routine:
+/* hctr_preprocess for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same result as hctr_preprocess with the early return switched off:
+ * like the reference's call it returns when all its work is done.  It calls no hipMalloc / hipFree and no allocating
+ * routine; it does synchronise the table's stream and reads counts back to the host, so it cannot be recorded into a
+ * HIP graph:
  *   - the index scratch (sort ping-pong buffers, per-tile digit counts, scan sums) lives in a static device array of
  *     7.0 MiB that every GPU the library runs on holds until the process ends;
  *   - n is at most 262144 keys (HCTR_NOALLOC_MAX_KEYS), larger batches are refused;
@@ -136,8 +143,10 @@ int hctr_stream(hctr_table *t, void **stream_out);
 
 /* Device time of the last preprocess and push_pull calls in milliseconds, measured with HIP events on
  * that stream around the launched work (host-side waits excluded).  The events cost host time in every call, so they
- * are recorded only from the first call of this function (or of hctr_last_push_ms) on: it returns zeros and
- * switches the measurement on for the calls that follow. */
+ * are recorded only while hctr_call_timing(t, 1) is in force (off when a table is created; switching it either way
+ * zeroes the stored times).  While it is off hctr_last_times and hctr_last_push_ms fail with an error instead of
+ * returning stale or zero times.  No counterpart in the reference. */
+int hctr_call_timing(hctr_table *t, int on);
 int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
 
 /* hctr_preprocess returns as soon as the caller's ids have been read (the buffer may be reused).  With several shards
@@ -149,7 +158,7 @@ int hctr_last_times(hctr_table *t, float *preprocess_ms, float *push_pull_ms);
  * that return, push_pull_ms covers the rest.  Anything that needs the batch's index earlier (a second hctr_preprocess,
  * hctr_debug_fetch, hctr_stage_timing) waits for it.  HETUCTR_DEFER_INDEX=0 in the environment restores a
  * preprocess that returns only when all its work is done (hetu_gpu_table.cu:64); with stage timing on it always is.
- * hctr_last_push_ms: device time from the start of the last hctr_push_pull to the end of its push stage, i.e. the
+ * hctr_last_push_ms (needs hctr_call_timing, like hctr_last_times): device time from the start of the last hctr_push_pull to the end of its push stage, i.e. the
  * push kernel while the index of the next batch runs beside it.  No counterpart in the reference. */
 int hctr_last_push_ms(hctr_table *t, float *push_ms);
 /* The same switch as HETUCTR_DEFER_INDEX for a table's group at run time: 0 makes hctr_preprocess return only when

@@ -12,11 +12,16 @@
 //
 // Pinning status of each function (what checks it, beyond re-typing it):
 //   init_values Zero/Uniform     closed form s*48271^(n+1) mod (2^31-1) in python
-//                                ints + the reference's own initializer.cu built
-//                                against the image's thrust (oracle/_ref)
-//   init_values Normal/Truncated formula pinned by oracle/_ref (rocThrust erfcinv);
-//                                the bit pattern of CUDA's erfcinvf is not
-//                                reproducible here: PARITY UNPINNED at bit level
+//                                ints and rationals (also committed as known answers)
+//   init_values Normal/Truncated formula pinned by the inverse normal CDF of python's
+//                                statistics.NormalDist in float64 (constants, sign,
+//                                mirror and redraw rule); the bit pattern of CUDA's
+//                                erfcinvf is not reproducible here: PARITY UNPINNED
+//                                at bit level
+//                                (oracle/_ref/libref_initializer.so, the reference's
+//                                initializer.cu compiled against the image's rocThrust,
+//                                is a cross-check only: rocThrust stands in for the
+//                                CUDA Thrust the reference uses, so it pins nothing)
 //   preprocess_index             numpy lexsort / unique / searchsorted, brute force
 //   preprocess_gradient, generate_gradient, handle_*, write_back
 //                                closed forms of tests/test_update.py (exact counts,

@@ -94,10 +94,30 @@ def test_refusals(tmp_path):
     perm = capi.Table(0, 1, 0, "", 0, length, width, 0, 0, root, st[::-1].copy(), ("Zero", 0, 0), 0.1)
     with pytest.raises(RuntimeError, match="resident ids"):
         perm.load(good)
+    assert not os.path.exists(good + ".tmp")              # written beside the target, renamed when complete
+    # a step moves the table away from what the file holds: a refused load must leave it exactly there
+    keys = torch.arange(0, 300, 3, dtype=torch.int64, device="cuda")
+    dst = torch.empty((100, width), device="cuda")
+    g = torch.full((100, width), 0.25, device="cuda")
+    torch.cuda.synchronize()
+    t.preprocess(keys.data_ptr(), 100)
+    t.push_pull(0, dst.data_ptr())
+    t.preprocess(keys.data_ptr(), 100)
+    t.push_pull(g.data_ptr(), dst.data_ptr())
+    emb, ver = t.fetch(capi.EMBEDDING), t.fetch(capi.VERSION)
+    saved = np.fromfile(good, dtype=np.float32, offset=64 + 8 * length, count=length * width)
+    assert not np.array_equal(emb, saved)
     cut = str(tmp_path / "cut.ckpt")
     open(cut, "wb").write(open(good, "rb").read()[:-100])
-    with pytest.raises(RuntimeError, match="short read"):
+    with pytest.raises(RuntimeError, match="shorter than the table"):
         t.load(cut)
+    longer = str(tmp_path / "long.ckpt")
+    open(longer, "wb").write(open(good, "rb").read() + b"\0" * 8)
+    with pytest.raises(RuntimeError, match="longer than the table"):
+        t.load(longer)
+    assert np.array_equal(t.fetch(capi.EMBEDDING), emb) and np.array_equal(t.fetch(capi.VERSION), ver)
+    with pytest.raises(RuntimeError, match="cannot open"):  # a target that cannot be written leaves nothing behind
+        t.save(str(tmp_path / "no_such_dir" / "t.ckpt"))
     junk = str(tmp_path / "junk.ckpt")
     open(junk, "wb").write(b"x" * 4096)
     with pytest.raises(RuntimeError, match="not a hetuCTR checkpoint"):

@@ -114,6 +114,47 @@ def test_skewed_keys_long_runs(alpha, width):
     p.close()
 
 
+@pytest.mark.parametrize("nrank", [1, 2])
+@pytest.mark.parametrize("width", [128, 20])
+def test_gradient_and_output_pointers_off_by_four_bytes(width, nrank):
+    # width % 4 == 0 but neither pointer 16-byte aligned: both kernels must fall back to 4-byte lanes (a 64-lane group
+    # per row at width 128) and still match the oracle bit for bit; skewed keys, so every role of the push runs
+    import torch
+    say("unaligned grad / dst, width", width, "shards", nrank)
+    rng = np.random.default_rng(700 + width + nrank)
+    length, n = 60_000, 50_000
+    root = rng.integers(0, nrank, size=length).astype(np.uint8)
+    storage = []
+    for r in range(nrank):
+        own, other = np.where(root == r)[0], np.where(root != r)[0]
+        storage.append(np.concatenate([other[::4], own]).astype(np.int64))
+    p = Pair(nrank, length, width, root, storage, init=("Uniform", -0.01, 0.01), lr=0.05, bounds=(2, 2) if nrank > 1 else (0, 0))
+    draw = zipf_sampler(length, 1.25, rng)
+    prev_n = 0
+    for step in range(4):
+        keys = [draw(n - 3 * step) for _ in range(nrank)]
+        p.preprocess(keys, device_keys=True)
+        grads = [rng.normal(0, 1e-3, size=(prev_n, width)).astype(np.float32) for _ in range(nrank)]
+        gbuf = [torch.empty(prev_n * width + 1, device="cuda") for _ in range(nrank)]   # one float of slack in front
+        dbuf = [torch.full((keys[r].shape[0] * width + 1,), float("nan"), device="cuda") for r in range(nrank)]
+        for r in range(nrank):
+            gbuf[r][1:].copy_(torch.from_numpy(grads[r].reshape(-1)))
+        torch.cuda.synchronize()
+        gptr = [gbuf[r].data_ptr() + 4 if prev_n else 0 for r in range(nrank)]
+        dptr = [dbuf[r].data_ptr() + 4 for r in range(nrank)]
+        assert all(q % 16 == 4 for q in dptr)
+        capi.group_push_pull(p.tables, gptr, dptr)
+        ref = p.oracle.push_pull([g if prev_n else None for g in grads])
+        for r in range(nrank):
+            out = dbuf[r][1:].cpu().numpy().reshape(-1, width)
+            assert_close(out, ref[r], 1e-5, "dst rank %d step %d" % (r, step))
+            assert np.isnan(dbuf[r][0].item())                 # nothing was written in front of the first row
+        p.compare_state(1e-5, "step %d" % step)
+        p.compare_ints([capi.VERSION, capi.UPDATES], "step %d" % step)
+        prev_n = n - 3 * step
+    p.close()
+
+
 @pytest.mark.parametrize("width", [48, 192, 256, 512, 1024])
 def test_long_runs_slice_layouts(width):
     # long runs with row widths that are cut into 1..32 column slices, or (48) take the path without slices
@@ -228,7 +269,9 @@ def test_key_buffer_is_free_when_preprocess_returns():
     length, width, n = 40_000, 32, 30_000
     p = single(length, width, lr=0.05)
     t, o = p.tables[0], p.oracle
-    assert t.last_times() == (0.0, 0.0)                   # and from now on the calls are timed
+    with pytest.raises(RuntimeError, match="call timing is off"):
+        t.last_times()                                    # no silent switch: the getter refuses while timing is off
+    t.call_timing(True)
     dev = torch.empty(n, dtype=torch.int64, device="cuda")
     host = np.empty(n, np.int64)
     dst = torch.empty((n, width), device="cuda")

@@ -85,6 +85,49 @@ def test_pooled_matches_the_plain_call_with_replicated_gradients():
     b.close()
 
 
+@pytest.mark.parametrize("nrank", [1, 2])
+def test_refused_bag_size_leaves_the_table_as_it_was(nrank):
+    # A pooled call whose bag does not divide the batch is refused before anything is launched, with the index of the
+    # current batch still pending from a preprocess that returned early: the same step repeated with a good bag must
+    # then give what a table that never saw the bad call gives, gradient of the previous batch included.
+    print("refused bag, shards", nrank, flush=True)
+    rng = np.random.default_rng(90 + nrank)
+    length, width, bag, bags = 9000, 16, 4, 1200
+    root = rng.integers(0, nrank, size=length).astype(np.uint8)
+    storage = []
+    for r in range(nrank):
+        own, other = np.where(root == r)[0], np.where(root != r)[0]
+        storage.append(np.concatenate([other[::3], own]).astype(np.int64))
+    mk = lambda: Pair(nrank, length, width, root, storage, init=("Uniform", -0.01, 0.01), lr=0.05, with_oracle=False)
+    a, b = mk(), mk()
+    draw = zipf_sampler(length, 1.15, rng)
+    prev = 0
+    for step in range(4):
+        keys = [draw(bags * bag) for _ in range(nrank)]
+        gp = [torch.from_numpy(rng.normal(0, 1e-3, size=(max(prev, 1), width)).astype(np.float32)).cuda() for _ in range(nrank)]
+        outs = []
+        for p in (a, b):
+            p.preprocess(keys, device_keys=True)
+            dd = [torch.full((bags, width), float("nan"), device="cuda") for _ in range(nrank)]
+            gptr = [g.data_ptr() if prev else 0 for g in gp]
+            torch.cuda.synchronize()
+            if p is b and step in (1, 2):
+                with pytest.raises(RuntimeError, match="whole number of bags"):   # 7 divides neither batch
+                    capi.group_push_pull_pooled(p.tables, gptr, [d.data_ptr() for d in dd], 7)
+                if step == 1:                                                     # the batches are still there (the
+                    for r in range(nrank):                                        # fetch waits for the pending index;
+                        assert p.tables[r].fetch(capi.SIZES)[1] > 0               # at step 2 the good call finds it pending)
+            capi.group_push_pull_pooled(p.tables, gptr, [d.data_ptr() for d in dd], bag)
+            outs.append([d.cpu().numpy() for d in dd])
+        for r in range(nrank):
+            assert np.array_equal(outs[0][r], outs[1][r]), "rank %d step %d" % (r, step)
+            for it in (capi.EMBEDDING, capi.VERSION, capi.PENDING, capi.UPDATES, capi.SIZES):
+                assert np.array_equal(a.tables[r].fetch(it), b.tables[r].fetch(it)), (r, step, it)
+        prev = bags
+    a.close()
+    b.close()
+
+
 @pytest.mark.parametrize("nrank,bounds", [(2, (0, 0)), (3, (3, 3))])
 def test_group_pooled(nrank, bounds):
     print("pooled group, shards", nrank, "bounds", bounds, flush=True)

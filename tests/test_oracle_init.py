@@ -1,10 +1,12 @@
 """Pins the oracle's table initialisers (reference: csrc/utils/initializer.cu:11-103).
 
 * Zero / Uniform: closed form of the minstd engine, computed here with python integers and exact
-  rationals (independent of the oracle's C++), and the reference's own initializer.cu compiled
-  against the image's thrust (oracle/_ref), when that library is present.
-* Normal / TruncatedNormal: the same reference build (its erfcinv is rocThrust's, not CUDA's, so
-  only a tolerance comparison is meaningful) + distribution moments + determinism.
+  rationals (independent of the oracle's C++): this is the pin.
+* Normal / TruncatedNormal: the inverse normal CDF of python's statistics.NormalDist in float64 (the pin of
+  the formula) + distribution moments + determinism.
+* The two *_vs_reference_build tests compare with the reference's own initializer.cu compiled against the
+  image's rocThrust (oracle/_ref), when that library is present.  rocThrust stands in for the CUDA Thrust the
+  reference is built with, so these are cross-checks that pin nothing.
 """
 from fractions import Fraction
 

@@ -44,7 +44,9 @@ def test_preprocess_noalloc_matches_preprocess(wide, monkeypatch):
         grad = torch.from_numpy(rng.normal(0, 1e-3, size=(max(prev_n, 1), width)).astype(np.float32)).cuda()
         torch.cuda.synchronize()
         a.preprocess(keys.data_ptr(), n)
+        free_before = torch.cuda.mem_get_info()[0]             # hipMemGetInfo: bytes free on the device
         b.preprocess_noalloc(keys.data_ptr(), n)
+        assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated or freed at step %d" % step
         for it in ITEMS:
             x, y = a.fetch(it), b.fetch(it)
             assert x.shape == y.shape and np.array_equal(x, y), "item %d differs at step %d" % (it, step)
