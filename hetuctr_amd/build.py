@@ -14,8 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIBDIR = os.path.join(HERE, "lib")
-HIP_SOURCES = ["radix_sort.hip", "preprocess.hip", "push.hip", "pull.hip", "init.hip", "table.hip", "checkpoint.hip", "loader.hip", "partition.hip", "c_api.hip"]
-HEADERS = ["common.h", "kernels.h", "radix_sort.h", "table.h", "partition.h", os.path.join("..", "..", "include", "hetuctr_hip.h")]
+HIP_SOURCES = ["radix_sort.hip", "tile_sort.hip", "preprocess.hip", "push.hip", "pull.hip", "init.hip", "table.hip", "checkpoint.hip", "loader.hip", "partition.hip", "c_api.hip"]
+HEADERS = ["common.h", "kernels.h", "radix_sort.h", "tile_sort.h", "run_lists.h", "table.h", "partition.h", os.path.join("..", "..", "include", "hetuctr_hip.h")]
 # packed-fp32 instruction selection is switched off for all device code; no fused multiply-add contraction, so
 # that "sum * -lr" then "row + that" rounds twice like the CPU restatement it is checked against (fused
 # operations are written explicitly where they are meant)

@@ -11,6 +11,7 @@ struct KeyLayout {
   int id_bits;    // bits of an id
   int total_bits; // id_bits + bits of an owner
   bool wide;      // 64-bit sort keys (total_bits > 32)
+  int max_digit_bits = 0; // widest digit of the tile-sorted passes (0: the most the sort takes); narrower for tests
 };
 
 // Device-side view of one preprocessed batch (the reference's PreprocessData,
@@ -78,15 +79,20 @@ struct TableView {
 // sort_counts: the sort's scratch, which receives the per-tile counts of the first pass' digit
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
                       void *comp_keys, uint32_t *err, uint32_t *nlong, uint32_t *sort_counts);
-// sorted keys -> everything per unique key + inverse index.  block_heads: scratch of scan_blocks(n) words.
+// sorted keys -> everything per unique key + inverse index.  heads: the head counts per chunk of sorted positions that
+// the last launch of the tile-sorted passes left (count_heads false), or storage for them (count_heads true: a launch
+// of its own counts them first, one chunk per tile of the unique pass).
 // u_copy (optional) receives the number of unique keys as well (b.d_U always does)
+struct HeadChunks;
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
-                   const BatchView &b, uint32_t *block_heads, uint32_t *u_copy);
+                   const BatchView &b, const HeadChunks &heads, bool count_heads, uint32_t *u_copy);
 
 // batch-order inverse index from sorted_arg and rank_sorted (introspection; the hot path does not need it)
 void launch_idx_map(hipStream_t s, const BatchView &b);
-// lists the runs longer than kLongRun by length class (after launch_unique)
+// the run lists of the batch (run_lists.h) by a launch of their own, after launch_unique; the gather builds them on its
+// way when PullArgs::list_chunks is set
 void launch_list_long_runs(hipStream_t s, const BatchView &b);
+inline uint32_t run_list_chunks(uint32_t n) { return (n + 255) / 256; } // enough for any number of unique keys <= n
 
 // device-wide exclusive scan of n (<= *d_n if d_n != nullptr) 32-bit values; block_sums: div_up(n_max,2048)+1 words.
 // total (optional) receives the sum.
@@ -212,6 +218,7 @@ struct PullArgs {
   const embed_t *in_val;
   embed_t *dst;              // [n][width]
   bool stream_stores;        // write dst with nontemporal stores (see Shard::write_back)
+  uint32_t list_chunks;      // the gather also builds the batch's run lists (run_lists.h): chunks of unique ranks, else 0
 };
 // Index of every returned row per unique key (a.ret_i), where the gather reads each key's row (a.src_row), the counts of
 // the step and the refresh of the cached rows that came back.  tile_sums: scratch of scan_blocks(n_unique) words;

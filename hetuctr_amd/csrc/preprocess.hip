@@ -5,6 +5,8 @@
 // cub RunLengthEncode / ExclusiveSum calls between them).
 #include "kernels.h"
 #include "radix_sort.h"
+#include "run_lists.h"
+#include "tile_sort.h"
 
 namespace hctr {
 namespace {
@@ -25,7 +27,8 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
                                                          uint32_t *__restrict__ counts) {
   __shared__ uint32_t h[kSortMaxBins];
   const uint32_t nb = 1u << dbits, mask = nb - 1;
-  for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
+  if (counts)
+    for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) h[i] = 0;
   if (blockIdx.x == 0 && threadIdx.x < kRunCounters && nlong) nlong[threadIdx.x] = 0; // counters of this batch
   const uint32_t base = blockIdx.x * (ITEMS * kSortBlock);
   uint64_t id[ITEMS];
@@ -53,8 +56,9 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
     const uint32_t i = base + k * kSortBlock + threadIdx.x;
     const K c = (K)((owner[k] << id_bits) | id[k]);
     if (i < n) comp[i] = c;
-    count_digit(h, (uint32_t)c & mask, i < n);
+    if (counts) count_digit(h, (uint32_t)c & mask, i < n);
   }
+  if (!counts) return; // the keys alone: another sort counts for itself
   __syncthreads();
   for (uint32_t i = threadIdx.x; i < nb; i += kSortBlock) counts[(size_t)blockIdx.x * nb + i] = h[i];
 }
@@ -67,65 +71,77 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
 constexpr int kUBlock = 512, kUItems = HCTR_UNIQUE_ITEMS, kUTile = kUBlock * kUItems;
 inline unsigned unique_tiles(uint32_t n) { return div_up(n, kUTile); }
 
-// the key before sorted position j of this lane: the neighbouring lane holds it, except for lane 0
-template <typename K>
-__device__ __forceinline__ K key_before(const K *__restrict__ sk, uint32_t j, bool valid, K mine) {
-  K edge = (K)0;
-  if (lane_id() == 0 && valid && j > 0) edge = sk[j - 1];
-  const K up = (K)__shfl_up(mine, 1, kWave);
-  return lane_id() == 0 ? edge : up;
-}
-
+// Heads (sorted positions that hold another key than the position before) are counted per chunk of sorted positions,
+// in a form that needs no look at a neighbouring chunk: the heads of a chunk other than its first position, and the
+// chunk's first and last key.  The last launch of the tile-sorted passes leaves these three per chunk (tile_sort.h);
+// after the other sort head_count makes them, one chunk per tile of the unique pass.
 template <typename K>
 __global__ __launch_bounds__(kUBlock) void head_count(const K *__restrict__ sk, uint32_t n,
-                                                      uint32_t *__restrict__ tile_heads) {
+                                                      uint32_t *__restrict__ inner, K *__restrict__ first,
+                                                      K *__restrict__ last) {
   __shared__ uint32_t sm[kUBlock / kWave + 1];
   const uint32_t base = blockIdx.x * kUTile;
-  K key[kUItems];
+  const unsigned lane = lane_id();
+  K key[kUItems], edge[kUItems];
 #pragma unroll
   for (int k = 0; k < kUItems; k++) {
     const uint32_t j = base + k * kUBlock + threadIdx.x;
     key[k] = j < n ? sk[j] : (K)0;
+    edge[k] = (lane == 0 && j < n && j > base) ? sk[j - 1] : (K)0; // the key before a wave's first position
   }
   uint32_t c = 0;
 #pragma unroll
   for (int k = 0; k < kUItems; k++) {
     const uint32_t j = base + k * kUBlock + threadIdx.x;
-    const K pk = key_before(sk, j, j < n, key[k]);
-    c += (j < n) && (j == 0 || key[k] != pk);
+    const K up = (K)__shfl_up(key[k], 1, kWave);
+    const K pk = lane == 0 ? edge[k] : up;
+    c += (j < n) && j > base && key[k] != pk;
   }
   uint32_t total;
   block_exclusive_scan<kUBlock>(c, sm, total);
-  if (threadIdx.x == 0) tile_heads[blockIdx.x] = total;
+  if (threadIdx.x == 0) {
+    inner[blockIdx.x] = total;
+    first[blockIdx.x] = key[0];
+    last[blockIdx.x] = sk[min(base + kUTile, n) - 1];
+  }
 }
 
-template <typename K>
+// One block per tile of ITEMS * kUBlock sorted positions; position j of a tile is handled by thread (j % kUBlock) in
+// round (j / kUBlock).  chunk: sorted positions per entry of the head counts (a divisor of the tile).
+template <typename K, int ITEMS>
 __global__ __launch_bounds__(kUBlock) void unique_emit(const K *__restrict__ sk, uint32_t n, int id_bits, int nrank,
                                                        const slot_t *__restrict__ slot,
-                                                       const uint32_t *__restrict__ tile_heads, BatchView b,
-                                                       uint32_t *__restrict__ u_copy) {
+                                                       const uint32_t *__restrict__ head_inner,
+                                                       const K *__restrict__ head_first, const K *__restrict__ head_last,
+                                                       uint32_t chunk, BatchView b, uint32_t *__restrict__ u_copy) {
   constexpr int NW = kUBlock / kWave;
+  constexpr uint32_t kTileU = ITEMS * kUBlock;
   __shared__ uint32_t sm[NW + 1];
-  __shared__ uint32_t wsum[kUItems * NW + 1];
-  const uint32_t base = blockIdx.x * kUTile;
+  __shared__ uint32_t wsum[ITEMS * NW + 1];
+  const uint32_t base = blockIdx.x * kTileU;
   const unsigned lane = lane_id();
   const int w = threadIdx.x / kWave;
-  // everything that comes from memory first: the keys of the tile and the head counts of the tiles before it
-  K key[kUItems], pk[kUItems];
+  // everything that comes from memory first: the keys of the tile, the key before every wave's first position and the
+  // head counts of the chunks before the tile
+  K key[ITEMS], edge[ITEMS], pk[ITEMS];
 #pragma unroll
-  for (int k = 0; k < kUItems; k++) {
+  for (int k = 0; k < ITEMS; k++) {
     const uint32_t j = base + k * kUBlock + threadIdx.x;
     key[k] = j < n ? sk[j] : (K)0;
+    edge[k] = (lane == 0 && j < n && j > 0) ? sk[j - 1] : (K)0;
   }
   uint32_t s = 0;
-  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kUBlock) s += tile_heads[i];
-  bool head[kUItems];
-  uint32_t before[kUItems];
+  const uint32_t chunks_before = base / chunk;
+  for (uint32_t i = threadIdx.x; i < chunks_before; i += kUBlock)
+    s += head_inner[i] + ((i == 0 || head_first[i] != head_last[i - 1]) ? 1u : 0u);
+  bool head[ITEMS];
+  uint32_t before[ITEMS];
 #pragma unroll
-  for (int k = 0; k < kUItems; k++) {
+  for (int k = 0; k < ITEMS; k++) {
     const uint32_t j = base + k * kUBlock + threadIdx.x;
     const bool valid = j < n;
-    pk[k] = key_before(sk, j, valid, key[k]);
+    const K up = (K)__shfl_up(key[k], 1, kWave);
+    pk[k] = lane == 0 ? edge[k] : up;
     head[k] = valid && (j == 0 || key[k] != pk[k]);
     const uint64_t m = __ballot(head[k]);
     before[k] = __popcll(m & ((1ull << lane) - 1ull));
@@ -133,24 +149,25 @@ __global__ __launch_bounds__(kUBlock) void unique_emit(const K *__restrict__ sk,
   }
   // the directory lookups of the heads travel while the ranks are worked out
   const K id_mask = (K)(((uint64_t)1 << id_bits) - 1);
-  slot_t off[kUItems];
+  slot_t off[ITEMS];
 #pragma unroll
-  for (int k = 0; k < kUItems; k++) off[k] = head[k] ? slot[(uint64_t)(key[k] & id_mask)] : kNoSlot;
+  for (int k = 0; k < ITEMS; k++) off[k] = head[k] ? slot[(uint64_t)(key[k] & id_mask)] : kNoSlot;
   uint32_t prefix;
   block_exclusive_scan<kUBlock>(s, sm, prefix); // unique ranks before this tile
   if (threadIdx.x < kWave) { // the wave totals, in item order, by one wave
     uint32_t run = 0;
-    for (int i0 = 0; i0 < kUItems * NW; i0 += kWave) {
-      const uint32_t v = wsum[i0 + lane];
+    for (int i0 = 0; i0 < ITEMS * NW; i0 += kWave) {
+      const bool in = i0 + (int)lane < ITEMS * NW;
+      const uint32_t v = in ? wsum[i0 + lane] : 0u;
       const uint32_t inc = wave_inclusive_scan(v);
-      wsum[i0 + lane] = run + inc - v;
+      if (in) wsum[i0 + lane] = run + inc - v;
       run += __shfl(inc, kWave - 1, kWave);
     }
   }
   __syncthreads();
   K *ukey = (K *)b.ukey;
 #pragma unroll
-  for (int k = 0; k < kUItems; k++) {
+  for (int k = 0; k < ITEMS; k++) {
     const uint32_t j = base + k * kUBlock + threadIdx.x;
     if (j >= n) continue;
     const uint32_t rank = prefix + wsum[k * NW + w] + before[k] + (head[k] ? 1u : 0u) - 1u;
@@ -181,32 +198,10 @@ __global__ __launch_bounds__(kBlock) void scatter_idx_map(BatchView b) {
   if (j < b.n) b.idx_map[b.sorted_arg[j]] = b.rank_sorted[j];
 }
 
-// one thread per unique rank: long runs are listed by length class, medium runs in one list, for the push.
-// Atomics on one address are served one after the other, so a block reserves its list entries with ONE atomic
-// per list: entries are counted and placed inside the block through LDS first.
-__global__ __launch_bounds__(kBlock) void list_long_runs(BatchView b) {
-  constexpr int kLists = kLongBuckets + 1; // length classes of long runs, then the medium list
-  __shared__ uint32_t cnt[kLists], base[kLists];
-  const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
-  if (blockIdx.x * kBlock >= *b.d_U) return; // whole block past the last unique key
-  if (threadIdx.x < kLists) cnt[threadIdx.x] = 0;
-  __syncthreads();
-  const bool valid = u < *b.d_U;
-  const uint32_t len = valid ? b.run_start[u + 1] - b.run_start[u] : 0u;
-  int list = -1;
-  if (len > kLongRun) list = long_bucket(len);
-  else if (len > kTinyRun) list = kLongBuckets;
-  uint32_t local = 0;
-  if (list >= 0) local = atomicAdd(&cnt[list], 1u); // LDS atomic: the order inside a list does not matter
-  __syncthreads();
-  if (threadIdx.x < kLists && cnt[threadIdx.x])
-    base[threadIdx.x] = atomicAdd(&b.d_nlong[threadIdx.x < kLongBuckets ? threadIdx.x : kMedCount], cnt[threadIdx.x]);
-  __syncthreads();
-  if (list >= 0) {
-    if (list < kLongBuckets)
-      b.long_list[(size_t)list * b.long_cap + base[list] + local] = make_uint4(u, b.run_start[u], len, (uint32_t)b.uoff[u]);
-    else b.med_list[base[list] + local] = u;
-  }
+// the run lists of a batch by a launch of their own (run_lists.h), for a batch no gather builds them for
+__global__ __launch_bounds__(kRunListBlock) void list_long_runs(BatchView b) {
+  __shared__ uint32_t cnt[kRunLists], base[kRunLists];
+  list_runs_chunk(b, blockIdx.x, cnt, base);
 }
 
 // ---- generic device-wide exclusive scan (two launches, no inter-block waiting) ----------------------
@@ -315,20 +310,33 @@ void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, co
 }
 
 void launch_unique(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *sorted_keys,
-                   const BatchView &b, uint32_t *block_heads, uint32_t *u_copy) {
+                   const BatchView &b, const HeadChunks &heads, bool count_heads, uint32_t *u_copy) {
   if (!b.n) return;
-  const unsigned nb = unique_tiles(b.n);
-  if (kl.wide) {
-    hipLaunchKernelGGL(head_count<uint64_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
-                       block_heads);
-    hipLaunchKernelGGL(unique_emit<uint64_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint64_t *)sorted_keys, b.n,
-                       kl.id_bits, t.nrank, t.slot, block_heads, b, u_copy);
-  } else {
-    hipLaunchKernelGGL(head_count<uint32_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
-                       block_heads);
-    hipLaunchKernelGGL(unique_emit<uint32_t>, dim3(nb), dim3(kUBlock), 0, s, (const uint32_t *)sorted_keys, b.n,
-                       kl.id_bits, t.nrank, t.slot, block_heads, b, u_copy);
-  }
+  // the tile of the pass: that of the sort that left the head counts, or kUTile when they are counted here
+  const int items = count_heads ? kUItems : (int)(heads.chunk / kWave);
+  const uint32_t chunk = count_heads ? (uint32_t)kUTile : heads.chunk;
+  const unsigned nb = div_up(b.n, (size_t)items * kUBlock);
+#define EMIT(K, I)                                                                                                  \
+  hipLaunchKernelGGL((unique_emit<K, I>), dim3(nb), dim3(kUBlock), 0, s, (const K *)sorted_keys, b.n, kl.id_bits,   \
+                     t.nrank, t.slot, heads.inner, (const K *)heads.first, (const K *)heads.last, chunk, b, u_copy)
+#define EMIT_K(K)                                                                                          \
+  do {                                                                                                     \
+    if (count_heads)                                                                                       \
+      hipLaunchKernelGGL(head_count<K>, dim3(nb), dim3(kUBlock), 0, s, (const K *)sorted_keys, b.n, heads.inner, \
+                         (K *)heads.first, (K *)heads.last);                                              \
+    switch (items) {                                                                                       \
+      case 2: EMIT(K, 2); break;                                                                           \
+      case 4: EMIT(K, 4); break;                                                                           \
+      case 8: EMIT(K, 8); break;                                                                           \
+      case 13: EMIT(K, 13); break;                                                                         \
+      case 16: EMIT(K, 16); break;                                                                         \
+      default: throw Error("hetuCTR: internal: no unique pass for this tile shape");                       \
+    }                                                                                                      \
+  } while (0)
+  if (kl.wide) EMIT_K(uint64_t);
+  else EMIT_K(uint32_t);
+#undef EMIT_K
+#undef EMIT
   HCTR_HIP(hipGetLastError());
 }
 
@@ -340,7 +348,7 @@ void launch_idx_map(hipStream_t s, const BatchView &b) {
 
 void launch_list_long_runs(hipStream_t s, const BatchView &b) { // the class counters were zeroed by make_keys
   if (!b.n) return;
-  hipLaunchKernelGGL(list_long_runs, dim3(div_up(b.n, kBlock)), dim3(kBlock), 0, s, b);
+  hipLaunchKernelGGL(list_long_runs, dim3(div_up(b.n, kRunListBlock)), dim3(kRunListBlock), 0, s, b);
   HCTR_HIP(hipGetLastError());
 }
 

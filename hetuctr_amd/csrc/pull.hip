@@ -4,11 +4,13 @@
 // Reference: csrc/core/generate_query.cu:91-106, csrc/core/handle_query.cu:7-116,
 // csrc/core/writeback.cu:8-56.
 #include "kernels.h"
+#include "run_lists.h"
 
 namespace hctr {
 namespace {
 
 constexpr int kBlock = 256;
+static_assert(kBlock == kRunListBlock, "the gather's blocks list runs chunk by chunk");
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 template <int VEC> struct RowVec;
@@ -410,6 +412,10 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
   const uint32_t n = c.n, W = t.width;
+  if (blockIdx.x < a.list_chunks) { // the batch's run lists for its push one step later, before the block's own rows
+    __shared__ uint32_t cnt[kRunLists], base[kRunLists];
+    for (uint32_t chunk = blockIdx.x; chunk < a.list_chunks; chunk += gridDim.x) list_runs_chunk(c, chunk, cnt, base);
+  }
   const uint32_t j0 = (blockIdx.x * kGroups + threadIdx.x / LPR) * kRows;
   if (j0 >= n) return;
   const uint32_t gl = threadIdx.x % LPR;
@@ -450,6 +456,10 @@ __global__ __launch_bounds__(kBlock) void gather_pooled(TableView t, BatchView c
                                                         uint32_t n_bags) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
+  if (blockIdx.x < a.list_chunks) { // the batch's run lists, as in gather
+    __shared__ uint32_t cnt[kRunLists], base[kRunLists];
+    for (uint32_t chunk = blockIdx.x; chunk < a.list_chunks; chunk += gridDim.x) list_runs_chunk(c, chunk, cnt, base);
+  }
   const uint32_t b = blockIdx.x * kGroups + threadIdx.x / LPR;
   if (b >= n_bags) return;
   const uint32_t gl = threadIdx.x % LPR, W = t.width;

@@ -27,11 +27,11 @@ constexpr int kSortMaxBins = 1 << kSortMaxDigitBits;
 #endif
 constexpr int kSortItemsSmall = HCTR_SORT_ITEMS_SMALL, kSortItemsDefault = HCTR_SORT_ITEMS_DEFAULT, kSortItemsLarge = HCTR_SORT_ITEMS_LARGE;
 constexpr size_t kSortSmallUpTo = (size_t)1 << 17, kSortLargeFrom = (size_t)1 << 20;
-inline int sort_items(size_t n) {
+constexpr inline int sort_items(size_t n) {
   return n <= kSortSmallUpTo ? kSortItemsSmall : (n >= kSortLargeFrom ? kSortItemsLarge : kSortItemsDefault);
 }
-inline size_t sort_tile(size_t n) { return (size_t)kSortBlock * sort_items(n); }
-inline size_t sort_tiles(size_t n) { return (n + sort_tile(n) - 1) / sort_tile(n); }
+constexpr inline size_t sort_tile(size_t n) { return (size_t)kSortBlock * sort_items(n); }
+constexpr inline size_t sort_tiles(size_t n) { return (n + sort_tile(n) - 1) / sort_tile(n); }
 // words of scratch a sort of n keys needs: per tile and bin the count of the digit in the earlier tiles (of its piece of
 // the scan), then the total of every bin (per piece).  Not monotonic in n (the tile grows with it): size the scratch for the n that is sorted.
 // An input of many tiles has its count columns scanned in up to kScanMaxChunks pieces of at least kScanChunkRows rows,
@@ -41,11 +41,11 @@ inline size_t sort_tiles(size_t n) { return (n + sort_tile(n) - 1) / sort_tile(n
 #define HCTR_SCAN_MAX_CHUNKS 16
 #endif
 constexpr uint32_t kScanMaxChunks = HCTR_SCAN_MAX_CHUNKS, kScanChunkRows = 256;
-inline uint32_t scan_chunks(size_t tiles) {
+constexpr inline uint32_t scan_chunks(size_t tiles) {
   const size_t c = tiles / kScanChunkRows;
   return c < 2 ? 1u : (c > kScanMaxChunks ? kScanMaxChunks : (uint32_t)c);
 }
-inline size_t sort_scratch_words(size_t n) { return (sort_tiles(n) + scan_chunks(sort_tiles(n))) * (size_t)kSortMaxBins; }
+constexpr inline size_t sort_scratch_words(size_t n) { return (sort_tiles(n) + scan_chunks(sort_tiles(n))) * (size_t)kSortMaxBins; }
 // the most words any input of up to n_max keys needs
 inline size_t sort_scratch_words_upto(size_t n_max) {
   size_t w = sort_scratch_words(n_max);
@@ -68,7 +68,7 @@ struct SortScratch {
   size_t n_cap = 0;            // the n they were sized for
 };
 // tiles of the scan / unique kernels of the preprocess (256 threads x 8 items), whatever the sort tile is
-inline size_t scan_blocks(size_t n) { return (n + 2047) / 2048; }
+constexpr inline size_t scan_blocks(size_t n) { return (n + 2047) / 2048; }
 
 // digit width of the first pass for a key of `bits` bits (the passes split the bits evenly)
 inline int sort_first_digit_bits(int bits) {

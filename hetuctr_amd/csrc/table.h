@@ -10,6 +10,7 @@
 #include "../../include/hetuctr_hip.h"
 #include "kernels.h"
 #include "radix_sort.h"
+#include "tile_sort.h"
 
 namespace hctr {
 
@@ -55,6 +56,11 @@ struct Batch {
   bool idx_map_valid = false;
   bool cleared = false; // the device side reads as an empty batch (U = 0, no buckets, no runs) since clear()
   bool planned = false; // the push plan (need, prefix, push_cnt) has been computed for the batch as it stands
+  bool lists_ready = true;  // the run lists of the batch's push have been built (or the batch is empty)
+  bool tile_sorted = false; // indexed by the tile-sorted passes (tile_sort.h)
+  bool keys_made = false;   // comp holds the batch's sort keys (a kernel of its own made them); else the first launch
+                            // of the tile-sorted passes read the ids itself and no copy in batch order exists: the ids
+                            // of the batch are read back through the index when somebody asks for them
   // comp: the batch's sort keys in batch order (id and owner of every position); staged: ids that arrived in
   // pageable host memory, on their way to the key kernel
   DeviceBuf comp, staged, sorted_arg, rank_sorted, idx_map, ukey, run_start, uoff, bucket_lo, dU, long_list, dnlong, med_list;
@@ -86,12 +92,21 @@ struct HostMirror {
 
 class Group;
 
-// launches of the sort that a deferred preprocess of a single shard enqueues itself: the column scan and the scatter
-// of the first pass and the count of the second (the first count comes from the key kernel)
+// launches of the sort that a deferred preprocess enqueues itself: the column scan and the scatter of the first pass
+// and the count of the second (the first count comes from the key kernel); with the tile-sorted passes, the first of
+// the launches that follow the key kernel
 #ifndef HCTR_EARLY_SORT_STEPS
 #define HCTR_EARLY_SORT_STEPS 4
 #endif
-constexpr int kEarlySortSteps = HCTR_EARLY_SORT_STEPS;
+#ifndef HCTR_EARLY_TILE_PASSES
+#define HCTR_EARLY_TILE_PASSES 1
+#endif
+constexpr int kEarlySortSteps = HCTR_EARLY_SORT_STEPS, kEarlyTilePasses = HCTR_EARLY_TILE_PASSES;
+// from this many keys on, a preprocess that returns early has its ids read by a kernel that only makes the sort keys
+#ifndef HCTR_KEYS_FIRST_FROM
+#define HCTR_KEYS_FIRST_FROM (1u << 20)
+#endif
+constexpr uint32_t kKeysFirstFrom = HCTR_KEYS_FIRST_FROM;
 
 // stages whose device time can be measured separately (HIP events on the group's stream)
 enum Stage { S_KEYS = 0, S_SORT, S_UNIQUE, S_PLAN, S_PUSH, S_QUERY, S_EXCHANGE, S_OWNER, S_REFRESH, S_GATHER, S_COUNT };
@@ -122,6 +137,8 @@ class Shard {
   // sort, unique, run lists of the ingested batch; u_out: where the number of unique keys goes besides the batch's
   // own device word (default: the device block that is read back after the call)
   void index_batch(uint32_t *u_out = nullptr, int part = 0);
+  TileSortBuffers tile_sort_buffers() const; // the index scratch as the tile-sorted passes take it
+  bool force_counting_sort = false;          // HETUCTR_TILE_SORT=0: every batch through the three-launch passes
   void plan_batch(Batch &b);  // enqueues the push plan of b; its counts reach the host when the stream has run it
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
@@ -147,11 +164,11 @@ class Shard {
   bool prev_active = false; // false: inference step or no previous batch, nothing is pushed
   DeviceBuf root, slot, emb, ver, pend, upd, store_ids;
   // scratch shared by the stages
-  DeviceBuf ktmp0, ktmp1, vtmp0, vtmp1, sortws, block_sums, dstat, stats;
+  DeviceBuf ktmp0, ktmp1, vtmp0, vtmp1, sortws, block_sums, headws, dstat, stats;
   // where the index stages of the current batch find their scratch: the buffers above or pieces of the static array
   struct ScratchPtrs {
     void *ktmp0 = nullptr, *ktmp1 = nullptr;
-    uint32_t *vtmp0 = nullptr, *vtmp1 = nullptr, *sortws = nullptr, *block_sums = nullptr;
+    uint32_t *vtmp0 = nullptr, *vtmp1 = nullptr, *sortws = nullptr, *block_sums = nullptr, *headws = nullptr;
   } sp;
   DeviceBuf plan_sums, query_sums; // query_sums: flags per tile of received queries // plan_sums: scan scratch of the push plan (the index has block_sums to itself)
   DevStat *dst_ = nullptr; // == dstat.p
@@ -178,11 +195,35 @@ class Shard {
 };
 
 // The entry point that allocates nothing takes batches of up to kNoAllocMaxKeys keys; kNoAllocScratchBytes is what
-// the index of such a batch needs with 64-bit sort keys (sort ping-pong buffers, per-tile digit counts, scan sums).
+// the index of such a batch needs with 64-bit sort keys (sort ping-pong buffers, per-tile digit tables, scan sums, head
+// counts per chunk), every piece rounded up to 256 bytes.
 constexpr size_t kNoAllocMaxKeys = 262144;
-size_t index_scratch_bytes(uint32_t n, bool wide);
-constexpr size_t kNoAllocScratchBytes = 2 * (kNoAllocMaxKeys * 8) + 2 * (kNoAllocMaxKeys * 4) +
-                                        (kNoAllocMaxKeys / (kSortBlock * kSortItemsSmall) + 2) * kSortMaxBins * 4 + 4096;
+constexpr size_t index_scratch_round(size_t b) { return (b + 255) / 256 * 256; }
+// words of digit tables either sort of a batch of n keys needs
+constexpr inline size_t index_table_words(size_t n) {
+  const size_t a = sort_scratch_words(n), b = tile_sort_fits(n) ? tile_sort_table_words(n) : 0;
+  return a > b ? a : b;
+}
+// bytes of index scratch a batch of n keys needs (n >= 1)
+constexpr inline size_t index_scratch_bytes(uint32_t n, bool wide) {
+  const size_t m = n < 1 ? 1 : n, ks = wide ? 8 : 4;
+  return 2 * index_scratch_round(m * ks) + 2 * index_scratch_round(m * 4) + index_scratch_round(index_table_words(m) * 4) +
+         index_scratch_round((scan_blocks(m) + 2) * 4) + index_scratch_round(head_chunk_words(m) * 4);
+}
+// An upper bound of index_scratch_bytes over all n <= kNoAllocMaxKeys that needs no loop: the tables of the smallest
+// tile shape (or of the most tiles the tile-sorted passes take) and the head counts of the smallest chunk at the largest n.
+constexpr size_t kNoAllocScratchBytes =
+    2 * (kNoAllocMaxKeys * 8) + 2 * (kNoAllocMaxKeys * 4) +
+    (kNoAllocMaxKeys / (kSortBlock * kSortItemsSmall) + 8) * kSortMaxBins * 4 + (kNoAllocMaxKeys / 2048 + 3) * 4 +
+    (kNoAllocMaxKeys / 128 + 1) * 5 * 4 + 64 + 8 * 256;
+static_assert((kTileSortMaxTiles + 7) / 8 * 8 <= kNoAllocMaxKeys / (kSortBlock * kSortItemsSmall) + 8, "tables of the tile-sorted passes");
+// the sizes where the tile shape of a sort changes, and the largest batch: changed tile constants fail here
+static_assert(index_scratch_bytes((uint32_t)kSortSmallUpTo, true) <= kNoAllocScratchBytes &&
+                  index_scratch_bytes((uint32_t)kSortSmallUpTo + 1, true) <= kNoAllocScratchBytes &&
+                  index_scratch_bytes((uint32_t)(2 * kTileSortMaxTiles * kSortBlock), true) <= kNoAllocScratchBytes &&
+                  index_scratch_bytes((uint32_t)(2 * kTileSortMaxTiles * kSortBlock) + 1, true) <= kNoAllocScratchBytes &&
+                  index_scratch_bytes((uint32_t)kNoAllocMaxKeys, true) <= kNoAllocScratchBytes,
+              "the static scratch of the entry point that allocates nothing is too small");
 
 // All shards of one loopback group live in one process on one device and share one stream.  The group
 // carries the collective calls: every shard's thread deposits its arguments, the last one to arrive runs the

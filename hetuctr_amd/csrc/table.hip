@@ -124,6 +124,10 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   kl.wide = kl.total_bits > 32;
   if (const char *f = getenv("HETUCTR_FORCE_WIDE_KEYS")) // exercises the 64-bit sort-key path on small tables
     if (f[0] == '1') kl.wide = true;
+  if (const char *f = getenv("HETUCTR_TILE_SORT")) // 0: every batch takes the three-launch passes of radix_sort.h
+    if (f[0] == '0') force_counting_sort = true;
+  if (const char *f = getenv("HETUCTR_TILE_DIGIT_BITS")) // many narrow passes exercise the hand-over between the launches
+    kl.max_digit_bits = atoi(f);
 
   // ---- host-side checks and the resident layout: cached ids first, then owned ids, order kept
   // (thrust::stable_partition at table_initialize.cu:81)
@@ -219,39 +223,35 @@ void Shard::reserve_batch_scratch(uint32_t n) {
   ktmp1.reserve(m * ks);
   vtmp0.reserve(m * 4);
   vtmp1.reserve(m * 4);
-  sortws.reserve(sort_scratch_words(m) * 4);
+  sortws.reserve(index_table_words(m) * 4);
   block_sums.reserve((scan_blocks(m) + 2) * 4);
+  headws.reserve(head_chunk_words(m) * 4);
   sp.ktmp0 = ktmp0.p;
   sp.ktmp1 = ktmp1.p;
   sp.vtmp0 = vtmp0.as<uint32_t>();
   sp.vtmp1 = vtmp1.as<uint32_t>();
   sp.sortws = sortws.as<uint32_t>();
   sp.block_sums = block_sums.as<uint32_t>();
+  sp.headws = headws.as<uint32_t>();
 }
 
-// bytes of index scratch a batch of n keys needs, every piece a multiple of 256 bytes
-size_t index_scratch_bytes(uint32_t n, bool wide) {
-  const size_t m = std::max<uint32_t>(n, 1), ks = wide ? 8 : 4;
-  auto up = [](size_t b) { return (b + 255) / 256 * 256; };
-  return 2 * up(m * ks) + 2 * up(m * 4) + up(sort_scratch_words(m) * 4) + up((scan_blocks(m) + 2) * 4);
-}
-
-// the same pieces cut out of one caller-provided area (the static array) instead of the shard's own buffers
+// the same pieces cut out of one caller-provided area (the static array) instead of the shard's own buffers, in the
+// order and with the rounding of index_scratch_bytes
 void Shard::use_scratch_area(void *area, uint32_t n) {
   const size_t m = std::max<uint32_t>(n, 1), ks = kl.wide ? 8 : 4;
-  auto up = [](size_t b) { return (b + 255) / 256 * 256; };
   unsigned char *p = (unsigned char *)area;
   auto take = [&](size_t bytes) {
     void *r = p;
-    p += up(bytes);
+    p += index_scratch_round(bytes);
     return r;
   };
   sp.ktmp0 = take(m * ks);
   sp.ktmp1 = take(m * ks);
   sp.vtmp0 = (uint32_t *)take(m * 4);
   sp.vtmp1 = (uint32_t *)take(m * 4);
-  sp.sortws = (uint32_t *)take(sort_scratch_words(m) * 4);
+  sp.sortws = (uint32_t *)take(index_table_words(m) * 4);
   sp.block_sums = (uint32_t *)take((scan_blocks(m) + 2) * 4);
+  sp.headws = (uint32_t *)take(head_chunk_words(m) * 4);
 }
 
 // csrc/core/preprocess.cu:92-141
@@ -263,6 +263,7 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
   cur.U = 0;
   cur.idx_map_valid = false;
   cur.planned = false;
+  cur.lists_ready = n == 0;
   if (!scratch_area) cur.reserve(cur.n, cfg.nrank, kl.wide); // else: the caller has checked that the buffers hold n keys
   if (n == 0) { // :93-95
     cur.clear(s, cfg.nrank);
@@ -285,41 +286,71 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
         cur.staged.reserve(n * sizeof(index_t));
         HCTR_HIP(hipMemcpyAsync(cur.staged.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
       }
-      launch_make_keys(s, tv, kl, visible ? (const index_t *)keys : (const index_t *)cur.staged.as<index_t>(), cur.n,
-                       cur.comp.p, flag ? flag : err_ptr(), cur.dnlong.as<uint32_t>(), sp.sortws);
+      const index_t *ids = visible ? (const index_t *)keys : (const index_t *)cur.staged.as<index_t>();
+      cur.tile_sorted = tile_sort_fits(cur.n) && !force_counting_sort;
+      // A call that returns as soon as the ids are read (flag: where it looks for a bad id) gets them read by the
+      // lightest kernel there is when the batch is large: the sort keys alone.  Sorting a tile as well keeps the
+      // caller -- whose next call starts the gradient push -- waiting several microseconds longer.
+      cur.keys_made = !cur.tile_sorted || (flag != nullptr && cur.n >= kKeysFirstFrom);
+      if (!cur.keys_made)
+        launch_tile_sort_keys(s, tv, kl, ids, nullptr, cur.n, tile_sort_buffers(), flag ? flag : err_ptr(),
+                              cur.dnlong.as<uint32_t>());
+      else
+        launch_make_keys(s, tv, kl, ids, cur.n, cur.comp.p, flag ? flag : err_ptr(), cur.dnlong.as<uint32_t>(),
+                         cur.tile_sorted ? nullptr : sp.sortws);
     }
   }
 }
 
+TileSortBuffers Shard::tile_sort_buffers() const {
+  TileSortBuffers b;
+  b.keys[0] = sp.ktmp0;
+  b.keys[1] = sp.ktmp1;
+  b.vals[0] = sp.vtmp0;
+  b.vals[1] = sp.vtmp1;
+  b.tables = sp.sortws;
+  return b;
+}
+
 void Shard::index_batch(uint32_t *u_out, int part) {
   hipStream_t s = group->stream;
-  // part 1: the first kEarlySortSteps launches of the sort; part 2: everything after them; 0: all of it
-  const int from = part == 2 ? kEarlySortSteps : 0, to = part == 1 ? kEarlySortSteps : (1 << 30);
+  // part 1: the first launches of the sort; part 2: everything after them; 0: all of it
   if (cur.n != 0) {
-    SortScratch sc;
-    sc.words = sp.sortws;
-    sc.n_cap = cur.n;
+    // head counts per chunk: one wave's share of a sort tile with the tile-sorted passes, else a tile of the unique pass
+    const HeadChunks heads = head_chunks_in(sp.headws, cur.n, kl.wide, cur.tile_sorted ? (uint32_t)tile_items(cur.n) * kWave : 4096u);
     const void *sorted_keys = nullptr;
     {
       StageScope sort_scope(*group, S_SORT);
-      if (kl.wide) {
-        const uint64_t *sk;
-        radix_sort_positions<uint64_t>(s, cur.comp.as<uint64_t>(), cur.n, kl.total_bits, (uint64_t *)sp.ktmp0,
-                                       (uint64_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
-                                       cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
-        sorted_keys = sk;
+      if (cur.tile_sorted) {
+        if (cur.keys_made && part != 2) // the sort's first launch, from the keys the call made before it returned
+          launch_tile_sort_keys(s, tv, kl, nullptr, cur.comp.p, cur.n, tile_sort_buffers(), nullptr, nullptr);
+        const int from = part == 2 ? 1 + kEarlyTilePasses : 1, to = part == 1 ? 1 + kEarlyTilePasses : (1 << 30);
+        launch_tile_sort_passes(s, kl, cur.n, tile_sort_buffers(), cur.sorted_arg.as<uint32_t>(), heads, &sorted_keys,
+                                from, to);
       } else {
-        const uint32_t *sk;
-        radix_sort_positions<uint32_t>(s, cur.comp.as<uint32_t>(), cur.n, kl.total_bits, (uint32_t *)sp.ktmp0,
-                                       (uint32_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
-                                       cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
-        sorted_keys = sk;
+        const int from = part == 2 ? kEarlySortSteps : 0, to = part == 1 ? kEarlySortSteps : (1 << 30);
+        SortScratch sc;
+        sc.words = sp.sortws;
+        sc.n_cap = cur.n;
+        if (kl.wide) {
+          const uint64_t *sk;
+          radix_sort_positions<uint64_t>(s, cur.comp.as<uint64_t>(), cur.n, kl.total_bits, (uint64_t *)sp.ktmp0,
+                                         (uint64_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
+                                         cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
+          sorted_keys = sk;
+        } else {
+          const uint32_t *sk;
+          radix_sort_positions<uint32_t>(s, cur.comp.as<uint32_t>(), cur.n, kl.total_bits, (uint32_t *)sp.ktmp0,
+                                         (uint32_t *)sp.ktmp1, sp.vtmp0, sp.vtmp1,
+                                         cur.sorted_arg.as<uint32_t>(), sc, &sk, true, from, to);
+          sorted_keys = sk;
+        }
       }
     }
     if (part == 1) return;
     StageScope st(*group, S_UNIQUE);
-    launch_unique(s, tv, kl, sorted_keys, cur.view(), sp.block_sums, u_out ? u_out : &dst_->U);
-    launch_list_long_runs(s, cur.view());
+    launch_unique(s, tv, kl, sorted_keys, cur.view(), heads, !cur.tile_sorted, u_out ? u_out : &dst_->U);
+    // the run lists follow in the gather of the step, or before the batch's push if no gather came (lists_ready)
   }
   if (part == 1) return;
   if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt, mirror->st.send_cnt, &mirror->st.U);
@@ -424,6 +455,10 @@ void Shard::generate_gradient(const uint32_t *delta) {
   a.g_idx = nullptr;
   a.g_cnt = nullptr;
   a.g_val = nullptr;
+  if (!prev.lists_ready) { // no gather has seen this batch (a second preprocess came first, or a call without output)
+    launch_list_long_runs(s, prev.view());
+    prev.lists_ready = true;
+  }
   StageScope st(*group, S_PUSH);
   if (cfg.nrank > 1) {
     // the pushed rows go straight into the group's receive area: plan position -> position there
@@ -522,6 +557,7 @@ void Shard::write_back(float *dst, uint32_t bag) {
   a.in_ver = nullptr;
   a.in_val = nullptr;
   a.dst = dst;
+  a.list_chunks = 0;
   // The gathered rows are not read again by this library: streamed past the caches they leave the table rows of the
   // batch there for the push that updates them next.  The one case where that loses is a batch of (almost) all
   // distinct keys, where the gather reads as many rows as it writes; the previous batch is the predictor.
@@ -542,6 +578,10 @@ void Shard::write_back(float *dst, uint32_t bag) {
   }
   if (dst != nullptr) {
     StageScope st(*group, S_GATHER);
+    if (!cur.lists_ready && cur.n != 0) { // the first blocks of the gather build the batch's run lists on their way
+      a.list_chunks = run_list_chunks(cur.n);
+      cur.lists_ready = true;
+    }
     if (bag > 1) { // sum-pooled bags: in batch order, through the inverse index
       HCTR_CHECK(cur.n % bag == 0, "pooled pull: the batch is not a whole number of bags");
       if (!cur.idx_map_valid) {
@@ -631,7 +671,11 @@ size_t Shard::fetch(int which, void *out, size_t cap) {
     case HCTR_F_STORE_IDS: return put64(download<index_t>(store_ids.p, tv.n_stored), tv.n_stored, out, cap);
     case HCTR_F_KEYS: { // the ids of the batch as its sort keys hold them (an id outside the table reads as 0)
       std::vector<uint64_t> k(cur.n);
-      if (kl.wide) {
+      if (!cur.keys_made) { // no copy in batch order was kept: position sorted_arg[j] holds the key of rank_sorted[j]
+        const auto uk = ukeys(cur);
+        const auto pos = download<uint32_t>(cur.sorted_arg.p, cur.n), rk = download<uint32_t>(cur.rank_sorted.p, cur.n);
+        for (size_t j = 0; j < cur.n; j++) k[pos[j]] = uk[rk[j]] & id_mask;
+      } else if (kl.wide) {
         auto h = download<uint64_t>(cur.comp.p, cur.n);
         for (size_t i = 0; i < cur.n; i++) k[i] = h[i] & id_mask;
       } else {

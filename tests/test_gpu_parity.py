@@ -329,28 +329,64 @@ def test_repeated_and_changing_batch_sizes():
     p.close()
 
 
+@pytest.mark.parametrize("tile_sorted", [True, False])
 @pytest.mark.parametrize("nrank", [1, 2])
-def test_batch_sizes_where_the_sort_changes_shape(nrank):
-    # 1024-key tiles up to 2^17 keys (up to 64 of them without scan launches), 4096-key tiles above: the sizes on both
-    # sides of every switch, one after the other on one table (the scratch of one size is reused by the next)
-    say("sort shapes, shards", nrank)
+def test_batch_sizes_where_the_sort_changes_shape(nrank, tile_sorted, monkeypatch):
+    # Both sorts of the index.  The tile-sorted passes: 2, 4, 8, 13 keys per thread (tiles of 1024 ... 6656 keys, at most
+    # 256 tiles) up to 1.5 M keys, the first launch from ids or -- from 2^20 keys on, when preprocess returns early --
+    # from keys made by a kernel of its own.  The three-launch passes (all sizes when HETUCTR_TILE_SORT=0, else above
+    # 1.5 M keys): 1024-key tiles up to 2^17 keys (up to 64 of them without scan launches), 4096- and 8192-key tiles
+    # above.  The sizes on both sides of every switch, one after the other on one table (the scratch of one size is
+    # reused by the next).
+    if not tile_sorted:
+        monkeypatch.setenv("HETUCTR_TILE_SORT", "0")
+    say("sort shapes, shards", nrank, "tile-sorted passes" if tile_sorted else "three-launch passes")
     rng = np.random.default_rng(35 + nrank)
     length, width = 3_000_000, 4                           # 22-bit ids (+ 1 bit of rank): three digit widths in a sort
     root = rng.integers(0, nrank, size=length).astype(np.uint8)
     storage = [np.flatnonzero(root == r).astype(np.int64) for r in range(nrank)]
     p = Pair(nrank, length, width, root, storage, init=("Zero", 0.0, 0.0), lr=0.5)
-    sizes = [1024, 1025, 65536, 65537, 65536 + 1024, 131072, 131073, 1023, 140_000, 64 * 1024 - 1]
+    sizes = [1024, 1025, 65536, 65537, 65536 + 1024, 131072, 131073, 1023, 140_000, 64 * 1024 - 1,
+             262144, 262145, 524288, 524289, 5000, 1048575, 1048576, 1048577, 3 << 19, (3 << 19) + 1, 2047]
     prev_n = [0] * nrank
     for step, n in enumerate(sizes):
         ns = [n if r == 0 else max(n // 3, 1) for r in range(nrank)]
         keys = [rng.integers(0, length, size=k).astype(np.int64) for k in ns]
         p.preprocess(keys, device_keys=True)
-        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.SIZES], "n %d" % n)
+        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.SIZES, capi.KEYS], "n %d" % n)
         out, ref = p.push_pull([rng.normal(0, 1e-2, size=(k, width)).astype(np.float32) for k in prev_n])
         for r in range(nrank):
             assert_close(out[r], ref[r], 1e-5, "dst n %d rank %d" % (n, r))
         prev_n = ns
     p.compare_state(1e-5, "end")
+    p.close()
+
+
+@pytest.mark.parametrize("bits,nrank,digit", [(3, 1, 0), (10, 1, 0), (11, 1, 0), (20, 1, 0), (21, 1, 0), (24, 2, 0),
+                                              (22, 1, 3), (23, 2, 5)])
+def test_sort_passes_for_every_key_width(bits, nrank, digit, monkeypatch):
+    # one, two and three digit passes with digits of 3 to 10 bits, and (digit: a narrower widest digit) eight and five
+    # passes; skewed keys, so that some blocks of a pass see a single digit value and others hundreds; preprocess
+    # returns early (first launch beside the call) and, every other step, only when all is done
+    if digit:
+        monkeypatch.setenv("HETUCTR_TILE_DIGIT_BITS", str(digit))
+    say("id bits", bits, "shards", nrank, "digits of at most", digit or 10, "bits")
+    rng = np.random.default_rng(900 + bits)
+    length, width = (1 << bits) - (3 if bits > 2 else 0), 1
+    root = rng.integers(0, nrank, size=length).astype(np.uint8)
+    storage = [np.flatnonzero(root == r).astype(np.int64) for r in range(nrank)]
+    p = Pair(nrank, length, width, root, storage, init=("Zero", 0.0, 0.0), lr=1.0)
+    prev_n = [0] * nrank
+    for step, n in enumerate([100_000, 300_000, 7, 40_000]):
+        p.tables[0].defer_index(step % 2 == 0)
+        # Zipf ranks spread over the id range by a fixed odd multiplier: hot ids everywhere, every digit in use
+        keys = [(np.minimum(rng.zipf(1.1, size=n), length) - 1) * 2654435761 % length for _ in range(nrank)]
+        p.preprocess(keys, device_keys=True)
+        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.IDX_MAP, capi.ROOT, capi.SIZES, capi.KEYS], "n %d" % n)
+        out, ref = p.push_pull([rng.integers(-2, 3, size=(k, width)).astype(np.float32) for k in prev_n])
+        for r in range(nrank):
+            assert_close(out[r], ref[r], 1e-5, "dst n %d rank %d" % (n, r))
+        prev_n = [n] * nrank
     p.close()
 
 
@@ -392,7 +428,7 @@ def test_64_bit_sort_keys_at_every_sort_shape(nrank, monkeypatch):
     storage = [np.flatnonzero(root == r).astype(np.int64) for r in range(nrank)]
     p = Pair(nrank, length, width, root, storage, init=("Zero", 0.0, 0.0), lr=0.5)
     prev_n = [0] * nrank
-    for n in [3000, 70_000, 200_000, 4_300_000, 1_100_000]:
+    for n in [3000, 70_000, 200_000, 4_300_000, 1_100_000, 300_000, 600_000, 1_572_864]:
         ns = [n if r == 0 else max(n // 5, 1) for r in range(nrank)]
         keys = [rng.integers(0, length, size=k).astype(np.int64) for k in ns]
         p.preprocess(keys, device_keys=True)
