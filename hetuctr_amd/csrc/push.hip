@@ -410,14 +410,16 @@ __device__ __forceinline__ void store_transposed(float *, uint32_t, const float 
 // a value that is the same in every lane, moved to a scalar register
 __device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
-__device__ __forceinline__ uint32_t bundle_runs(int cls) { // runs per bundle: classes halve in length
-  return cls <= 6 ? 1u : min(1u << (cls - 6), (uint32_t)kTable); // one run of 2048 or more, 2 of 1024.., 4, 8, 16
+// runs per bundle: classes halve in length -- one run of 2048 or more, 2 of 1024.., 4, 8, 16; `shrink` halves that
+// (down to single runs) for batches with few long runs
+__device__ __forceinline__ uint32_t bundle_runs(int cls, uint32_t shrink) {
+  return cls <= 6 ? 1u : max(min(1u << (cls - 6), (uint32_t)kTable) >> shrink, 1u);
 }
 
 template <int VEC, typename K, int CSC, bool kPooled> // CSC: columns per slice if known at compile time, else 0
 __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const BatchView &p, const PushArgs &a,
-                                          float *lds, uint4 *table, uint32_t *shared, int c_lo, int c_hi,
-                                          uint32_t bidx, uint32_t nblk, uint32_t *counters) {
+                                          float *lds, uint4 *table, uint32_t *shared, float *row_stash, int c_lo,
+                                          int c_hi, uint32_t bidx, uint32_t nblk, uint32_t *counters) {
   typedef typename Vec<VEC>::T V;
   const uint32_t W = t.width;
   const uint32_t CS = CSC ? (uint32_t)CSC : min((uint32_t)kSlice, (W + VEC - 1) / VEC * VEC);
@@ -447,11 +449,18 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
   const uint32_t n_sl = (slices - lane_id + share - 1) / share; // slices lane_id, lane_id + share, ...
   const uint32_t group_blocks = (nblk - lane_id + share - 1) / share; // blocks drawing from this counter
   uint32_t cnt[kLongBuckets];
-  uint32_t nbundles = 0;
 #pragma unroll
-  for (int c = 0; c < kLongBuckets; c++) {
-    cnt[c] = (c >= c_lo && c < c_hi) ? uni(p.d_nlong[c]) : 0u;
-    nbundles += (cnt[c] + bundle_runs(c) - 1) / bundle_runs(c);
+  for (int c = 0; c < kLongBuckets; c++) cnt[c] = (c >= c_lo && c < c_hi) ? uni(p.d_nlong[c]) : 0u;
+  // A block streams a bundle at the pace its rows in flight allow (a few ns per occurrence), whatever the other
+  // blocks do: a small batch, whose long runs make fewer tickets than there are blocks to draw them, gets smaller
+  // bundles until every block has work or every bundle is a single run.  Every block computes the same value.
+  uint32_t shrink = 0, nbundles;
+  for (;;) {
+    nbundles = 0;
+#pragma unroll
+    for (int c = 0; c < kLongBuckets; c++) nbundles += (cnt[c] + bundle_runs(c, shrink) - 1) / bundle_runs(c, shrink);
+    if (shrink == 4 || nbundles * slices >= 2 * nblk) break;
+    shrink++;
   }
   if (!nbundles) return;
   const uint32_t tickets = nbundles * n_sl;
@@ -479,7 +488,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
     bool found = false;
 #pragma unroll
     for (int c = 0; c < kLongBuckets; c++) {
-      const uint32_t bs = bundle_runs(c), nb = (cnt[c] + bs - 1) / bs;
+      const uint32_t bs = bundle_runs(c, shrink), nb = (cnt[c] + bs - 1) / bs;
       if (!found) {
         if (bundle < nb) {
           found = true;
@@ -589,12 +598,24 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
       const bool col_ok = threadIdx.x < CS && mycol < W;
       const bool direct = t.nrank == 1; // every key is owned and resident; the version counters move elsewhere
       uint32_t slot = 0;
+      if (direct) {
+        // The table rows the sums are added to, for every run of the bundle at once and parked in LDS: requested
+        // run by run, each would arrive a memory round trip after its run had been summed (a run of a few hundred
+        // occurrences is summed in a fraction of one), and the loaders would wait behind the full ring meanwhile.
+        // This wait happens once per bundle, while the loaders' first rows are on their way.
+        float rows[kTable];
+#pragma unroll
+        for (int j = 0; j < kTable; j++) {
+          rows[j] = 0.f;
+          if ((uint32_t)j < J && col_ok) rows[j] = t.emb[(size_t)table[j].w * W + mycol];
+        }
+#pragma unroll
+        for (int j = 0; j < kTable; j++) row_stash[j * kWave + threadIdx.x] = rows[j];
+      }
       for (uint32_t j = 0; j < J; j++) {
         const uint4 m = table[j];
         const uint32_t L = m.z;
         const uint32_t nfull = L / CR, nch = (L + CR - 1) / CR;
-        float e = 0.f;
-        if (direct && col_ok) e = t.emb[(size_t)m.w * W + mycol]; // needed only after the last chunk
         float acc = 0.f; // the reference starts every sum from 0
         uint32_t c = 0;
         if (CSC) {
@@ -671,7 +692,7 @@ __device__ __forceinline__ void long_role(const TableView &t, int id_bits, const
         }
         if (col_ok) {
           const float scaled = acc * neg_lr;
-          if (direct) t.emb[(size_t)m.w * W + mycol] = e + scaled;
+          if (direct) t.emb[(size_t)m.w * W + mycol] = row_stash[j * kWave + threadIdx.x] + scaled;
           else apply_row<1, K>(t, id_bits, p, a, m.x, scaled, mycol);
         }
       }
@@ -694,18 +715,19 @@ __global__ __launch_bounds__(kPushBlock) __attribute__((amdgpu_waves_per_eu(HCTR
   __shared__ __align__(16) float lds[kRingWords > kStageWords ? kRingWords : kStageWords];
   __shared__ uint4 run_table[kTable];
   __shared__ uint32_t run_totals[3];
+  __shared__ float row_stash[kTable * kWave]; // long role: the table rows of a bundle's runs (one slice, one lane each)
   if (blockIdx.x < kLongBlocks) {
     // Every block first takes tickets of the longest runs, which are cut into narrower column slices so that more
     // blocks feed each of them (the blocks of a saturated memory system get equal shares of it, and a chain
     // advances with the share of the block that feeds it), then tickets of the other long runs.
     uint32_t *tk = p.d_nlong + kTicketBase;
     if (VEC == 4 && t.width % kSlice == 0) {
-      long_role<VEC, K, (VEC == 4 ? kGiantSlice : 0), kPooled>(t, id_bits, p, a, lds, run_table, run_totals, 0, kGiantClasses,
+      long_role<VEC, K, (VEC == 4 ? kGiantSlice : 0), kPooled>(t, id_bits, p, a, lds, run_table, run_totals, row_stash, 0, kGiantClasses,
                                                       blockIdx.x, kLongBlocks, tk);
-      long_role<VEC, K, (VEC == 4 ? kSlice : 0), kPooled>(t, id_bits, p, a, lds, run_table, run_totals, kGiantClasses, kLongBuckets,
+      long_role<VEC, K, (VEC == 4 ? kSlice : 0), kPooled>(t, id_bits, p, a, lds, run_table, run_totals, row_stash, kGiantClasses, kLongBuckets,
                                                  blockIdx.x, kLongBlocks, tk + kTicketLanes);
     } else {
-      long_role<VEC, K, 0, kPooled>(t, id_bits, p, a, lds, run_table, run_totals, 0, kLongBuckets, blockIdx.x, kLongBlocks, tk);
+      long_role<VEC, K, 0, kPooled>(t, id_bits, p, a, lds, run_table, run_totals, row_stash, 0, kLongBuckets, blockIdx.x, kLongBlocks, tk);
     }
   } else if (blockIdx.x < kLongBlocks + kMedBlocks) { // medium runs take long per block: they start early
     medium_role<VEC, LPR, K, kSingle, kPooled>(t, id_bits, p, a, (uint32_t *)lds, blockIdx.x - kLongBlocks, kMedBlocks);

@@ -138,7 +138,8 @@ class Shard {
   // own device word (default: the device block that is read back after the call)
   void index_batch(uint32_t *u_out = nullptr, int part = 0);
   TileSortBuffers tile_sort_buffers() const; // the index scratch as the tile-sorted passes take it
-  bool force_counting_sort = false;          // HETUCTR_TILE_SORT=0: every batch through the three-launch passes
+  int tile_sort_mode = 1;                    // HETUCTR_TILE_SORT: 0 no batch takes the tile-sorted passes, 1 those of up
+                                             // to kTileSortMaxKeys keys, 2 every batch whose tiles they can hold
   void plan_batch(Batch &b);  // enqueues the push plan of b; its counts reach the host when the stream has run it
   void enqueue_readback_preprocess();
   void finish_preprocess();                 // after the stream sync: mirrors -> host fields, error checks
@@ -201,7 +202,7 @@ constexpr size_t kNoAllocMaxKeys = 262144;
 constexpr size_t index_scratch_round(size_t b) { return (b + 255) / 256 * 256; }
 // words of digit tables either sort of a batch of n keys needs
 constexpr inline size_t index_table_words(size_t n) {
-  const size_t a = sort_scratch_words(n), b = tile_sort_fits(n) ? tile_sort_table_words(n) : 0;
+  const size_t a = sort_scratch_words(n), b = tile_sort_possible(n) ? tile_sort_table_words(n) : 0;
   return a > b ? a : b;
 }
 // bytes of index scratch a batch of n keys needs (n >= 1)

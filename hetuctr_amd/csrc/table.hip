@@ -124,8 +124,9 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   kl.wide = kl.total_bits > 32;
   if (const char *f = getenv("HETUCTR_FORCE_WIDE_KEYS")) // exercises the 64-bit sort-key path on small tables
     if (f[0] == '1') kl.wide = true;
-  if (const char *f = getenv("HETUCTR_TILE_SORT")) // 0: every batch takes the three-launch passes of radix_sort.h
-    if (f[0] == '0') force_counting_sort = true;
+  // which sort indexes a batch: 0 the three-launch passes of radix_sort.h always, 2 the tile-sorted passes whenever
+  // they can hold the batch (measurements of either sort at any size); default: tile_sort_fits()
+  if (const char *f = getenv("HETUCTR_TILE_SORT")) tile_sort_mode = f[0] == '0' ? 0 : (f[0] == '2' ? 2 : 1);
   if (const char *f = getenv("HETUCTR_TILE_DIGIT_BITS")) // many narrow passes exercise the hand-over between the launches
     kl.max_digit_bits = atoi(f);
 
@@ -287,7 +288,7 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
         HCTR_HIP(hipMemcpyAsync(cur.staged.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
       }
       const index_t *ids = visible ? (const index_t *)keys : (const index_t *)cur.staged.as<index_t>();
-      cur.tile_sorted = tile_sort_fits(cur.n) && !force_counting_sort;
+      cur.tile_sorted = tile_sort_mode == 2 ? tile_sort_possible(cur.n) : (tile_sort_mode == 1 && tile_sort_fits(cur.n));
       // A call that returns as soon as the ids are read (flag: where it looks for a bad id) gets them read by the
       // lightest kernel there is when the batch is large: the sort keys alone.  Sorting a tile as well keeps the
       // caller -- whose next call starts the gradient push -- waiting several microseconds longer.

@@ -46,9 +46,8 @@ constexpr inline size_t tile_count(size_t n) { return (n + tile_keys(n) - 1) / t
 #define HCTR_TILE_SORT_MAX_KEYS (3u << 19)
 #endif
 constexpr size_t kTileSortMaxKeys = HCTR_TILE_SORT_MAX_KEYS;
-constexpr inline bool tile_sort_fits(size_t n) {
-  return n != 0 && n <= kTileSortMaxKeys && tile_count(n) <= kTileSortMaxTiles;
-}
+constexpr inline bool tile_sort_possible(size_t n) { return n != 0 && tile_count(n) <= kTileSortMaxTiles; }
+constexpr inline bool tile_sort_fits(size_t n) { return n <= kTileSortMaxKeys && tile_sort_possible(n); }
 
 // Per chunk of sorted positions (one wave's share of a tile: tile_items(n) * 64 positions): how many positions of the
 // chunk other than its first hold another key than the position before, and the chunk's first and last key.

@@ -488,7 +488,7 @@ DigitPlan plan_digits(const KeyLayout &kl) {
 void launch_tile_sort_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *ids,
                            const void *made_keys, uint32_t n, const TileSortBuffers &b, uint32_t *err, uint32_t *nlong) {
   if (!n) return;
-  HCTR_CHECK(tile_sort_fits(n), "internal: batch too large for the tile-sorted passes");
+  HCTR_CHECK(tile_sort_possible(n), "internal: batch too large for the tile-sorted passes");
   const DigitPlan p = plan_digits(kl);
   const unsigned tiles = (unsigned)tile_count(n), pitch = (unsigned)tile_table_pitch(n);
   uint16_t *table0 = (uint16_t *)b.tables;
