@@ -14,15 +14,15 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIBDIR = os.path.join(HERE, "lib")
-HIP_SOURCES = ["radix_sort.hip", "tile_sort.hip", "preprocess.hip", "push.hip", "pull.hip", "init.hip", "table.hip", "checkpoint.hip", "loader.hip", "partition.hip", "c_api.hip"]
-HEADERS = ["common.h", "kernels.h", "radix_sort.h", "tile_sort.h", "run_lists.h", "table.h", "partition.h", os.path.join("..", "..", "include", "hetuctr_hip.h")]
+HIP_SOURCES = ["radix_sort.hip", "tile_sort.hip", "preprocess.hip", "push.hip", "pull.hip", "init.hip", "table.hip", "checkpoint.hip", "loader.hip", "partition.hip", "host_copy.hip", "c_api.hip"]
+HEADERS = ["common.h", "host_copy.h", "kernels.h", "radix_sort.h", "tile_sort.h", "run_lists.h", "table.h", "partition.h", os.path.join("..", "..", "include", "hetuctr_hip.h")]
 # packed-fp32 instruction selection is switched off for all device code; no fused multiply-add contraction, so
 # that "sum * -lr" then "row + that" rounds twice like the CPU restatement it is checked against (fused
 # operations are written explicitly where they are meant)
 HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # host code of the partitioner's sweeps: AVX2 (no fused multiply-add is formed: contraction is off above)
-EXTRA_FLAGS = {"partition.hip": ["-Xarch_host", "-march=x86-64-v3"]}
+EXTRA_FLAGS = {"partition.hip": ["-Xarch_host", "-march=x86-64-v3"], "host_copy.hip": ["-Xarch_host", "-march=x86-64-v3"]}
 LIB = os.path.join(LIBDIR, "libhetuctr_hip.so")
 PYMOD = os.path.join(LIBDIR, "hetuCTR" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 

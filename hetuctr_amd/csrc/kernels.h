@@ -77,8 +77,10 @@ struct TableView {
 // ids -> sort keys; flags ids outside [0, id_max) in *err (and sorts them as id 0)
 // comp_keys is the batch's copy of the ids as well (the reference's d_idx); nlong (optional) is zeroed;
 // sort_counts: the sort's scratch, which receives the per-tile counts of the first pass' digit
+// ids32: `keys` points to 32-bit ids (narrowed on their way from pageable host memory; one that did not fit is
+// 0xffffffff, which the range check flags like the id it stands for)
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err, uint32_t *nlong, uint32_t *sort_counts);
+                      void *comp_keys, uint32_t *err, uint32_t *nlong, uint32_t *sort_counts, bool ids32 = false);
 // sorted keys -> everything per unique key + inverse index.  heads: the head counts per chunk of sorted positions that
 // the last launch of the tile-sorted passes left (count_heads false), or storage for them (count_heads true: a launch
 // of its own counts them first, one chunk per tile of the unique pass).

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
                                                          int id_bits, int nrank, const worker_t *__restrict__ root,
                                                          K *__restrict__ comp, uint32_t *__restrict__ err,
                                                          uint32_t *__restrict__ nlong, int dbits,
-                                                         uint32_t *__restrict__ counts) {
+                                                         uint32_t *__restrict__ counts, bool ids32) {
   __shared__ uint32_t h[kSortMaxBins];
   const uint32_t nb = 1u << dbits, mask = nb - 1;
   if (counts)
@@ -35,7 +35,8 @@ __global__ __launch_bounds__(kSortBlock) void make_keys(const index_t *__restric
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = base + k * kSortBlock + threadIdx.x;
-    id[k] = i < n ? (uint64_t)load_once(&keys[i]) : 0; // the caller's ids are read here and nowhere else
+    // the caller's ids are read here and nowhere else (ids32: as narrowed on their way from pageable host memory)
+    id[k] = i >= n ? 0 : ids32 ? (uint64_t)load_once(&((const uint32_t *)keys)[i]) : (uint64_t)load_once(&keys[i]);
   }
   __syncthreads();
   bool bad = false;
@@ -291,7 +292,8 @@ __global__ void bucket_sizes(BatchView b, int nrank, uint64_t *__restrict__ cnt_
 } // namespace
 
 void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *keys, uint32_t n,
-                      void *comp_keys, uint32_t *err, uint32_t *nlong, uint32_t *sort_counts) {
+                      void *comp_keys, uint32_t *err, uint32_t *nlong, uint32_t *sort_counts, bool ids32) {
+  HCTR_CHECK(!ids32 || t.id_max <= 0xffffffffull, "internal: narrowed ids and a table of 2^32 rows or more");
   if (!n) return;
   const unsigned nblocks = (unsigned)sort_tiles(n);
   const int dbits = sort_first_digit_bits(kl.total_bits);
@@ -299,10 +301,12 @@ void launch_make_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, co
   do {                                                                                                                \
     if (kl.wide)                                                                                                      \
       hipLaunchKernelGGL((make_keys<uint64_t, I>), dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max,          \
-                         kl.id_bits, t.nrank, t.root, (uint64_t *)comp_keys, err, nlong, dbits, sort_counts);         \
+                         kl.id_bits, t.nrank, t.root, (uint64_t *)comp_keys, err, nlong, dbits, sort_counts,  \
+                         ids32);         \
     else                                                                                                              \
       hipLaunchKernelGGL((make_keys<uint32_t, I>), dim3(nblocks), dim3(kSortBlock), 0, s, keys, n, t.id_max,          \
-                         kl.id_bits, t.nrank, t.root, (uint32_t *)comp_keys, err, nlong, dbits, sort_counts);         \
+                         kl.id_bits, t.nrank, t.root, (uint32_t *)comp_keys, err, nlong, dbits, sort_counts,  \
+                         ids32);         \
   } while (0)
   HCTR_SORT_ITEMS_DISPATCH(n, CALL);
 #undef CALL

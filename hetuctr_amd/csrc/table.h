@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "../../include/hetuctr_hip.h"
+#include "host_copy.h"
 #include "kernels.h"
 #include "radix_sort.h"
 #include "tile_sort.h"
@@ -138,6 +139,7 @@ class Shard {
   // own device word (default: the device block that is read back after the call)
   void index_batch(uint32_t *u_out = nullptr, int part = 0);
   TileSortBuffers tile_sort_buffers() const; // the index scratch as the tile-sorted passes take it
+  HostStager stager;                         // ids that arrive in pageable host memory go through its pinned buffer
   int tile_sort_mode = 1;                    // HETUCTR_TILE_SORT: 0 no batch takes the tile-sorted passes, 1 those of up
                                              // to kTileSortMaxKeys keys, 2 every batch whose tiles they can hold
   void plan_batch(Batch &b);  // enqueues the push plan of b; its counts reach the host when the stream has run it

@@ -280,12 +280,15 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
       hipPointerAttribute_t attr;
       const bool visible = hipPointerGetAttributes(&attr, keys) == hipSuccess &&
                            (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged);
+      bool narrowed = false;
       if (!visible) {
         (void)hipGetLastError(); // an unregistered host pointer leaves a sticky "invalid value"
         HCTR_CHECK(!scratch_area, "preprocess without allocations takes ids in device memory only (a transfer from "
                                   "pageable host memory is staged by the runtime)");
+        // through pinned memory, as 32-bit ids when the table's ids fit (half the bytes on the bus)
+        narrowed = tv.id_max <= 0xffffffffull;
         cur.staged.reserve(n * sizeof(index_t));
-        HCTR_HIP(hipMemcpyAsync(cur.staged.p, keys, n * sizeof(index_t), hipMemcpyDefault, s));
+        stager.copy(cur.staged.p, keys, n * sizeof(index_t), s, narrowed);
       }
       const index_t *ids = visible ? (const index_t *)keys : (const index_t *)cur.staged.as<index_t>();
       cur.tile_sorted = tile_sort_mode == 2 ? tile_sort_possible(cur.n) : (tile_sort_mode == 1 && tile_sort_fits(cur.n));
@@ -295,10 +298,10 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
       cur.keys_made = !cur.tile_sorted || (flag != nullptr && cur.n >= kKeysFirstFrom);
       if (!cur.keys_made)
         launch_tile_sort_keys(s, tv, kl, ids, nullptr, cur.n, tile_sort_buffers(), flag ? flag : err_ptr(),
-                              cur.dnlong.as<uint32_t>());
+                              cur.dnlong.as<uint32_t>(), narrowed);
       else
         launch_make_keys(s, tv, kl, ids, cur.n, cur.comp.p, flag ? flag : err_ptr(), cur.dnlong.as<uint32_t>(),
-                         cur.tile_sorted ? nullptr : sp.sortws);
+                         cur.tile_sorted ? nullptr : sp.sortws, narrowed);
     }
   }
 }

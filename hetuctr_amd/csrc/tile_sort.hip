@@ -159,7 +159,7 @@ __global__ __launch_bounds__(kSortBlock) void keys_tile_sort(const void *__restr
                                                               const worker_t *__restrict__ root, uint32_t *__restrict__ err,
                                                               uint32_t *__restrict__ nlong, int dbits, uint32_t pitch,
                                                               K *__restrict__ out_keys, uint32_t *__restrict__ out_vals,
-                                                              uint16_t *__restrict__ table) {
+                                                              uint16_t *__restrict__ table, bool ids32) {
   using S = TileShape<K, ITEMS>;
   __shared__ __align__(16) uint32_t area[S::kAreaWords];
   __shared__ uint32_t bin_start[kSortMaxBins];
@@ -185,7 +185,8 @@ __global__ __launch_bounds__(kSortBlock) void keys_tile_sort(const void *__restr
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
       const uint32_t e = w * S::kSub + r * kWave + lane;
-      id[r] = e < tile_n ? (uint64_t)load_once(&ids[tile_lo + e]) : 0; // the caller's ids are read here and nowhere else
+      // the caller's ids are read here and nowhere else (ids32: as narrowed on their way from pageable host memory)
+      id[r] = e >= tile_n ? 0 : ids32 ? (uint64_t)load_once(&((const uint32_t *)ids)[tile_lo + e]) : (uint64_t)load_once(&ids[tile_lo + e]);
     }
     bool bad = false;
 #pragma unroll
@@ -486,8 +487,10 @@ DigitPlan plan_digits(const KeyLayout &kl) {
   } while (0)
 
 void launch_tile_sort_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *ids,
-                           const void *made_keys, uint32_t n, const TileSortBuffers &b, uint32_t *err, uint32_t *nlong) {
+                           const void *made_keys, uint32_t n, const TileSortBuffers &b, uint32_t *err, uint32_t *nlong,
+                           bool ids32) {
   if (!n) return;
+  HCTR_CHECK(!ids32 || t.id_max <= 0xffffffffull, "internal: narrowed ids and a table of 2^32 rows or more");
   HCTR_CHECK(tile_sort_possible(n), "internal: batch too large for the tile-sorted passes");
   const DigitPlan p = plan_digits(kl);
   const unsigned tiles = (unsigned)tile_count(n), pitch = (unsigned)tile_table_pitch(n);
@@ -496,11 +499,12 @@ void launch_tile_sort_keys(hipStream_t s, const TableView &t, const KeyLayout &k
   do {                                                                                                                \
     if (made_keys)                                                                                                    \
       hipLaunchKernelGGL((keys_tile_sort<K, I, D, true>), dim3(tiles), dim3(kSortBlock), 0, s, made_keys, n, t.id_max, \
-                         kl.id_bits, t.nrank, t.root, err, nlong, p.dbits[0], pitch, (K *)b.keys[0], b.vals[0], table0); \
+                         kl.id_bits, t.nrank, t.root, err, nlong, p.dbits[0], pitch, (K *)b.keys[0], b.vals[0], table0, \
+                         false);                                                                                      \
     else                                                                                                              \
       hipLaunchKernelGGL((keys_tile_sort<K, I, D, false>), dim3(tiles), dim3(kSortBlock), 0, s, (const void *)ids, n, \
                          t.id_max, kl.id_bits, t.nrank, t.root, err, nlong, p.dbits[0], pitch, (K *)b.keys[0],        \
-                         b.vals[0], table0);                                                                          \
+                         b.vals[0], table0, ids32);                                                                   \
   } while (0)
   HCTR_TILE_SORT_DISPATCH(kl.wide, n, p.dbits[0], CALL);
 #undef CALL

@@ -398,7 +398,9 @@ def test_large_batches_of_ids_in_pageable_host_memory():
     length, width = 500_000, 4
     p = single(length, width, init=("Zero", 0.0, 0.0), lr=0.5)
     buf = np.zeros(400_003, np.int64)
-    for step, n in enumerate([262_143, 262_144, 262_145, 400_003, 131_072 * 3 + 1, 300_000, 5]):
+    # (a copy of 1 MiB or more is staged by several threads in 128 KiB pieces and transferred 1 MiB at a time)
+    for step, n in enumerate([262_143, 262_144, 262_145, 400_003, 131_072 * 3 + 1, 300_000, 5, 100_000, 131_071, 131_072,
+                              16_384 * 9 + 1, 16_384 * 17 - 1]):
         want = rng.integers(0, length, size=n).astype(np.int64)
         buf[:n] = want
         p.tables[0].preprocess(buf.ctypes.data, n)
@@ -409,10 +411,17 @@ def test_large_batches_of_ids_in_pageable_host_memory():
         out, ref = p.push_pull([None])
         assert_close(out[0], ref[0], 1e-5, "dst n %d" % n)
     # an id out of range in the middle of a large host batch is reported by the call
-    keys = rng.integers(0, length, size=300_000).astype(np.int64)
-    keys[123_456] = length
-    with pytest.raises(RuntimeError, match="outside"):
-        p.tables[0].preprocess(keys.ctypes.data, keys.shape[0])
+    # (ids from host memory travel as 32-bit words when the table's ids fit: one that does not fit must not alias a valid id)
+    for bad in (length, -1, 1 << 40, (1 << 32) + 5, -(1 << 33)):
+        keys = rng.integers(0, length, size=300_000).astype(np.int64)
+        keys[123_456] = bad
+        with pytest.raises(RuntimeError, match="outside"):
+            p.tables[0].preprocess(keys.ctypes.data, keys.shape[0])
+        want = keys.copy()
+        want[123_456] = 0                                   # "it was treated as id 0"
+        p.oracle.preprocess([want])
+        p.n = [keys.shape[0]]
+        p.compare_ints([capi.UNIQUE, capi.SORTED_ARG, capi.RUN_START, capi.KEYS], "bad id %d" % bad)
     p.close()
 
 
