@@ -284,7 +284,7 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
       if (!visible) {
         (void)hipGetLastError(); // an unregistered host pointer leaves a sticky "invalid value"
         HCTR_CHECK(!scratch_area, "preprocess without allocations takes ids in device memory only (a transfer from "
-                                  "pageable host memory is staged by the runtime)");
+                                  "pageable host memory needs a staging buffer)");
         // through pinned memory, as 32-bit ids when the table's ids fit (half the bytes on the bus)
         narrowed = tv.id_max <= 0xffffffffull;
         cur.staged.reserve(n * sizeof(index_t));
@@ -1099,7 +1099,7 @@ void Group::preprocess_noalloc(const int64_t *keys, size_t n) {
                          (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged);
     if (!visible) (void)hipGetLastError();
     HCTR_CHECK(visible, "preprocess without allocations takes ids in device memory only (a transfer from pageable "
-                        "host memory is staged by the runtime)");
+                        "host memory needs a staging buffer)");
   }
   m->swap_batches();
   m->ingest_keys(keys, n, nullptr, noalloc_scratch);
