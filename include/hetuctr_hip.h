@@ -67,10 +67,11 @@ int hctr_preprocess(hctr_table *t, const int64_t *keys, size_t n);
  * like the reference's call it returns when all its work is done.  It calls no hipMalloc / hipFree and no allocating
  * routine; it does synchronise the table's stream and reads counts back to the host, so it cannot be recorded into a
  * HIP graph:
- *   - the index scratch (sort ping-pong buffers, per-tile digit counts, scan sums) lives in a static device array of
- *     7.0 MiB that every GPU the library runs on holds until the process ends;
+ *   - the index scratch (sort ping-pong buffers, per-tile digit tables, scan sums, head counts) lives in a static device array of
+ *     7.1 MiB that every GPU the library runs on holds until the process ends;
  *   - n is at most 262144 keys (HCTR_NOALLOC_MAX_KEYS), larger batches are refused;
- *   - keys must be DEVICE memory (a transfer from pageable host memory is staged by the runtime);
+ *   - keys must be DEVICE memory (ids in pageable host memory go through a pinned staging buffer the library
+ *     would have to allocate);
  *   - the table has one shard, and its two batch buffers already hold n keys: they are sized by ordinary
  *     hctr_preprocess calls (two in a row with the largest batch size both); otherwise the call is refused.
  * All tables on one GPU share that GPU's array: calls that overlap on one GPU race. */
