@@ -166,9 +166,10 @@ void launch_push(hipStream_t s, const TableView &t, const KeyLayout &kl, const B
                  const PushArgs &a);
 
 // ---- query / owner side / pull -------------------------------------------------------------------------
-// id and local version of every unique key of the current batch (n_unique: the host's count of them), written to place
-// (unique rank + delta[owner of the key]) of q_idx / q_ver (delta: nrank words in device memory)
-void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t n_unique,
+// id and local version of every unique key of the current batch, written to place (unique rank + delta[owner of the
+// key]) of q_idx / q_ver (delta: nrank words in device memory).  unique_max: no more unique keys than this (the batch's
+// size); how many there are the kernel reads from cur.d_U.
+void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t unique_max,
                           const uint32_t *delta, index_t *q_idx, version_t *q_ver);
 // Owner side of a step: applying the received pushes (per target row in source order) and serving the received
 // queries (outdated flags, positions of the rows to return, rows packed, first returned row of every requester).
@@ -182,7 +183,12 @@ struct OwnerShard {
   uint32_t rg_seg[258];
   int longest;               // the source with the most rows
   uint32_t push_blocks;      // blocks the push kernel needs for this shard (rows of `longest` / rows per block)
-  // received queries; rq_seg[0..nsrc]: first query of every requester; [rq_seg[rank], rq_seg[rank + 1]) are its own
+  // Received queries; rq_seg[0..nsrc]: first query of every requester; [rq_seg[rank], rq_seg[rank + 1]) are its own.
+  // How many unique keys every shard asks every owner for is known on the device only (the host does not wait for the
+  // index of the current batches): send_cnt / n_keys are filled in on the host, and place_queries -- a launch in front
+  // of the query kernels -- cuts the group's receive area from them and writes rq_idx .. ret_slot and got_delta below.
+  const uint64_t *send_cnt;  // [nsrc] unique keys of THIS shard's current batch per owner (written by its index)
+  uint32_t n_keys;           // keys of this shard's current batch; 0: the shard asks for nothing (send_cnt is stale)
   const index_t *rq_idx;
   const version_t *rq_ver;
   uint32_t rq_seg[258];
@@ -199,7 +205,7 @@ struct OwnerShard {
   uint32_t *ret_delta;       // [nsrc]
   // The flag of every received query goes straight to its requester as well: got = THIS shard's flags as a requester
   // (one per unique key, owners in rank order); got_delta[s]: what an owner adds to the place of a query in its receive
-  // buffer to get the place of the flag in requester s' array (known on the host).
+  // buffer to get the place of the flag in requester s' array (written by place_queries).
   uint32_t *got;
   uint32_t got_delta[257];
   uint32_t *err;             // the shard's error word
@@ -208,9 +214,27 @@ struct OwnerShard {
 };
 size_t query_tiles(uint32_t q);                       // tile_cnt needs this many words + 1
 uint32_t owner_push_rows_per_block(uint32_t width);   // rows of the longest source one block of the push kernel takes
-// shards_dev: the array in device memory; shards_host: the same values on the host (launch geometry).  nshards == nsrc:
-// every shard of the group is in the array, in rank order (an owner looks its requesters up there).
-void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerShard *shards_host, int nshards, int nsrc);
+// The receive area of the queries of a step, shared by all owners of the group: every array holds one entry per unique
+// key of all current batches at most (`capacity`).  launch_place_queries cuts it: one piece per owner, inside it one per
+// requester, both in rank order (csrc/core/all2all.cu:18-46), from the counts the shards' index kernels left on the
+// device, and writes into every shard's record where its piece lies, and into query_delta[s * nsrc + d] what requester
+// s adds to the rank of a unique key owned by d to get the key's place in the area.
+struct QueryArea {
+  index_t *idx;
+  version_t *ver;
+  uint32_t *outdated;
+  slot_t *q_slot, *ret_slot;
+  uint32_t *query_delta;     // [nsrc * nsrc]
+};
+// (shards_host: the records as the host filled them in, for the addresses of the counts)
+void launch_place_queries(hipStream_t s, OwnerShard *shards_dev, const OwnerShard *shards_host, int nsrc,
+                          const QueryArea &area);
+// shards_dev: the array in device memory.  nshards == nsrc: every shard of the group is in the array, in rank order (an
+// owner looks its requesters up there).  push_blocks: the most blocks a shard's received pushes need; queries_max: no
+// shard receives more queries than this; queries_guess: what the busiest shard probably receives (the grids are cut
+// from it; what a shard does receive, the kernels read from the records and stride over).
+void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, int nshards, int nsrc, uint32_t width,
+                       uint32_t push_blocks, uint32_t queries_max, uint32_t queries_guess);
 // requester: refresh cached rows that came back, then gather every key's row into dst
 struct PullArgs {
   const uint32_t *got;       // [U] or nullptr: nothing came back (nrank == 1)
@@ -223,10 +247,11 @@ struct PullArgs {
   uint32_t list_chunks;      // the gather also builds the batch's run lists (run_lists.h): chunks of unique ranks, else 0
 };
 // Index of every returned row per unique key (a.ret_i), where the gather reads each key's row (a.src_row), the counts of
-// the step and the refresh of the cached rows that came back.  tile_sums: scratch of scan_blocks(n_unique) words;
+// the step and the refresh of the cached rows that came back.  tile_sums: scratch of scan_blocks(unique_max) words (unique_max: the batch's size; the number of unique keys is read from cur.d_U; unique_guess: the grid of the row kernel is cut from it);
 // stats: five device words that read zero before the first call (the launch leaves them zero again); host_stats: four
 // words the device can write (hit / miss / refreshed counts of the step, error bits)
-void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
+void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t unique_max, uint32_t unique_guess,
+                    const PullArgs &a,
                     uint32_t *tile_sums, uint32_t *stats, uint32_t *host_stats);
 void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a);
 // sum-pooled lookups: dst[b] = the rows of positions b * bag .. b * bag + bag - 1 added up in that order

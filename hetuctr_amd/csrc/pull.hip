@@ -148,6 +148,70 @@ __global__ __launch_bounds__(kBlock) void apply_remote_all(const OwnerShard *__r
 // device memory, where place_returns reads it, and to the host.
 // pack_rows: version and row of every flagged query packed at its position (:24-40), from the list of their slots
 // that scan_positions leaves.
+// One block.  Thread d, owner: its queries per requester in rank order (rq_seg), their number, the tiles of its flag
+// scan; then the owners' pieces of the area in rank order; thread s, requester: what it adds to a unique key's rank
+// per owner (query_delta), and what owner d adds to the place of one of s' queries to get the place of its flag in
+// s' array (got_delta: s' flags stand in owner order).  Up to kPlaceLds shards the matrix of counts is fetched into LDS
+// by all threads at once (one memory round trip instead of one per entry and thread).
+constexpr int kPlaceLds = 48;
+struct PlaceSources { // of the first kPlaceLds shards: where their counts lie, and whether they ask at all
+  const uint64_t *send_cnt[kPlaceLds];
+  uint32_t n_keys[kPlaceLds];
+};
+__global__ __launch_bounds__(kBlock) void place_queries(OwnerShard *shards, int R, QueryArea area, PlaceSources src) {
+  __shared__ uint32_t sm[kBlock / kWave + 1];
+  __shared__ uint32_t base[kBlock];
+  __shared__ uint32_t cnt[kPlaceLds * kPlaceLds];  // [requester][owner] unique keys asked for
+  __shared__ uint32_t segm[kPlaceLds * kPlaceLds]; // [owner][requester] first query of the requester at the owner
+  const int t = threadIdx.x;
+  const bool in_lds = R <= kPlaceLds;
+  if (in_lds) {
+    for (int i = t; i < R * R; i += kBlock) {
+      const int s = i / R, d = i % R;
+      cnt[i] = src.n_keys[s] ? (uint32_t)src.send_cnt[s][d] : 0u;
+    }
+    __syncthreads();
+  }
+  auto asked = [&](int s, int d) -> uint32_t { // unique keys requester s asks owner d for
+    if (in_lds) return cnt[s * R + d];
+    return shards[s].n_keys ? (uint32_t)shards[s].send_cnt[d] : 0u;
+  };
+  uint32_t Q = 0;
+  if (t < R) {
+    OwnerShard &D = shards[t];
+    for (int s = 0; s < R; s++) {
+      D.rq_seg[s] = Q;
+      if (in_lds) segm[t * R + s] = Q;
+      Q += asked(s, t);
+    }
+    D.rq_seg[R] = Q;
+    D.q = Q;
+    D.query_tiles = max(1u, (Q + kBlock - 1) / kBlock); // one tile even without queries: the segment table is written
+  }
+  uint32_t total;
+  const uint32_t lo = block_exclusive_scan<kBlock>(Q, sm, total);
+  base[t] = lo;
+  if (t < R) {
+    OwnerShard &D = shards[t];
+    D.rq_idx = area.idx + lo;
+    D.rq_ver = area.ver + lo;
+    D.outdated = area.outdated + lo;
+    D.q_slot = area.q_slot + lo;
+    D.ret_slot = area.ret_slot + lo;
+  }
+  __syncthreads(); // rq_seg of every owner is written (global memory, this block), base[] too
+  if (t < R) {
+    uint32_t ulo = 0; // unique keys of requester t that belong to the owners before d
+    for (int d = 0; d < R; d++) {
+      const uint32_t seg = in_lds ? segm[d * R + t] : shards[d].rq_seg[t];
+      // (place in the area) - (rank among the requester's unique keys), modulo 2^32 like the sum the kernel forms
+      area.query_delta[(size_t)t * R + d] = base[d] + seg - ulo;
+      shards[d].got_delta[t] = ulo - seg;
+      ulo += asked(t, d);
+    }
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restrict__ shards, int nseg) {
   const OwnerShard &S = shards[blockIdx.y];
   if (blockIdx.x >= S.query_tiles) return;
@@ -156,70 +220,76 @@ __global__ __launch_bounds__(kBlock) void decide_count(const OwnerShard *__restr
   __shared__ uint32_t sseg[258];
   for (int i = threadIdx.x; i <= nseg; i += kBlock) sseg[i] = S.rq_seg[i];
   __syncthreads();
-  const uint32_t k = blockIdx.x * kBlock + threadIdx.x;
-  uint32_t flag = 0;
-  if (k < S.q) {
-    const slot_t o = owned_slot(t.slot, (uint64_t)S.rq_idx[k], t.id_max, t.n_cached);
-    S.q_slot[k] = o;
-    // the requester: the segment of the receive buffer the query lies in (segments may be empty)
-    uint32_t lo = 0, hi = nseg - 1;
-    while (lo < hi) { // the first segment that ends behind k
-      const uint32_t mid = (lo + hi) / 2;
-      if (sseg[mid + 1] <= k) lo = mid + 1;
-      else hi = mid;
+  // the grid is cut from a guess (the number of queries is known on the device only): a block takes every gridDim.x-th tile
+  for (uint32_t tile = blockIdx.x; tile < S.query_tiles; tile += gridDim.x) {
+    const uint32_t k = tile * kBlock + threadIdx.x;
+    uint32_t flag = 0;
+    if (k < S.q) {
+      const slot_t o = owned_slot(t.slot, (uint64_t)S.rq_idx[k], t.id_max, t.n_cached);
+      S.q_slot[k] = o;
+      // the requester: the segment of the receive buffer the query lies in (segments may be empty)
+      uint32_t lo = 0, hi = nseg - 1;
+      while (lo < hi) { // the first segment that ends behind k
+        const uint32_t mid = (lo + hi) / 2;
+        if (sseg[mid + 1] <= k) lo = mid + 1;
+        else hi = mid;
+      }
+      if (o == kNoSlot) {
+        atomicOr(S.err, 4u);
+      } else {
+        const version_t local = S.rq_ver[k], global = t.ver[o];
+        const bool from_self = lo == (uint32_t)t.rank;
+        const bool out = local == kInvalidVersion || local + t.pull_bound < global;
+        flag = (out && !from_self) ? 1u : 0u;
+      }
+      S.outdated[k] = flag;
+      shards[lo].got[k + S.got_delta[lo]] = flag; // the requester reads it from its own array
     }
-    if (o == kNoSlot) {
-      atomicOr(S.err, 4u);
-    } else {
-      const version_t local = S.rq_ver[k], global = t.ver[o];
-      const bool from_self = lo == (uint32_t)t.rank;
-      const bool out = local == kInvalidVersion || local + t.pull_bound < global;
-      flag = (out && !from_self) ? 1u : 0u;
+    const uint64_t m = __ballot(flag != 0);
+    if (lane_id() == 0) wcnt[threadIdx.x / kWave] = __popcll(m);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t c = 0;
+      for (int i = 0; i < kBlock / kWave; i++) c += wcnt[i];
+      S.tile_cnt[tile] = c;
     }
-    S.outdated[k] = flag;
-    shards[lo].got[k + S.got_delta[lo]] = flag; // the requester reads it from its own array
-  }
-  const uint64_t m = __ballot(flag != 0);
-  if (lane_id() == 0) wcnt[threadIdx.x / kWave] = __popcll(m);
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t c = 0;
-    for (int i = 0; i < kBlock / kWave; i++) c += wcnt[i];
-    S.tile_cnt[blockIdx.x] = c;
+    __syncthreads(); // wcnt is rewritten for the next tile
   }
 }
 
 __global__ __launch_bounds__(kBlock) void scan_positions(const OwnerShard *__restrict__ shards, int nseg) {
   const OwnerShard &S = shards[blockIdx.y];
-  if (blockIdx.x >= S.query_tiles) return;
   __shared__ uint32_t sm[kBlock / kWave + 1];
   __shared__ uint32_t excl[kBlock + 1]; // position of every query of the tile among the returned rows; [kBlock]: after it
   const uint32_t q = S.q;
-  const uint32_t tile_lo = blockIdx.x * kBlock, k = tile_lo + threadIdx.x;
-  const uint32_t f = k < q ? S.outdated[k] : 0u;
-  uint32_t s = 0;
-  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kBlock) s += S.tile_cnt[i];
-  uint32_t before;
-  block_exclusive_scan<kBlock>(s, sm, before); // flagged queries in the tiles before this one
-  uint32_t total;
-  const uint32_t pos = before + block_exclusive_scan<kBlock>(f, sm, total);
-  if (f) S.ret_slot[pos] = S.q_slot[k]; // the rows to return, in the order they go back
-  excl[threadIdx.x] = pos;
-  if (threadIdx.x == 0) excl[kBlock] = before + total;
-  __syncthreads();
-  // the first returned row of a requester's segment is the position of the segment's first query
-  const bool last_block = blockIdx.x == S.query_tiles - 1;
-  for (int g = threadIdx.x; g <= nseg; g += kBlock) {
-    const uint32_t start = S.rq_seg[g];
-    uint32_t v = ~0u;
-    if (start >= tile_lo && start < tile_lo + kBlock && start < q) v = excl[start - tile_lo];
-    else if (last_block && start >= q) v = excl[kBlock]; // segments that start at the end: the total
-    if (v != ~0u) {
-      S.seg_dev[g] = v;
-      S.seg_host[g] = v;
+  for (uint32_t tile = blockIdx.x; tile < S.query_tiles; tile += gridDim.x) { // as in decide_count
+    const uint32_t tile_lo = tile * kBlock, k = tile_lo + threadIdx.x;
+    const uint32_t f = k < q ? S.outdated[k] : 0u;
+    uint32_t s = 0;
+    for (uint32_t i = threadIdx.x; i < tile; i += kBlock) s += S.tile_cnt[i];
+    uint32_t before;
+    block_exclusive_scan<kBlock>(s, sm, before); // flagged queries in the tiles before this one
+    uint32_t total;
+    const uint32_t pos = before + block_exclusive_scan<kBlock>(f, sm, total);
+    if (f) S.ret_slot[pos] = S.q_slot[k]; // the rows to return, in the order they go back
+    excl[threadIdx.x] = pos;
+    if (threadIdx.x == 0) excl[kBlock] = before + total;
+    __syncthreads();
+    // the first returned row of a requester's segment is the position of the segment's first query
+    const bool last_tile = tile == S.query_tiles - 1;
+    for (int g = threadIdx.x; g <= nseg; g += kBlock) {
+      const uint32_t start = S.rq_seg[g];
+      uint32_t v = ~0u;
+      if (start >= tile_lo && start < tile_lo + kBlock && start < q) v = excl[start - tile_lo];
+      else if (last_tile && start >= q) v = excl[kBlock]; // segments that start at the end: the total
+      if (v != ~0u) {
+        S.seg_dev[g] = v;
+        S.seg_host[g] = v;
+      }
     }
+    if (last_tile && threadIdx.x == 0) S.seg_host[257] = *S.err;
+    __syncthreads(); // excl is rewritten for the next tile
   }
-  if (last_block && threadIdx.x == 0) S.seg_host[257] = *S.err;
 }
 
 // Where the rows an owner returns stand in the requesters' buffers: a requester's rows arrive in owner order
@@ -250,11 +320,10 @@ __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict
   for (int i = threadIdx.x; i <= nseg; i += kBlock) sseg[i] = S.seg_dev[i];
   for (int i = threadIdx.x; i < nseg; i += kBlock) sdelta[i] = S.ret_delta[i];
   __syncthreads();
-  const uint32_t total = sseg[nseg]; // rows this shard returns
-  const uint32_t k0 = blockIdx.x * (kGroups * kPackAhead) + threadIdx.x / LPR;
-  if (k0 >= total) return;
+  const uint32_t total = sseg[nseg]; // rows this shard returns: known on the device only, the grid is cut for the most
   const embed_t *__restrict__ emb = S.t.emb;
   const uint32_t gl = threadIdx.x % LPR, W = S.t.width;
+  for (uint32_t k0 = blockIdx.x * (kGroups * kPackAhead) + threadIdx.x / LPR; k0 < total; k0 += gridDim.x * (kGroups * kPackAhead)) {
   slot_t o[kPackAhead];
 #pragma unroll
   for (int a = 0; a < kPackAhead; a++) o[a] = k0 + a * kGroups < total ? S.ret_slot[k0 + a * kGroups] : kNoSlot;
@@ -288,6 +357,7 @@ __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict
     for (int a = 0; a < kPackAhead; a++)
       if (o[a] != kNoSlot) __builtin_nontemporal_store(v[a], (V *)(dst_val[a] + col)); // read next by another shard's kernels
   }
+  }
 }
 
 // What comes back per unique key of the step, in two launches over tiles of kRTile keys:
@@ -301,9 +371,11 @@ __global__ __launch_bounds__(kBlock) void pack_rows(const OwnerShard *__restrict
 // counters back to zero for the next step: no clearing launch before, no copy after.
 constexpr uint32_t kReturnedRow = 0x80000000u;
 constexpr int kRItems = 8, kRTile = kBlock * kRItems; // 2048 keys: the tile scan_blocks() sizes the scratch for
-__global__ __launch_bounds__(kBlock) void got_tile_sums(const uint32_t *__restrict__ got, uint32_t U,
+__global__ __launch_bounds__(kBlock) void got_tile_sums(const uint32_t *__restrict__ got, const uint32_t *__restrict__ d_U,
                                                         uint32_t *__restrict__ tile_sums) {
   __shared__ uint32_t sm[kBlock / kWave + 1];
+  const uint32_t U = *d_U; // the grid is cut for the batch's keys: the host has not seen the number of unique ones
+  if (blockIdx.x * kRTile >= U) return;
   const uint32_t j0 = blockIdx.x * kRTile + threadIdx.x * kRItems;
   uint32_t c = 0;
 #pragma unroll
@@ -313,10 +385,13 @@ __global__ __launch_bounds__(kBlock) void got_tile_sums(const uint32_t *__restri
   if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
 }
 __global__ __launch_bounds__(kBlock) void remote_emit(TableView t, BatchView c, const uint32_t *__restrict__ got,
-                                                      const uint32_t *__restrict__ tile_sums, uint32_t U,
+                                                      const uint32_t *__restrict__ tile_sums,
                                                       uint32_t *__restrict__ ret_i, uint32_t *__restrict__ src_row,
                                                       uint32_t *__restrict__ stats, uint32_t *__restrict__ host_stats) {
   __shared__ uint32_t sm[kBlock / kWave + 1];
+  const uint32_t U = *c.d_U;
+  const uint32_t tiles = (U + kRTile - 1) / kRTile; // of the grid's blocks (cut for the batch's keys) these have work
+  if (blockIdx.x >= tiles) return;
   __shared__ uint32_t tot[4];
   __shared__ bool last;
   if (threadIdx.x < 4) tot[threadIdx.x] = 0;
@@ -370,7 +445,7 @@ __global__ __launch_bounds__(kBlock) void remote_emit(TableView t, BatchView c, 
   __syncthreads();
   if (threadIdx.x == 0) {
     __threadfence();
-    last = atomicAdd(&stats[4], 1u) == gridDim.x - 1;
+    last = atomicAdd(&stats[4], 1u) == tiles - 1;
   }
   __syncthreads();
   if (last && threadIdx.x < 4) {
@@ -385,17 +460,17 @@ template <int VEC, int LPR>
 __global__ __launch_bounds__(kBlock) void refresh(TableView t, BatchView c, PullArgs a) {
   typedef typename RowVec<VEC>::T V;
   constexpr int kGroups = kBlock / LPR;
-  const uint32_t u = blockIdx.x * kGroups + threadIdx.x / LPR;
-  if (u >= *c.d_U) return;
-  const uint32_t gl = threadIdx.x % LPR, W = t.width;
-  const slot_t o = c.uoff[u];
-  const bool got = a.got[u] != 0;
-  if (!got || o == kNoSlot || (uint32_t)o >= t.n_cached) return; // (an owned row that came back is reported by remote_emit)
-  const uint32_t k = a.ret_i[u];
-  if (gl == 0) t.ver[o] = a.in_ver[k];
-  for (uint32_t col = gl * VEC; col < W; col += LPR * VEC)
-    *(V *)(t.emb + (size_t)o * W + col) =
-        *(const V *)(a.in_val + (size_t)k * W + col) + *(const V *)(t.pend + (size_t)o * W + col);
+  const uint32_t U = *c.d_U, gl = threadIdx.x % LPR, W = t.width;
+  for (uint32_t u = blockIdx.x * kGroups + threadIdx.x / LPR; u < U; u += gridDim.x * kGroups) {
+    const slot_t o = c.uoff[u];
+    const bool got = a.got[u] != 0;
+    if (!got || o == kNoSlot || (uint32_t)o >= t.n_cached) continue; // (an owned row that came back is reported by remote_emit)
+    const uint32_t k = a.ret_i[u];
+    if (gl == 0) t.ver[o] = a.in_ver[k];
+    for (uint32_t col = gl * VEC; col < W; col += LPR * VEC)
+      *(V *)(t.emb + (size_t)o * W + col) =
+          *(const V *)(a.in_val + (size_t)k * W + col) + *(const V *)(t.pend + (size_t)o * W + col);
+  }
 }
 
 // Gather in SORTED order: one group per kRows consecutive sorted positions.  Duplicates of a key are adjacent,
@@ -526,10 +601,10 @@ inline int lanes_for(uint32_t width, int vec) {
 
 } // namespace
 
-void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t n_unique,
+void launch_build_queries(hipStream_t s, const TableView &t, const KeyLayout &kl, const BatchView &cur, uint32_t unique_max,
                           const uint32_t *delta, index_t *q_idx, version_t *q_ver) {
-  if (!n_unique) return;
-  const dim3 grid(div_up(n_unique, kBlock));
+  if (!unique_max) return;
+  const dim3 grid(div_up(unique_max, kBlock)); // the kernel reads the number of unique keys itself
   if (kl.wide) hipLaunchKernelGGL(build_queries<uint64_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, delta, q_idx, q_ver);
   else hipLaunchKernelGGL(build_queries<uint32_t>, grid, dim3(kBlock), 0, s, t, kl.id_bits, cur, delta, q_idx, q_ver);
   HCTR_HIP(hipGetLastError());
@@ -542,14 +617,28 @@ uint32_t owner_push_rows_per_block(uint32_t width) {
   return kApplyBatches * kApplyAhead * (kBlock / lpr);
 }
 
-void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerShard *shards_host, int nshards, int nsrc) {
-  uint32_t push_blocks = 0, tiles = 0, q_max = 0;
-  const uint32_t width = shards_host[0].t.width;
-  for (int i = 0; i < nshards; i++) {
-    push_blocks = std::max(push_blocks, shards_host[i].push_blocks);
-    tiles = std::max(tiles, shards_host[i].query_tiles);
-    q_max = std::max(q_max, shards_host[i].q);
+void launch_place_queries(hipStream_t s, OwnerShard *shards_dev, const OwnerShard *shards_host, int nsrc,
+                          const QueryArea &area) {
+  HCTR_CHECK(nsrc <= kBlock, "internal: more shards than the placing block has threads");
+  PlaceSources src;
+  for (int i = 0; i < kPlaceLds; i++) {
+    src.send_cnt[i] = i < nsrc ? shards_host[i].send_cnt : nullptr;
+    src.n_keys[i] = i < nsrc ? shards_host[i].n_keys : 0;
   }
+  hipLaunchKernelGGL(place_queries, dim3(1), dim3(kBlock), 0, s, shards_dev, nsrc, area, src);
+  HCTR_HIP(hipGetLastError());
+}
+
+// Grids of kernels whose work is known on the device only are cut from a guess (what the step before had, and some)
+// and never beyond the most there can be; the kernels stride over what there is.
+static uint32_t guessed_blocks(uint32_t guess, uint32_t most, uint32_t per_block) {
+  const uint64_t g = (uint64_t)guess + guess / 4 + 4 * per_block;
+  return std::max(1u, div_up(std::min<uint64_t>(g, most), per_block));
+}
+
+void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, int nshards, int nsrc, uint32_t width,
+                       uint32_t push_blocks, uint32_t queries_max, uint32_t queries_guess) {
+  const uint32_t tiles = guessed_blocks(queries_guess, queries_max, kBlock);
   const bool vec4 = width % 4 == 0;
   const int lpr = lanes_for(width, vec4 ? 4 : 1);
   if (push_blocks) {
@@ -561,27 +650,28 @@ void launch_owner_side(hipStream_t s, const OwnerShard *shards_dev, const OwnerS
   }
   hipLaunchKernelGGL(decide_count, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
   hipLaunchKernelGGL(scan_positions, dim3(tiles, nshards), dim3(kBlock), 0, s, shards_dev, nsrc);
-  if (q_max) {
+  if (queries_max) {
     hipLaunchKernelGGL(place_returns, dim3(div_up((uint32_t)(nsrc * nsrc), kBlock)), dim3(kBlock), 0, s, shards_dev, nsrc);
-#define CALL(V, L) \
-  hipLaunchKernelGGL((pack_rows<V, L>), dim3(div_up(q_max, kPackAhead * (kBlock / L)), nshards), dim3(kBlock), 0, s, shards_dev, nsrc)
+#define CALL(V, L)                                                                                                     \
+  hipLaunchKernelGGL((pack_rows<V, L>), dim3(guessed_blocks(queries_guess, queries_max, kPackAhead * (kBlock / L)), nshards), \
+                     dim3(kBlock), 0, s, shards_dev, nsrc)
     HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   }
   HCTR_HIP(hipGetLastError());
 }
 
-void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t n_unique, const PullArgs &a,
-                    uint32_t *tile_sums, uint32_t *stats, uint32_t *host_stats) {
-  if (!n_unique || !a.got) return;
-  const unsigned tiles = div_up(n_unique, kRTile);
-  hipLaunchKernelGGL(got_tile_sums, dim3(tiles), dim3(kBlock), 0, s, a.got, n_unique, tile_sums);
-  hipLaunchKernelGGL(remote_emit, dim3(tiles), dim3(kBlock), 0, s, t, cur, a.got, tile_sums, n_unique, a.ret_i, a.src_row,
-                     stats, host_stats);
+void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uint32_t unique_max, uint32_t unique_guess,
+                    const PullArgs &a, uint32_t *tile_sums, uint32_t *stats, uint32_t *host_stats) {
+  if (!unique_max || !a.got) return;
+  const unsigned tiles = div_up(unique_max, kRTile); // for the batch's keys; the kernels read how many are unique
+  hipLaunchKernelGGL(got_tile_sums, dim3(tiles), dim3(kBlock), 0, s, a.got, cur.d_U, tile_sums);
+  hipLaunchKernelGGL(remote_emit, dim3(tiles), dim3(kBlock), 0, s, t, cur, a.got, tile_sums, a.ret_i, a.src_row, stats,
+                     host_stats);
   const bool vec4 = t.width % 4 == 0;
   const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
-#define CALL(V, L) \
-  hipLaunchKernelGGL((refresh<V, L>), dim3(div_up(n_unique, kBlock / L)), dim3(kBlock), 0, s, t, cur, a)
+#define CALL(V, L)                                                                                                      \
+  hipLaunchKernelGGL((refresh<V, L>), dim3(guessed_blocks(unique_guess, unique_max, kBlock / L)), dim3(kBlock), 0, s, t, cur, a)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL
   HCTR_HIP(hipGetLastError());

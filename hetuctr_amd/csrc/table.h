@@ -153,7 +153,9 @@ class Shard {
   void begin_push(const float *grad, uint32_t bag = 1);  // which batch is pushed (none on an inference step), checks
   void generate_gradient(const uint32_t *delta);         // the push kernel; delta: see Group::place_pushes
   void generate_query(const uint32_t *delta); // delta: see Group::place_queries
-  void fill_owner_args(OwnerShard &o);      // handleGradient + handleQuery: what the group's owner-side launches need
+  // handleGradient + handleQuery: what the group's owner-side launches need of this shard (queries_max: no shard
+  // receives more queries than this)
+  void fill_owner_args(OwnerShard &o, uint64_t queries_max);
   void finish_handle_query();               // after the step: return counts and error flags from the pinned block
   void write_back(float *dst, uint32_t bag = 1);
   void finish_push_pull();
@@ -180,10 +182,11 @@ class Shard {
   const float *push_grad_ = nullptr; // arguments of the push between begin_push and generate_gradient
   uint32_t push_bag_ = 1;
   // receive side (owner role)
-  DeviceBuf outdated, ret_slot, q_slot, src_row, ret_seg_dev;
+  DeviceBuf src_row, ret_seg_dev;
   std::vector<uint64_t> rq_seg, rg_seg, ret_seg; // R+1 prefix offsets per source / requester
   uint64_t rg_base = 0;      // first row of this shard's piece of the group's receive area for pushed rows
-  uint64_t rq_base = 0;      // first query of its piece of the receive area for queries
+  uint64_t rq_base = 0;      // first query of its piece of the receive area for queries (rq_seg, rq_base: the host's
+                             // copy of what place_queries computed on the device, made when the step is over)
   DeviceBuf push_pos;        // place of every unique key's pushed row in that area (plan position + distance)
   // requester side of the return
   DeviceBuf got, ret_i, in_ver, in_val;
@@ -254,17 +257,22 @@ class Group {
   // owner-side arguments of every shard: pinned staging and the device copy the kernels read
   OwnerShard *owner_host = nullptr;
   DeviceBuf owner_dev, ret_delta_dev;    // ret_delta_dev: nrank words per owner, see OwnerShard::ret_delta
-  void owner_side();
+  void owner_side(uint64_t queries_max);
   // Where every shard's pushed rows go: one receive area for the whole group (ids, counts, rows), cut into one piece
   // per owner and, inside it, per source; sized from the plans before any push kernel runs.  Every sender gets, per
   // owner, the distance between a row's place in its own plan and its place in the area (nrank words per sender).
   void place_pushes();
   DeviceBuf rg_idx_all, rg_cnt_all, rg_val_all, push_delta_dev;
   uint32_t *push_delta_host = nullptr;   // pinned staging of the distances
-  // the same for the queries of a step: one receive area (ids, versions), nrank distances per requester
-  void place_queries();
-  DeviceBuf rq_idx_all, rq_ver_all, query_delta_dev;
-  uint32_t *query_delta_host = nullptr;
+  // The same for the queries of a step: one receive area (ids, versions, and what the owners keep per query), nrank
+  // distances per requester.  How many queries go where is known on the device only: reserve_queries() sizes the area
+  // for the most there can be, launch_place_queries (behind the upload of the owners' records) cuts it.
+  uint64_t reserve_queries();
+  QueryArea query_area();
+  void note_query_places(); // rq_seg / rq_base of every shard from the counts the host has once the step is over
+  uint32_t queries_guess_ = 0; // queries the busiest owner received in the step before
+  bool queries_seen_ = false;
+  DeviceBuf rq_idx_all, rq_ver_all, rq_outdated_all, rq_slot_all, rq_ret_all, query_delta_dev;
   bool time_calls = false;               // bracket the two calls with events (hctr_call_timing)
   std::vector<Shard *> members;
   double wait_seconds = 120.0;

@@ -483,7 +483,7 @@ void Shard::generate_query(const uint32_t *delta) {
   hipStream_t s = group->stream;
   StageScope st(*group, S_QUERY);
   // every query is written where its owner reads it: the group's receive area (see Group::place_queries)
-  launch_build_queries(s, tv, kl, cur.view(), cur.U, delta, group->rq_idx_all.as<index_t>(),
+  launch_build_queries(s, tv, kl, cur.view(), cur.n, delta, group->rq_idx_all.as<index_t>(),
                        group->rq_ver_all.as<version_t>());
 }
 
@@ -491,50 +491,40 @@ void Shard::generate_query(const uint32_t *delta) {
 // and queries, the buffers of the rows that go back.  The number of rows that go back to every requester stays on the
 // device, where the owners' kernels read it; the host copy (statistics, error flags) is written by the same kernel
 // into pinned memory and read when the step is over.
-void Shard::fill_owner_args(OwnerShard &o) {
+void Shard::fill_owner_args(OwnerShard &o, uint64_t queries_max) {
   const int R = cfg.nrank;
-  const uint32_t Q = (uint32_t)rq_seg[R];
-  outdated.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
-  ret_slot.reserve((size_t)std::max<uint32_t>(Q, 1) * 4);
-  q_slot.reserve((size_t)std::max<uint32_t>(Q, 1) * sizeof(slot_t));
-  // requester role: what comes back lands here (a row per unique key at most), written by the owners
-  const size_t rows_ub = std::max<uint32_t>(cur.U, 1);
+  query_sums.reserve((query_tiles((uint32_t)queries_max) + 2) * 4);
+  // requester role: what comes back lands here (a row per unique key at most, and the host has not seen how many of
+  // the batch's keys are unique), written by the owners
+  const size_t rows_ub = std::max<uint32_t>(cur.n, 1);
   got.reserve(rows_ub * 4);
   in_ver.reserve(rows_ub * sizeof(version_t));
   in_val.reserve(rows_ub * cfg.width * sizeof(embed_t));
-  query_sums.reserve((query_tiles(Q) + 2) * 4);
   last_stats[5] = (long long)rg_seg[R];
   o.t = tv;
   o.rg_idx = group->rg_idx_all.as<index_t>() + rg_base;
   o.rg_cnt = group->rg_cnt_all.as<version_t>() + rg_base;
   o.rg_val = group->rg_val_all.as<embed_t>() + rg_base * cfg.width;
   o.longest = 0;
-  for (int i = 0; i <= R; i++) {
-    o.rg_seg[i] = (uint32_t)rg_seg[i];
-    o.rq_seg[i] = (uint32_t)rq_seg[i];
-  }
+  for (int i = 0; i <= R; i++) o.rg_seg[i] = (uint32_t)rg_seg[i];
   for (int i = 1; i < R; i++)
     if (rg_seg[i + 1] - rg_seg[i] > rg_seg[o.longest + 1] - rg_seg[o.longest]) o.longest = i;
   o.push_blocks = div_up(rg_seg[o.longest + 1] - rg_seg[o.longest], owner_push_rows_per_block(tv.width));
-  o.rq_idx = group->rq_idx_all.as<index_t>() + rq_base;
-  o.rq_ver = group->rq_ver_all.as<version_t>() + rq_base;
-  o.q = Q;
-  o.query_tiles = (uint32_t)query_tiles(Q); // one tile even without queries: the segment table is written
-  o.outdated = outdated.as<uint32_t>();
+  // the received queries: place_queries fills in where they lie and how many they are (rq_idx .. got_delta)
+  o.send_cnt = dst_->send_cnt;
+  o.n_keys = cur.n;
+  o.rq_idx = nullptr;
+  o.rq_ver = nullptr;
+  o.q = 0;
+  o.query_tiles = 1;
+  o.outdated = nullptr;
+  o.ret_slot = nullptr;
+  o.q_slot = nullptr;
   o.tile_cnt = query_sums.as<uint32_t>();
-  o.ret_slot = ret_slot.as<slot_t>();
-  o.q_slot = q_slot.as<slot_t>();
   o.in_ver = in_ver.as<version_t>();
   o.in_val = in_val.as<embed_t>();
   o.ret_delta = group->ret_delta_dev.as<uint32_t>() + (size_t)cfg.rank * R;
   o.got = got.as<uint32_t>();
-  // csrc/core/all2all.cu:89-130: the flags of requester s' queries stand in its array in owner order; this owner's
-  // begin behind the queries s sent to the owners before it
-  for (int s = 0; s < R; s++) {
-    uint64_t before = 0;
-    for (int e = 0; e < cfg.rank; e++) before += group->members[s]->cur.send_cnt[e];
-    o.got_delta[s] = (uint32_t)(before - rq_seg[s]);
-  }
   o.err = err_ptr();
   o.seg_dev = ret_seg_dev.as<uint32_t>();
   o.seg_host = mirror->ret_seg;
@@ -566,19 +556,20 @@ void Shard::write_back(float *dst, uint32_t bag) {
   // batch there for the push that updates them next.  The one case where that loses is a batch of (almost) all
   // distinct keys, where the gather reads as many rows as it writes; the previous batch is the predictor.
   a.stream_stores = !(prev.n != 0 && (double)prev.U >= 0.9 * (double)prev.n);
-  if (cfg.nrank > 1 && cur.U == 0) {
+  if (cfg.nrank > 1 && cur.n == 0) {
     memset(mirror->stats, 0, sizeof mirror->stats); // no keys: nothing came back (nothing in flight writes the block)
   } else if (cfg.nrank > 1) {
-    ret_i.reserve((size_t)std::max<uint32_t>(cur.U, 1) * 4);
-    reserve_batch_scratch(cur.U);
+    // sized for the batch's keys: how many of them are unique the kernels read on the device (the host has not
+    // waited for the index); the scan scratch is the one the batch's index was given, its kernels are through
+    ret_i.reserve((size_t)cur.n * 4);
+    src_row.reserve((size_t)cur.n * 4);
     StageScope st(*group, S_REFRESH);
     a.got = got.as<uint32_t>();
     a.ret_i = ret_i.as<uint32_t>();
-    src_row.reserve((size_t)std::max<uint32_t>(cur.U, 1) * 4);
     a.src_row = src_row.as<uint32_t>();
     a.in_ver = in_ver.as<version_t>();
     a.in_val = in_val.as<embed_t>();
-    launch_refresh(s, tv, cur.view(), cur.U, a, sp.block_sums, stats.as<uint32_t>(), mirror->stats);
+    launch_refresh(s, tv, cur.view(), cur.n, prev.U ? prev.U : cur.n, a, sp.block_sums, stats.as<uint32_t>(), mirror->stats);
   }
   if (dst != nullptr) {
     StageScope st(*group, S_GATHER);
@@ -664,7 +655,7 @@ size_t Shard::fetch(int which, void *out, size_t cap) {
     case HCTR_F_PUSHRECV_CNT: return put64(prev.pushrecv_cnt, R, out, cap);
     case HCTR_F_OUTDATED: {
       if (R == 1) { std::vector<long long> z(cur.U, 0); return put64(z, cur.U, out, cap); }
-      return put64(download<uint32_t>(outdated.p, rq_seg[R]), rq_seg[R], out, cap);
+      return put64(download<uint32_t>(group->rq_outdated_all.as<uint32_t>() + rq_base, rq_seg[R]), rq_seg[R], out, cap);
     }
     case HCTR_F_GOT: {
       if (R == 1) { std::vector<long long> z(cur.U, 0); return put64(z, cur.U, out, cap); }
@@ -749,7 +740,6 @@ Group::~Group() {
   if (ev_plan) (void)hipEventDestroy(ev_plan);
   if (owner_host) (void)hipHostFree(owner_host);
   if (push_delta_host) (void)hipHostFree(push_delta_host);
-  if (query_delta_host) (void)hipHostFree(query_delta_host);
 }
 
 void Group::join(Shard *s) {
@@ -807,16 +797,14 @@ void Group::collect_marks() {
 }
 
 // handleGradient + handleQuery of every shard (csrc/core/hetu_gpu_table.cu:27-31): one set of launches for the group
-void Group::owner_side() {
-  if (!owner_host) {
-    HCTR_HIP(hipHostMalloc((void **)&owner_host, (size_t)nrank * sizeof(OwnerShard), hipHostMallocDefault));
-    owner_dev.reserve((size_t)nrank * sizeof(OwnerShard));
-    ret_delta_dev.reserve((size_t)nrank * nrank * sizeof(uint32_t));
-  }
-  for (Shard *m : members) m->fill_owner_args(owner_host[m->cfg.rank]);
+void Group::owner_side(uint64_t queries_max) {
+  uint32_t push_blocks = 0;
+  for (int r = 0; r < nrank; r++) push_blocks = std::max(push_blocks, owner_host[r].push_blocks);
   StageScope st(*this, S_OWNER);
-  HCTR_HIP(hipMemcpyAsync(owner_dev.p, owner_host, (size_t)nrank * sizeof(OwnerShard), hipMemcpyHostToDevice, stream));
-  launch_owner_side(stream, owner_dev.as<OwnerShard>(), owner_host, nrank, nrank);
+  // the grids of the query kernels: from what the busiest owner received in the step before (the first step: the most)
+  const uint32_t guess = queries_seen_ ? queries_guess_ : (uint32_t)queries_max;
+  launch_owner_side(stream, owner_dev.as<OwnerShard>(), nrank, nrank, members[0]->cfg.width, push_blocks, (uint32_t)queries_max,
+                    guess);
 }
 
 void Group::set_defer_index(bool on) {
@@ -886,17 +874,43 @@ void Group::place_pushes() {
 }
 
 // csrc/core/all2all.cu:18-46: every owner's receive buffer is the requesters' buckets for it, in source order.  The
-// queries do not pass through a send buffer either: how many unique keys every shard asks every owner for is known on the
-// host once the index is done, so the group's receive area is cut (one piece per owner, inside it one per source) and
-// every shard's query kernel writes into it; a unique key of rank u lands u + (distance for its owner) into the area.
-void Group::place_queries() {
+// queries do not pass through a send buffer either: every shard's query kernel writes into one receive area of the
+// group, cut into one piece per owner and, inside it, one per source; a unique key of rank u lands u + (distance for its
+// owner) into the area.  How many unique keys every shard asks every owner for is left on the device by the shards'
+// index kernels, and the host does not wait for them: the area is sized here for the most queries there can be (a batch
+// has no more unique keys than keys) and cut on the device (launch_place_queries), which also tells every owner where
+// its piece lies.  Returns that maximum.
+uint64_t Group::reserve_queries() {
   const int R = nrank;
-  if (R == 1) return;
-  if (!query_delta_host) {
-    HCTR_HIP(hipHostMalloc((void **)&query_delta_host, (size_t)R * R * sizeof(uint32_t), hipHostMallocDefault));
-    query_delta_dev.reserve((size_t)R * R * sizeof(uint32_t));
-  }
-  uint64_t total = 0;
+  if (R == 1) return 0;
+  uint64_t most = 0;
+  for (Shard *m : members) most += m->cur.n;
+  HCTR_CHECK(most < 0xfffffff0ull, "more than 2^32 queries in one step");
+  const uint64_t cap = std::max<uint64_t>(most, 1);
+  rq_idx_all.reserve(cap * sizeof(index_t));
+  rq_ver_all.reserve(cap * sizeof(version_t));
+  rq_outdated_all.reserve(cap * 4);
+  rq_slot_all.reserve(cap * sizeof(slot_t));
+  rq_ret_all.reserve(cap * sizeof(slot_t));
+  query_delta_dev.reserve((size_t)R * R * sizeof(uint32_t));
+  return most;
+}
+
+QueryArea Group::query_area() {
+  QueryArea a;
+  a.idx = rq_idx_all.as<index_t>();
+  a.ver = rq_ver_all.as<version_t>();
+  a.outdated = rq_outdated_all.as<uint32_t>();
+  a.q_slot = rq_slot_all.as<slot_t>();
+  a.ret_slot = rq_ret_all.as<slot_t>();
+  a.query_delta = query_delta_dev.as<uint32_t>();
+  return a;
+}
+
+// what launch_place_queries computed, once more on the host when the step is over (introspection reads it)
+void Group::note_query_places() {
+  const int R = nrank;
+  uint64_t total = 0, busiest = 0;
   for (int d = 0; d < R; d++) {
     Shard &dst = *members[d];
     dst.rq_base = total;
@@ -907,21 +921,10 @@ void Group::place_queries() {
     }
     dst.rq_seg[R] = Q;
     total += Q;
+    busiest = std::max(busiest, Q);
   }
-  HCTR_CHECK(total < 0xfffffff0ull, "more than 2^32 queries in one step");
-  rq_idx_all.reserve(std::max<uint64_t>(total, 1) * sizeof(index_t));
-  rq_ver_all.reserve(std::max<uint64_t>(total, 1) * sizeof(version_t));
-  if (!total) return;
-  for (int s = 0; s < R; s++) {
-    uint64_t ulo = 0; // unique keys of this shard that belong to the owners before d
-    for (int d = 0; d < R; d++) {
-      const Shard &dst = *members[d];
-      query_delta_host[(size_t)s * R + d] = (uint32_t)(dst.rq_base + dst.rq_seg[s] - ulo);
-      ulo += members[s]->cur.send_cnt[d];
-    }
-    HCTR_CHECK(ulo == members[s]->cur.U, "internal: the queries per owner do not add up to the unique keys");
-  }
-  HCTR_HIP(hipMemcpyAsync(query_delta_dev.p, query_delta_host, (size_t)R * R * sizeof(uint32_t), hipMemcpyHostToDevice, stream));
+  queries_guess_ = (uint32_t)busiest;
+  queries_seen_ = true;
 }
 
 // csrc/core/hetu_gpu_table.cu:43-65 for every shard of the group
@@ -1160,41 +1163,42 @@ void Group::push_pull_steps(const float *const *grads, float *const *dsts, uint3
   if (time_calls) HCTR_HIP(hipEventRecord(ev_push, stream));
   if (nrank > 1) HCTR_HIP(hipEventRecord(ev_pushed, stream));
   enqueue_index_rest(); // the pushes are in their queue, now the rest of the current batches' index
+  const bool join_index = index_pending;
   if (nrank > 1) {
-    const bool wait_index = index_pending;
-    if (wait_index) HCTR_HIP(hipEventRecord(ev_index, index_stream));
+    if (join_index) HCTR_HIP(hipEventRecord(ev_index, index_stream));
     {
       // the push plans of the current batches, for the step in which they are the previous ones: after the pushes of
-      // this step (they move the update counters the plan reads), beside everything else the step still does; queued
-      // before the host looks at the index, so that nothing but the queries stands between that look and the owner side
+      // this step (they move the update counters the plan reads), beside everything else the step still does
       StreamSwitch on(*this, index_stream);
       HCTR_HIP(hipStreamWaitEvent(stream, ev_pushed, 0));
       for (Shard *m : members) m->plan_batch(m->cur);
       HCTR_HIP(hipEventRecord(ev_plan, stream));
     }
-    if (wait_index) {
-      // the queries are built from the index of the current batches, which the host needs too (unique keys and queries
-      // per owner place the queries)
-      index_pending = false;
-      index_joining_ = true;
-      HCTR_HIP(hipEventSynchronize(ev_index));
-      for (Shard *m : members) m->finish_index();
-      exchange_shapes();
-      index_joining_ = false;
-    }
   }
-  place_queries();
-  for (Shard *m : members) m->generate_query(nrank > 1 ? query_delta_dev.as<uint32_t>() + (size_t)nrank * m->cfg.rank : nullptr);
-  const bool join_index = index_pending;
   if (join_index) {
-    // the push kernel is in the main stream's queue; the gather below also needs the index of the current batch,
-    // still running or done on the second stream
+    // The push kernels are in the main stream's queue; everything below needs the index of the current batches, still
+    // running or done on the second stream.  The host does not wait for it (the reference waits twice inside this
+    // call, csrc/core/hetu_gpu_table.cu:23,33): what the index leaves -- unique keys per shard, queries per owner --
+    // is read on the device by the kernels that need it, and by the host when the step is over.
     index_pending = false;
     index_joining_ = true;
     HCTR_HIP(hipStreamWaitEvent(stream, ev_index, 0));
   }
   if (nrank > 1) {
-    owner_side();
+    if (!owner_host) {
+      HCTR_HIP(hipHostMalloc((void **)&owner_host, (size_t)nrank * sizeof(OwnerShard), hipHostMallocDefault));
+      owner_dev.reserve((size_t)nrank * sizeof(OwnerShard));
+      ret_delta_dev.reserve((size_t)nrank * nrank * sizeof(uint32_t));
+    }
+    const uint64_t queries_max = reserve_queries();
+    for (Shard *m : members) m->fill_owner_args(owner_host[m->cfg.rank], queries_max);
+    HCTR_HIP(hipMemcpyAsync(owner_dev.p, owner_host, (size_t)nrank * sizeof(OwnerShard), hipMemcpyHostToDevice, stream));
+    {
+      StageScope st(*this, S_QUERY);
+      launch_place_queries(stream, owner_dev.as<OwnerShard>(), owner_host, nrank, query_area());
+    }
+    for (Shard *m : members) m->generate_query(query_delta_dev.as<uint32_t>() + (size_t)nrank * m->cfg.rank);
+    owner_side(queries_max);
     // the reference waits here for the return counts (hetu_gpu_table.cu:33); they stay on the device
   }
   for (Shard *m : members) m->write_back(dsts[m->cfg.rank], bag);
@@ -1206,9 +1210,12 @@ void Group::push_pull_steps(const float *const *grads, float *const *dsts, uint3
     for (Shard *m : members) m->finish_plan(m->cur);
   if (join_index) {
     index_joining_ = false; // from here on the results are taken over, or the batch's own error is reported
-    members[0]->finish_preprocess();
+    if (nrank == 1) members[0]->finish_preprocess();
+    else
+      for (Shard *m : members) m->finish_index();
     exchange_shapes();
   }
+  if (nrank > 1) note_query_places();
   float ms = 0.f, push_ms = 0.f;
   if (time_calls) {
     HCTR_HIP(hipEventElapsedTime(&ms, ev0, ev1));
