@@ -1177,9 +1177,10 @@ void Group::push_pull_steps(const float *const *grads, float *const *dsts, uint3
   }
   if (join_index) {
     // The push kernels are in the main stream's queue; everything below needs the index of the current batches, still
-    // running or done on the second stream.  The host does not wait for it (the reference waits twice inside this
-    // call, csrc/core/hetu_gpu_table.cu:23,33): what the index leaves -- unique keys per shard, queries per owner --
-    // is read on the device by the kernels that need it, and by the host when the step is over.
+    // running or done on the second stream.  The host does not wait for it (the reference has the shapes on the host
+    // because its preprocess waits for all of its work, csrc/core/hetu_gpu_table.cu:60-64): what the index leaves --
+    // unique keys per shard, queries per owner -- is read on the device by the kernels that need it, and by the host
+    // when the step is over.
     index_pending = false;
     index_joining_ = true;
     HCTR_HIP(hipStreamWaitEvent(stream, ev_index, 0));

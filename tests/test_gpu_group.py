@@ -107,6 +107,35 @@ def test_stepwise_parity_with_staleness(nrank, bounds, cache, width):
     p.close()
 
 
+@pytest.mark.parametrize("nrank,cache,width", [(3, "third", 20), (5, "lower", 128)])
+def test_steps_without_a_look_at_the_index(nrank, cache, width):
+    # Nothing is fetched between preprocess and push_pull, so push_pull finds the index of the current batches still
+    # running and never waits for it on the host: the queries are placed and counted on the device, and the grids of
+    # the query kernels are cut from what the step before had.  Batch sizes jump by orders of magnitude both ways,
+    # shards sit steps out, one step has no keys at all.
+    say("no look at the index", nrank, cache, width)
+    length = 40_000
+    p, root = update_pair(nrank, length, width, bounds=(1, 2), init=("Uniform", -1.0, 1.0), lr=0.5, cache=cache, seed=5)
+    rng = np.random.default_rng(nrank)
+    draw = zipf_sampler(length, 1.05, rng)
+    sizes = [300, 120_000, 7, 60_000, 0, 1, 90_000, 2_000]
+    prev_n = [0] * nrank
+    for step, bs in enumerate(sizes):
+        keys = [draw(max(bs - 5 * r, 0)) if step % 2 else rng.integers(0, length, max(bs - 5 * r, 0)).astype(np.int64)
+                for r in range(nrank)]
+        if step in (1, 6):
+            keys[step % nrank] = np.zeros(0, np.int64)     # a shard sits out a large step
+        p.preprocess(keys, device_keys=bool(step % 3))
+        grads = [rng.normal(0, 0.1, size=(prev_n[r], width)).astype(np.float32) for r in range(nrank)]
+        out, ref = p.push_pull(grads)
+        p.compare_ints(INT_ITEMS_PRE + INT_ITEMS_POST, "step %d" % step)
+        for r in range(nrank):
+            assert_close(out[r], ref[r], 1e-5, "dst step %d rank %d" % (step, r))
+        p.compare_state(1e-5, "step %d" % step)
+        prev_n = [k.shape[0] for k in keys]
+    p.close()
+
+
 @pytest.mark.parametrize("bounds,cached", [((0, 0), (0,)), ((2, 3), tuple(range(8)))])
 def test_partitioned_table_with_hot_row_cache(bounds, cached):
     # the 8-way partition of the Criteo-like table at 1/100 scale: uniform owners, the hottest 10 % of the remote
