@@ -1164,12 +1164,27 @@ void Group::push_pull_steps(const float *const *grads, float *const *dsts, uint3
   if (nrank > 1) HCTR_HIP(hipEventRecord(ev_pushed, stream));
   enqueue_index_rest(); // the pushes are in their queue, now the rest of the current batches' index
   const bool join_index = index_pending;
+  uint64_t queries_max = 0;
   if (nrank > 1) {
-    if (join_index) HCTR_HIP(hipEventRecord(ev_index, index_stream));
+    if (!owner_host) {
+      HCTR_HIP(hipHostMalloc((void **)&owner_host, (size_t)nrank * sizeof(OwnerShard), hipHostMallocDefault));
+      owner_dev.reserve((size_t)nrank * sizeof(OwnerShard));
+      ret_delta_dev.reserve((size_t)nrank * nrank * sizeof(uint32_t));
+    }
+    queries_max = reserve_queries();
+    for (Shard *m : members) m->fill_owner_args(owner_host[m->cfg.rank], queries_max);
     {
+      // Behind the index, on its stream and beside the pushes: the owners' records go to the device and the receive
+      // area of the queries is cut there from the counts the index left (nothing of this needs the host to know them).
+      StreamSwitch on(*this, index_stream);
+      HCTR_HIP(hipMemcpyAsync(owner_dev.p, owner_host, (size_t)nrank * sizeof(OwnerShard), hipMemcpyHostToDevice, stream));
+      {
+        StageScope st(*this, S_QUERY);
+        launch_place_queries(stream, owner_dev.as<OwnerShard>(), owner_host, nrank, query_area());
+      }
+      HCTR_HIP(hipEventRecord(ev_index, stream));
       // the push plans of the current batches, for the step in which they are the previous ones: after the pushes of
       // this step (they move the update counters the plan reads), beside everything else the step still does
-      StreamSwitch on(*this, index_stream);
       HCTR_HIP(hipStreamWaitEvent(stream, ev_pushed, 0));
       for (Shard *m : members) m->plan_batch(m->cur);
       HCTR_HIP(hipEventRecord(ev_plan, stream));
@@ -1183,21 +1198,9 @@ void Group::push_pull_steps(const float *const *grads, float *const *dsts, uint3
     // when the step is over.
     index_pending = false;
     index_joining_ = true;
-    HCTR_HIP(hipStreamWaitEvent(stream, ev_index, 0));
   }
+  if (join_index || nrank > 1) HCTR_HIP(hipStreamWaitEvent(stream, ev_index, 0));
   if (nrank > 1) {
-    if (!owner_host) {
-      HCTR_HIP(hipHostMalloc((void **)&owner_host, (size_t)nrank * sizeof(OwnerShard), hipHostMallocDefault));
-      owner_dev.reserve((size_t)nrank * sizeof(OwnerShard));
-      ret_delta_dev.reserve((size_t)nrank * nrank * sizeof(uint32_t));
-    }
-    const uint64_t queries_max = reserve_queries();
-    for (Shard *m : members) m->fill_owner_args(owner_host[m->cfg.rank], queries_max);
-    HCTR_HIP(hipMemcpyAsync(owner_dev.p, owner_host, (size_t)nrank * sizeof(OwnerShard), hipMemcpyHostToDevice, stream));
-    {
-      StageScope st(*this, S_QUERY);
-      launch_place_queries(stream, owner_dev.as<OwnerShard>(), owner_host, nrank, query_area());
-    }
     for (Shard *m : members) m->generate_query(query_delta_dev.as<uint32_t>() + (size_t)nrank * m->cfg.rank);
     owner_side(queries_max);
     // the reference waits here for the return counts (hetu_gpu_table.cu:33); they stay on the device
