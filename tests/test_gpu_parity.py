@@ -425,6 +425,41 @@ def test_large_batches_of_ids_in_pageable_host_memory():
     p.close()
 
 
+def test_host_ids_from_two_threads_at_once():
+    # two tables, each fed large host batches by a thread of its own: the threads that stage host ids are shared by
+    # the process, a copy posted while another is under way must leave both batches intact
+    import threading
+    say("host ids from two threads")
+    length, width, steps = 300_000, 4, 6
+    tables = [single(length, width, init=("Zero", 0.0, 0.0), lr=0.5) for _ in range(2)]
+    errors = []
+
+    def feed(i):
+        try:
+            rng = np.random.default_rng(50 + i)
+            t = tables[i].tables[0]
+            for step in range(steps):
+                n = 200_000 + 37 * i + 1000 * step               # 1.6 MB of ids: staged by the crew
+                want = rng.integers(0, length, size=n).astype(np.int64)
+                buf = want.copy()
+                t.preprocess(buf.ctypes.data, n)
+                buf[:] = -1
+                got = t.fetch(capi.KEYS)
+                if not np.array_equal(got, want):
+                    errors.append("table %d step %d: %d ids differ" % (i, step, int((got != want).sum())))
+        except Exception as e:                                   # noqa: BLE001 - reported by the main thread
+            errors.append("table %d: %r" % (i, e))
+
+    threads = [threading.Thread(target=feed, args=(i,)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    for p in tables:
+        p.close()
+    assert not errors, errors
+
+
 @pytest.mark.parametrize("nrank", [1, 3])
 def test_64_bit_sort_keys_at_every_sort_shape(nrank, monkeypatch):
     # sort keys wider than 32 bits (owner and id of a huge id space) are forced on a small table; batch sizes from
