@@ -254,6 +254,10 @@ void launch_refresh(hipStream_t s, const TableView &t, const BatchView &cur, uin
                     const PullArgs &a,
                     uint32_t *tile_sums, uint32_t *stats, uint32_t *host_stats);
 void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a);
+// one shard: dst[i] = row of the id in keys[i] (the batch's sort keys in batch order), for all n positions; needs
+// nothing of the batch's index
+void launch_gather_direct(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *keys, uint32_t n, embed_t *dst,
+                          bool stream_stores);
 // sum-pooled lookups: dst[b] = the rows of positions b * bag .. b * bag + bag - 1 added up in that order
 // (cur.idx_map must be filled: launch_idx_map)
 void launch_gather_pooled(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a, uint32_t bag);

@@ -522,6 +522,40 @@ __global__ __launch_bounds__(kBlock) void gather(TableView t, BatchView c, PullA
   }
 }
 
+// Gather in BATCH order straight from the batch's keys, for one shard: dst[i] = emb[slot[id of position i]].  It needs
+// nothing of the batch's index (sort, unique pass), so a step whose index is longer than its push -- a small batch --
+// does not wait for it; what it gives up is the order in which the duplicates of a key are adjacent, which only matters
+// once the rows of a batch no longer fit the caches.
+template <int VEC, int LPR, typename K, bool kStream>
+__global__ __launch_bounds__(kBlock) void gather_direct(TableView t, const K *__restrict__ keys, int id_bits, uint32_t n,
+                                                        embed_t *__restrict__ dst_rows) {
+  typedef typename RowVec<VEC>::T V;
+  constexpr int kGroups = kBlock / LPR;
+  const uint32_t W = t.width;
+  const uint32_t i0 = (blockIdx.x * kGroups + threadIdx.x / LPR) * kRows;
+  if (i0 >= n) return;
+  const uint32_t gl = threadIdx.x % LPR;
+  const K id_mask = (K)(((uint64_t)1 << id_bits) - 1);
+  const embed_t *src[kRows];
+#pragma unroll
+  for (int k = 0; k < kRows; k++) {
+    const uint32_t i = min(i0 + k, n - 1);
+    src[k] = t.emb + (size_t)t.slot[(uint64_t)(keys[i] & id_mask)] * W; // one shard: every id is resident
+  }
+  for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
+    V v[kRows];
+#pragma unroll
+    for (int k = 0; k < kRows; k++) v[k] = *(const V *)(src[k] + col);
+#pragma unroll
+    for (int k = 0; k < kRows; k++)
+      if (i0 + k < n) {
+        V *d = (V *)(dst_rows + (size_t)(i0 + k) * W + col);
+        if (kStream) __builtin_nontemporal_store(v[k], d);
+        else *d = v[k];
+      }
+  }
+}
+
 // Sum-pooled lookups: one group per bag of `bag` consecutive batch positions.  The rows of the bag are requested
 // kPoolAhead at a time and added in position order (fp32, starting from the first row), so a bag costs one output
 // row instead of `bag`.  Works in batch order, through the inverse index of the batch.
@@ -689,6 +723,25 @@ void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, cons
     else if (local_only) hipLaunchKernelGGL((gather<V, L, true, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a); \
     else if (a.stream_stores) hipLaunchKernelGGL((gather<V, L, false, true>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a); \
     else hipLaunchKernelGGL((gather<V, L, false, false>), dim3(blocks), dim3(kBlock), 0, s, t, cur, a);          \
+  } while (0)
+  HCTR_DISPATCH_ROW(vec4, lpr, CALL);
+#undef CALL
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_gather_direct(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *keys, uint32_t n, embed_t *dst,
+                          bool stream_stores) {
+  if (!n) return;
+  HCTR_CHECK(t.nrank == 1, "internal: the gather from the keys is for one shard");
+  const bool vec4 = t.width % 4 == 0 && ((uintptr_t)dst % 16) == 0;
+  const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
+#define CALL(V, L)                                                                                                    \
+  do {                                                                                                                \
+    const unsigned blocks = div_up(n, (kBlock / L) * kRows);                                                          \
+    if (kl.wide && stream_stores) hipLaunchKernelGGL((gather_direct<V, L, uint64_t, true>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint64_t *)keys, kl.id_bits, n, dst); \
+    else if (kl.wide) hipLaunchKernelGGL((gather_direct<V, L, uint64_t, false>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint64_t *)keys, kl.id_bits, n, dst); \
+    else if (stream_stores) hipLaunchKernelGGL((gather_direct<V, L, uint32_t, true>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint32_t *)keys, kl.id_bits, n, dst); \
+    else hipLaunchKernelGGL((gather_direct<V, L, uint32_t, false>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint32_t *)keys, kl.id_bits, n, dst); \
   } while (0)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL

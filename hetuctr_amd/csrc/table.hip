@@ -127,6 +127,8 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   // which sort indexes a batch: 0 the three-launch passes of radix_sort.h always, 2 the tile-sorted passes whenever
   // they can hold the batch (measurements of either sort at any size); default: tile_sort_fits()
   if (const char *f = getenv("HETUCTR_TILE_SORT")) tile_sort_mode = f[0] == '0' ? 0 : (f[0] == '2' ? 2 : 1);
+  direct_gather_max = (uint32_t)std::min<uint64_t>(HCTR_DIRECT_GATHER_BYTES / ((uint64_t)c.width * sizeof(embed_t)), 0xfffffff0u);
+  if (const char *f = getenv("HETUCTR_DIRECT_GATHER_MAX")) direct_gather_max = (uint32_t)strtoul(f, nullptr, 10);
   if (const char *f = getenv("HETUCTR_TILE_DIGIT_BITS")) // many narrow passes exercise the hand-over between the launches
     kl.max_digit_bits = atoi(f);
 
@@ -265,6 +267,8 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
   cur.idx_map_valid = false;
   cur.planned = false;
   cur.lists_ready = n == 0;
+  cur.direct_gather = false;
+  cur.comp_valid = false;
   if (!scratch_area) cur.reserve(cur.n, cfg.nrank, kl.wide); // else: the caller has checked that the buffers hold n keys
   if (n == 0) { // :93-95
     cur.clear(s, cfg.nrank);
@@ -295,10 +299,14 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
       // A call that returns as soon as the ids are read (flag: where it looks for a bad id) gets them read by the
       // lightest kernel there is when the batch is large: the sort keys alone.  Sorting a tile as well keeps the
       // caller -- whose next call starts the gradient push -- waiting several microseconds longer.
+      // One shard and a small batch: the step's gather works from the keys in batch order and leaves the index off
+      // the step's critical path (write_back); the keys are then made by a kernel of their own here as well.
+      cur.direct_gather = cfg.nrank == 1 && flag != nullptr && cur.n <= direct_gather_max;
       cur.keys_made = !cur.tile_sorted || (flag != nullptr && cur.n >= kKeysFirstFrom);
+      cur.comp_valid = cur.keys_made || cur.direct_gather;
       if (!cur.keys_made)
         launch_tile_sort_keys(s, tv, kl, ids, nullptr, cur.n, tile_sort_buffers(), flag ? flag : err_ptr(),
-                              cur.dnlong.as<uint32_t>(), narrowed);
+                              cur.dnlong.as<uint32_t>(), narrowed, cur.direct_gather ? cur.comp.p : nullptr);
       else
         launch_make_keys(s, tv, kl, ids, cur.n, cur.comp.p, flag ? flag : err_ptr(), cur.dnlong.as<uint32_t>(),
                          cur.tile_sorted ? nullptr : sp.sortws, narrowed);
@@ -354,7 +362,8 @@ void Shard::index_batch(uint32_t *u_out, int part) {
     if (part == 1) return;
     StageScope st(*group, S_UNIQUE);
     launch_unique(s, tv, kl, sorted_keys, cur.view(), heads, !cur.tile_sorted, u_out ? u_out : &dst_->U);
-    // the run lists follow in the gather of the step, or before the batch's push if no gather came (lists_ready)
+    // the run lists follow in the gather of the step, or before the batch's push if that gather did not look at the
+    // index or never came (lists_ready)
   }
   if (part == 1) return;
   if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt, mirror->st.send_cnt, &mirror->st.U);
@@ -541,6 +550,9 @@ void Shard::finish_handle_query() {
   }
 }
 
+// whether this step's gather works from the keys in batch order (and the step does not wait for the index)
+bool Shard::direct_now(uint32_t bag) const { return cur.direct_gather && cur.comp_valid && bag == 1 && cur.n != 0; }
+
 // csrc/core/writeback.cu:43-56
 void Shard::write_back(float *dst, uint32_t bag) {
   hipStream_t s = group->stream;
@@ -571,7 +583,10 @@ void Shard::write_back(float *dst, uint32_t bag) {
     a.in_val = in_val.as<embed_t>();
     launch_refresh(s, tv, cur.view(), cur.n, prev.U ? prev.U : cur.n, a, sp.block_sums, stats.as<uint32_t>(), mirror->stats);
   }
-  if (dst != nullptr) {
+  if (dst != nullptr && direct_now(bag)) {
+    StageScope st(*group, S_GATHER);
+    launch_gather_direct(s, tv, kl, cur.comp.p, cur.n, dst, a.stream_stores);
+  } else if (dst != nullptr) {
     StageScope st(*group, S_GATHER);
     if (!cur.lists_ready && cur.n != 0) { // the first blocks of the gather build the batch's run lists on their way
       a.list_chunks = run_list_chunks(cur.n);
@@ -666,7 +681,7 @@ size_t Shard::fetch(int which, void *out, size_t cap) {
     case HCTR_F_STORE_IDS: return put64(download<index_t>(store_ids.p, tv.n_stored), tv.n_stored, out, cap);
     case HCTR_F_KEYS: { // the ids of the batch as its sort keys hold them (an id outside the table reads as 0)
       std::vector<uint64_t> k(cur.n);
-      if (!cur.keys_made) { // no copy in batch order was kept: position sorted_arg[j] holds the key of rank_sorted[j]
+      if (!cur.comp_valid) { // no copy in batch order was kept: position sorted_arg[j] holds the key of rank_sorted[j]
         const auto uk = ukeys(cur);
         const auto pos = download<uint32_t>(cur.sorted_arg.p, cur.n), rk = download<uint32_t>(cur.rank_sorted.p, cur.n);
         for (size_t j = 0; j < cur.n; j++) k[pos[j]] = uk[rk[j]] & id_mask;
@@ -1163,7 +1178,11 @@ void Group::push_pull_steps(const float *const *grads, float *const *dsts, uint3
   if (time_calls) HCTR_HIP(hipEventRecord(ev_push, stream));
   if (nrank > 1) HCTR_HIP(hipEventRecord(ev_pushed, stream));
   enqueue_index_rest(); // the pushes are in their queue, now the rest of the current batches' index
-  const bool join_index = index_pending;
+  // One shard and a small batch: the gather works from the batch's keys and needs nothing of its index, which is
+  // longer than the push of such a batch.  The step then leaves the index pending: whatever needs it next (the next
+  // preprocess, which makes this batch the previous one; a fetch) waits for it, by then long done.
+  const bool index_not_needed = nrank == 1 && (dsts[0] == nullptr || members[0]->direct_now(bag));
+  const bool join_index = index_pending && !index_not_needed;
   uint64_t queries_max = 0;
   if (nrank > 1) {
     if (!owner_host) {

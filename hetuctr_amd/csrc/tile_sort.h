@@ -86,10 +86,11 @@ struct TileSortBuffers {
 // batch's run counters (nlong, optional), writes the tiles sorted by the first digit into buffers 0.
 // made_keys (optional): the batch's sort keys in batch order, already made and checked by make_keys; the launch then
 // starts from them and looks at neither ids, err nor nlong.
-// ids32: `ids` points to 32-bit ids (see launch_make_keys).
+// ids32: `ids` points to 32-bit ids (see launch_make_keys).  keys_out (optional, with ids): receives the sort keys in
+// batch order as well.
 void launch_tile_sort_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *ids,
                            const void *made_keys, uint32_t n, const TileSortBuffers &b, uint32_t *err, uint32_t *nlong,
-                           bool ids32 = false);
+                           bool ids32 = false, void *keys_out = nullptr);
 // Launches [from, to) of the 1..P that follow (P = passes of kl.total_bits), for callers that enqueue them in pieces.
 // The last one writes the sorted positions to sorted_arg, the sorted keys to *sorted_keys (one of b.keys) and `heads`.
 // Returns P.

@@ -159,7 +159,8 @@ __global__ __launch_bounds__(kSortBlock) void keys_tile_sort(const void *__restr
                                                               const worker_t *__restrict__ root, uint32_t *__restrict__ err,
                                                               uint32_t *__restrict__ nlong, int dbits, uint32_t pitch,
                                                               K *__restrict__ out_keys, uint32_t *__restrict__ out_vals,
-                                                              uint16_t *__restrict__ table, bool ids32) {
+                                                              uint16_t *__restrict__ table, bool ids32,
+                                                              K *__restrict__ keys_out) {
   using S = TileShape<K, ITEMS>;
   __shared__ __align__(16) uint32_t area[S::kAreaWords];
   __shared__ uint32_t bin_start[kSortMaxBins];
@@ -205,6 +206,8 @@ __global__ __launch_bounds__(kSortBlock) void keys_tile_sort(const void *__restr
     for (int r = 0; r < ITEMS; r++) {
       key[r] = (K)((owner[r] << id_bits) | id[r]);
       val[r] = tile_lo + w * S::kSub + r * kWave + lane;
+      // the sort keys in batch order as well, for a caller that works on the batch before it is sorted (optional)
+      if (keys_out && w * S::kSub + r * kWave + lane < tile_n) keys_out[val[r]] = key[r];
     }
   }
   tile_sort_by_digit<K, ITEMS, DBITS>(key, val, tile_n, 0, dbits, area, bin_start, sm);
@@ -488,7 +491,7 @@ DigitPlan plan_digits(const KeyLayout &kl) {
 
 void launch_tile_sort_keys(hipStream_t s, const TableView &t, const KeyLayout &kl, const index_t *ids,
                            const void *made_keys, uint32_t n, const TileSortBuffers &b, uint32_t *err, uint32_t *nlong,
-                           bool ids32) {
+                           bool ids32, void *keys_out) {
   if (!n) return;
   HCTR_CHECK(!ids32 || t.id_max <= 0xffffffffull, "internal: narrowed ids and a table of 2^32 rows or more");
   HCTR_CHECK(tile_sort_possible(n), "internal: batch too large for the tile-sorted passes");
@@ -500,11 +503,11 @@ void launch_tile_sort_keys(hipStream_t s, const TableView &t, const KeyLayout &k
     if (made_keys)                                                                                                    \
       hipLaunchKernelGGL((keys_tile_sort<K, I, D, true>), dim3(tiles), dim3(kSortBlock), 0, s, made_keys, n, t.id_max, \
                          kl.id_bits, t.nrank, t.root, err, nlong, p.dbits[0], pitch, (K *)b.keys[0], b.vals[0], table0, \
-                         false);                                                                                      \
+                         false, (K *)nullptr);                                                                        \
     else                                                                                                              \
       hipLaunchKernelGGL((keys_tile_sort<K, I, D, false>), dim3(tiles), dim3(kSortBlock), 0, s, (const void *)ids, n, \
                          t.id_max, kl.id_bits, t.nrank, t.root, err, nlong, p.dbits[0], pitch, (K *)b.keys[0],        \
-                         b.vals[0], table0, ids32);                                                                   \
+                         b.vals[0], table0, ids32, (K *)keys_out);                                                    \
   } while (0)
   HCTR_TILE_SORT_DISPATCH(kl.wide, n, p.dbits[0], CALL);
 #undef CALL

@@ -53,9 +53,14 @@ def test_uniform_init_golden_vectors():
         p.close()
 
 
+@pytest.mark.parametrize("gather", ["from the keys", "sorted"])
 @pytest.mark.parametrize("width", [1, 3, 4, 16, 20, 64, 128, 200, 256, 300, 512])
-def test_single_shard_steps_all_widths(width):
-    say("single shard width", width)
+def test_single_shard_steps_all_widths(width, gather, monkeypatch):
+    # a small batch of one shard is gathered in batch order straight from its keys, a large one in sorted order behind
+    # the index: both at every width
+    if gather == "sorted":
+        monkeypatch.setenv("HETUCTR_DIRECT_GATHER_MAX", "0")
+    say("single shard width", width, gather)
     rng = np.random.default_rng(width)
     length, n = 5000, 3000
     p = single(length, width, lr=0.05)
@@ -70,6 +75,35 @@ def test_single_shard_steps_all_widths(width):
         p.compare_ints(INT_ITEMS_POST, "step %d" % step)
         p.compare_state(1e-5, "step %d" % step)
         prev_n = keys.shape[0]
+    p.close()
+
+
+@pytest.mark.parametrize("gather", ["from the keys", "sorted"])
+def test_one_shard_steps_without_a_look_at_the_index(gather, monkeypatch):
+    # nothing is fetched between preprocess and push_pull: with the gather from the keys push_pull returns while the
+    # index of its batch may still be running, and the next preprocess (or the fetch below) takes it over
+    if gather == "sorted":
+        monkeypatch.setenv("HETUCTR_DIRECT_GATHER_MAX", "0")
+    say("one shard, no look at the index", gather)
+    rng = np.random.default_rng(91)
+    length, width = 150_000, 20
+    draw = zipf_sampler(length, 1.1, rng)
+    p = single(length, width, lr=0.05)
+    prev_n = 0
+    for step, n in enumerate([5000, 180_000, 3, 70_000, 0, 1, 40_000, 40_000]):
+        keys = draw(n) if step % 2 else rng.integers(0, length, size=n).astype(np.int64)
+        p.preprocess([keys], device_keys=bool(step % 3))
+        g = rng.normal(0, 1e-3, size=(prev_n, width)).astype(np.float32)
+        out, ref = p.push_pull([g])
+        if step == 6:                                           # the same batches once more, no preprocess in between
+            out, ref = p.push_pull([g])
+        assert_close(out[0], ref[0], 1e-5, "dst step %d" % step)
+        if step % 2:
+            p.compare_ints(INT_ITEMS_PRE + INT_ITEMS_POST, "step %d" % step)
+            p.compare_state(1e-5, "step %d" % step)
+        prev_n = n
+    p.compare_ints(INT_ITEMS_PRE + INT_ITEMS_POST, "end")
+    p.compare_state(1e-5, "end")
     p.close()
 
 
