@@ -364,6 +364,7 @@ void Shard::index_batch(uint32_t *u_out, int part) {
     launch_unique(s, tv, kl, sorted_keys, cur.view(), heads, !cur.tile_sorted, u_out ? u_out : &dst_->U);
     // the run lists follow in the gather of the step, or before the batch's push if that gather did not look at the
     // index or never came (lists_ready)
+    // (built behind the index instead, they make the index the longer of a small step's two chains: 78 us against 64)
   }
   if (part == 1) return;
   if (cfg.nrank > 1) launch_bucket_sizes(s, cur.view(), cfg.nrank, dst_->send_cnt, mirror->st.send_cnt, &mirror->st.U);
