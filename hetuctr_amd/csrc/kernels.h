@@ -258,6 +258,9 @@ void launch_gather(hipStream_t s, const TableView &t, const BatchView &cur, cons
 // nothing of the batch's index
 void launch_gather_direct(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *keys, uint32_t n, embed_t *dst,
                           bool stream_stores);
+// the same for bags of `bag` consecutive positions, one summed output row per bag (n a multiple of bag)
+void launch_gather_pooled_direct(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *keys, uint32_t n,
+                                 embed_t *dst, uint32_t bag);
 // sum-pooled lookups: dst[b] = the rows of positions b * bag .. b * bag + bag - 1 added up in that order
 // (cur.idx_map must be filled: launch_idx_map)
 void launch_gather_pooled(hipStream_t s, const TableView &t, const BatchView &cur, const PullArgs &a, uint32_t bag);

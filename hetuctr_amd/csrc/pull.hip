@@ -600,6 +600,38 @@ __global__ __launch_bounds__(kBlock) void gather_pooled(TableView t, BatchView c
   }
 }
 
+// The same for one shard from the batch's keys in batch order (as gather_direct): a bag's positions are consecutive in
+// the batch, so this order costs no locality the other would have, and nothing of the batch's index is needed.
+template <int VEC, int LPR, typename K>
+__global__ __launch_bounds__(kBlock) void gather_pooled_direct(TableView t, const K *__restrict__ keys, int id_bits,
+                                                               embed_t *__restrict__ dst_rows, uint32_t bag, uint32_t n_bags) {
+  typedef typename RowVec<VEC>::T V;
+  constexpr int kGroups = kBlock / LPR;
+  const uint32_t b = blockIdx.x * kGroups + threadIdx.x / LPR;
+  if (b >= n_bags) return;
+  const uint32_t gl = threadIdx.x % LPR, W = t.width;
+  const uint32_t i0 = b * bag;
+  const K id_mask = (K)(((uint64_t)1 << id_bits) - 1);
+  for (uint32_t col = gl * VEC; col < W; col += LPR * VEC) {
+    V acc;
+    for (uint32_t h0 = 0; h0 < bag; h0 += kPoolAhead) {
+      const embed_t *src[kPoolAhead];
+#pragma unroll
+      for (int k = 0; k < kPoolAhead; k++)
+        src[k] = t.emb + (size_t)t.slot[(uint64_t)(keys[i0 + min(h0 + k, bag - 1)] & id_mask)] * W;
+      V v[kPoolAhead];
+#pragma unroll
+      for (int k = 0; k < kPoolAhead; k++) v[k] = *(const V *)(src[k] + col);
+#pragma unroll
+      for (int k = 0; k < kPoolAhead; k++) {
+        if (h0 + k == 0) acc = v[k];
+        else if (h0 + k < bag) acc = acc + v[k];
+      }
+    }
+    __builtin_nontemporal_store(acc, (V *)(dst_rows + (size_t)b * W + col));
+  }
+}
+
 // plain 16-byte-lane copy of known size: the yardstick the HBM byte counters are scaled with
 __global__ __launch_bounds__(kBlock) void plain_copy(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
   const size_t stride = (size_t)gridDim.x * kBlock;
@@ -742,6 +774,24 @@ void launch_gather_direct(hipStream_t s, const TableView &t, const KeyLayout &kl
     else if (kl.wide) hipLaunchKernelGGL((gather_direct<V, L, uint64_t, false>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint64_t *)keys, kl.id_bits, n, dst); \
     else if (stream_stores) hipLaunchKernelGGL((gather_direct<V, L, uint32_t, true>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint32_t *)keys, kl.id_bits, n, dst); \
     else hipLaunchKernelGGL((gather_direct<V, L, uint32_t, false>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint32_t *)keys, kl.id_bits, n, dst); \
+  } while (0)
+  HCTR_DISPATCH_ROW(vec4, lpr, CALL);
+#undef CALL
+  HCTR_HIP(hipGetLastError());
+}
+
+void launch_gather_pooled_direct(hipStream_t s, const TableView &t, const KeyLayout &kl, const void *keys, uint32_t n,
+                                 embed_t *dst, uint32_t bag) {
+  if (!n) return;
+  HCTR_CHECK(t.nrank == 1, "internal: the gather from the keys is for one shard");
+  const uint32_t n_bags = n / bag;
+  const bool vec4 = t.width % 4 == 0 && ((uintptr_t)dst % 16) == 0;
+  const int lpr = lanes_for(t.width, vec4 ? 4 : 1);
+#define CALL(V, L)                                                                                                    \
+  do {                                                                                                                \
+    const unsigned blocks = div_up(n_bags, kBlock / L);                                                               \
+    if (kl.wide) hipLaunchKernelGGL((gather_pooled_direct<V, L, uint64_t>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint64_t *)keys, kl.id_bits, dst, bag, n_bags); \
+    else hipLaunchKernelGGL((gather_pooled_direct<V, L, uint32_t>), dim3(blocks), dim3(kBlock), 0, s, t, (const uint32_t *)keys, kl.id_bits, dst, bag, n_bags); \
   } while (0)
   HCTR_DISPATCH_ROW(vec4, lpr, CALL);
 #undef CALL

@@ -151,6 +151,7 @@ class Shard {
   void index_batch(uint32_t *u_out = nullptr, int part = 0);
   TileSortBuffers tile_sort_buffers() const; // the index scratch as the tile-sorted passes take it
   HostStager stager;                         // ids that arrive in pageable host memory go through its pinned buffer
+  bool pooled_from_keys = true;   // HETUCTR_POOLED_FROM_KEYS=0: pooled gathers of one shard go through the inverse index
   uint32_t direct_gather_max = 0; // keys: HCTR_DIRECT_GATHER_BYTES / bytes of a row, or HETUCTR_DIRECT_GATHER_MAX
   int tile_sort_mode = 1;                    // HETUCTR_TILE_SORT: 0 no batch takes the tile-sorted passes, 1 those of up
                                              // to kTileSortMaxKeys keys, 2 every batch whose tiles they can hold

@@ -127,6 +127,7 @@ Shard::Shard(const hctr_config &c, const uint8_t *root_arr, const int64_t *stora
   // which sort indexes a batch: 0 the three-launch passes of radix_sort.h always, 2 the tile-sorted passes whenever
   // they can hold the batch (measurements of either sort at any size); default: tile_sort_fits()
   if (const char *f = getenv("HETUCTR_TILE_SORT")) tile_sort_mode = f[0] == '0' ? 0 : (f[0] == '2' ? 2 : 1);
+  if (const char *f = getenv("HETUCTR_POOLED_FROM_KEYS")) pooled_from_keys = f[0] != '0';
   direct_gather_max = (uint32_t)std::min<uint64_t>(HCTR_DIRECT_GATHER_BYTES / ((uint64_t)c.width * sizeof(embed_t)), 0xfffffff0u);
   if (const char *f = getenv("HETUCTR_DIRECT_GATHER_MAX")) direct_gather_max = (uint32_t)strtoul(f, nullptr, 10);
   if (const char *f = getenv("HETUCTR_TILE_DIGIT_BITS")) // many narrow passes exercise the hand-over between the launches
@@ -303,10 +304,10 @@ void Shard::ingest_keys(const int64_t *keys, size_t n, uint32_t *flag, void *scr
       // the step's critical path (write_back); the keys are then made by a kernel of their own here as well.
       cur.direct_gather = cfg.nrank == 1 && flag != nullptr && cur.n <= direct_gather_max;
       cur.keys_made = !cur.tile_sorted || (flag != nullptr && cur.n >= kKeysFirstFrom);
-      cur.comp_valid = cur.keys_made || cur.direct_gather;
+      cur.comp_valid = true; // either kernel leaves the sort keys in batch order (a gather from the keys reads them)
       if (!cur.keys_made)
         launch_tile_sort_keys(s, tv, kl, ids, nullptr, cur.n, tile_sort_buffers(), flag ? flag : err_ptr(),
-                              cur.dnlong.as<uint32_t>(), narrowed, cur.direct_gather ? cur.comp.p : nullptr);
+                              cur.dnlong.as<uint32_t>(), narrowed, cur.comp.p);
       else
         launch_make_keys(s, tv, kl, ids, cur.n, cur.comp.p, flag ? flag : err_ptr(), cur.dnlong.as<uint32_t>(),
                          cur.tile_sorted ? nullptr : sp.sortws, narrowed);
@@ -552,7 +553,11 @@ void Shard::finish_handle_query() {
 }
 
 // whether this step's gather works from the keys in batch order (and the step does not wait for the index)
-bool Shard::direct_now(uint32_t bag) const { return cur.direct_gather && cur.comp_valid && bag == 1 && cur.n != 0; }
+// (bags: a pooled gather walks the batch in its own order anyway, so it always works from the keys when they are there)
+bool Shard::direct_now(uint32_t bag) const {
+  if (cfg.nrank != 1 || !cur.comp_valid || cur.n == 0) return false;
+  return bag == 1 ? cur.direct_gather : pooled_from_keys;
+}
 
 // csrc/core/writeback.cu:43-56
 void Shard::write_back(float *dst, uint32_t bag) {
@@ -586,7 +591,9 @@ void Shard::write_back(float *dst, uint32_t bag) {
   }
   if (dst != nullptr && direct_now(bag)) {
     StageScope st(*group, S_GATHER);
-    launch_gather_direct(s, tv, kl, cur.comp.p, cur.n, dst, a.stream_stores);
+    HCTR_CHECK(cur.n % bag == 0, "pooled pull: the batch is not a whole number of bags");
+    if (bag > 1) launch_gather_pooled_direct(s, tv, kl, cur.comp.p, cur.n, dst, bag);
+    else launch_gather_direct(s, tv, kl, cur.comp.p, cur.n, dst, a.stream_stores);
   } else if (dst != nullptr) {
     StageScope st(*group, S_GATHER);
     if (!cur.lists_ready && cur.n != 0) { // the first blocks of the gather build the batch's run lists on their way

@@ -24,8 +24,12 @@ def pooled_step(p, keys, grads_pooled, bag):
     return out, p.oracle.push_pull_pooled(grads_pooled, bag)
 
 
+@pytest.mark.parametrize("gather", ["from the keys", "through the inverse index"])
 @pytest.mark.parametrize("bag,width", [(1, 32), (2, 128), (3, 20), (10, 64), (17, 8)])
-def test_single_shard_pooled(bag, width):
+def test_single_shard_pooled(bag, width, gather, monkeypatch):
+    if gather != "from the keys":          # one shard pools straight from the batch's keys unless told otherwise
+        monkeypatch.setenv("HETUCTR_POOLED_FROM_KEYS", "0")
+        monkeypatch.setenv("HETUCTR_DIRECT_GATHER_MAX", "0")
     print("pooled single shard, bag", bag, "width", width, flush=True)
     rng = np.random.default_rng(60 + bag)
     length, bags = 20_000, 3000
